@@ -1,0 +1,137 @@
+/*
+ * nmspmm.h — C-ABI of the MI355X (gfx950) N:M sparse x dense fp32 matrix-multiply library.
+ *
+ * Plain pointers and sizes only; every function returns an nmspmm_status and never prints.
+ * The C++ drop-in header NM-SpMM.h (same directory) is a thin layer over these entry points.
+ *
+ * Operands (the reference project's device layouts, src/kernel_64x128_8x8.cu:14-16):
+ *   A            fp32, column-major M x K: element (i,k) at A[i + k*M]
+ *   B            fp32, row-major   W x N: compressed values, W = K * kept / window
+ *   D            int32, preprocessed indices, blocked [N/Ns][W][Ns/vec_len]
+ *   column_info  int32, [N/Ns][W/kept][window], -1 padded (high-sparsity path only)
+ *   C            fp32, row-major M x N
+ * "window" is the number of dense K rows one index window spans (the M of N:M after any
+ * widening), "kept" the number of rows kept in it, "vec_len" the number of adjacent columns of
+ * B that share one index pattern, "Ns" the column-block width the indices were preprocessed for.
+ *
+ * Device pointers are HIP device pointers on the current device; `stream` is a hipStream_t
+ * passed as void* (NULL = the default stream).  Launches are asynchronous.
+ */
+#ifndef NMSPMM_C_API_H
+#define NMSPMM_C_API_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum nmspmm_status {
+    NMSPMM_OK = 0,
+    NMSPMM_ERR_NULL_POINTER = 1, /* a required pointer is NULL */
+    NMSPMM_ERR_BAD_SHAPE = 2,    /* sizes are non-positive or violate a divisibility rule */
+    NMSPMM_ERR_BAD_PATTERN = 3,  /* window / kept / vec_len / sparsity not representable */
+    NMSPMM_ERR_WRONG_PATH = 4,   /* sparsity belongs to the other (low/high) entry point */
+    NMSPMM_ERR_BAD_SPLIT = 5,    /* split_k < 1 or larger than the number of windows */
+    NMSPMM_ERR_WORKSPACE = 6,    /* split_k > 1 and the workspace is missing or too small */
+    NMSPMM_ERR_HIP = 7,          /* a HIP runtime call failed (no device, out of memory, ...) */
+    NMSPMM_ERR_ALIGNMENT = 8     /* a pointer is not aligned as the kernels require (16 bytes) */
+} nmspmm_status;
+
+/* Column-block widths of the four named entry points of the reference API
+ * (reference tests/test_nmspmm.cu:207-237: small 32, medium 64, large 64, huge 128). */
+typedef enum nmspmm_tile {
+    NMSPMM_TILE_SMALL = 32,
+    NMSPMM_TILE_MEDIUM = 64,
+    NMSPMM_TILE_LARGE = 64,
+    NMSPMM_TILE_HUGE = 128
+} nmspmm_tile;
+
+int nmspmm_version(void);
+const char* nmspmm_status_string(int status);
+
+/* Maps a sparsity in {0, 0.5, 0.625, 0.75, 0.875} (matched within 1e-6, as the reference
+ * launchers do, src/kernel_64x128_8x8.cu:264-289,584-602) to the window geometry the kernels
+ * use: 0 -> 32/32, 0.5 -> 32/16, 0.625 -> 32/12 (low path), 0.75 -> 64/16, 0.875 -> 64/8
+ * (high path).  *is_high is set to 1 for the high path.  Any other value:
+ * NMSPMM_ERR_BAD_PATTERN. */
+int nmspmm_pattern_from_sparsity(float sparsity, int* window, int* kept, int* is_high);
+
+/* ---- index preprocessing ------------------------------------------------------------------ */
+
+/* Replaces transIndex (reference include/NM-SpMM.h:12, src/preprocessing.cu:3-15): merges each
+ * pair of adjacent windows of the row-major int32 DT[W][Q] by adding *pruning_M to the indices
+ * of every odd window, then doubles *pruning_N and *pruning_M.  N is accepted for signature
+ * parity and only checked against Q * vec_len.  Host-pointer form: DT is host memory, updated
+ * in place (staged through the device, the work is done by the HIP kernel). */
+int nmspmm_trans_index_host(int32_t* DT, int W, int N, int Q, int* pruning_N, int* pruning_M);
+/* Device-pointer form of the same operation, in place on device memory, asynchronous. */
+int nmspmm_trans_index_device(int32_t* dDT, int W, int N, int Q, int* pruning_N, int* pruning_M,
+                              void* stream);
+
+/* Replaces PreProcessing_low_sparsity (reference include/NM-SpMM.h:10,
+ * src/preprocessing.cu:80-100): re-blocks DT[W][Q] to [Q/Qs][W][Qs], Qs = Ns / vec_len.
+ * Host form works in place on host memory. */
+int nmspmm_preprocess_low_host(int32_t* DT, int W, int Q, int Ns, int vec_len);
+/* Device form: reads dDT_in, writes dDT_out (distinct buffers of W*Q int32). */
+int nmspmm_preprocess_low_device(const int32_t* dDT_in, int32_t* dDT_out, int W, int Q, int Ns,
+                                 int vec_len, void* stream);
+
+/* Replaces PreProcessing_high_sparsity (reference include/NM-SpMM.h:11,
+ * src/preprocessing.cu:17-78): per (column block, window) writes the ascending list of used
+ * window-local rows to column_info (-1 padded to pruning_M), renumbers the indices to ranks in
+ * that list, then re-blocks like the low form.  column_info must hold at least
+ * nmspmm_column_info_ints() int32; only that many are written.  pruning_M <= 1024. */
+int nmspmm_preprocess_high_host(int32_t* column_info, int pruning_M, int pruning_N, int32_t* DT,
+                                int W, int Q, int N, int Ns, int vec_len);
+int nmspmm_preprocess_high_device(int32_t* d_column_info, int pruning_M, int pruning_N,
+                                  const int32_t* dDT_in, int32_t* dDT_out, int W, int Q, int N,
+                                  int Ns, int vec_len, void* stream);
+
+/* Number of int32 the high-sparsity preprocessing writes: (N/Ns) * (W/pruning_N) * pruning_M.
+ * (The reference driver allocates one extra window of slack, tests/test_nmspmm.cu:23; this
+ * library neither needs nor touches it.)  Returns 0 for invalid arguments. */
+size_t nmspmm_column_info_ints(int W, int pruning_N, int pruning_M, int N, int Ns);
+
+/* ---- multiplication ----------------------------------------------------------------------- */
+
+/* Bytes of device workspace nmspmm_spmm needs for a given split_k (0 when split_k <= 1):
+ * split_k partial M x N fp32 results that a second pass sums in a fixed order. */
+size_t nmspmm_workspace_bytes(int M, int N, int split_k);
+
+/* General entry point: C = A . B for one (window, kept, vec_len, Ns) geometry.
+ * column_info == NULL selects the low-sparsity layout (all window rows staged), non-NULL the
+ * high-sparsity layout (only the rows column_info lists are staged, D holds ranks).
+ * split_k > 1 requires `workspace` of at least nmspmm_workspace_bytes(); unlike the reference's
+ * atomicAdd reduction (include/ptx.h:34-40) C is overwritten, not accumulated into.
+ * Requirements: N % Ns == 0, Ns % vec_len == 0, W % kept == 0, 1 <= split_k <= W / kept,
+ * K * kept == W * window, 16-byte aligned A, B and C. */
+int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t* column_info,
+                float* C, int M, int N, int K, int W, int window, int kept, int vec_len, int Ns,
+                int split_k, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Replace the reference launchers nmGEMM_{small,medium,large,huge}_matrices_low_sparsity
+ * (reference include/NM-SpMM.h:14,17,20,23) and ..._high_sparsity (:15,18,21,24): `tile` is the
+ * nmspmm_tile of the named entry point, `sparsity` selects the geometry as
+ * nmspmm_pattern_from_sparsity does, vec_len is 32.  A sparsity that belongs to the other path
+ * returns NMSPMM_ERR_WRONG_PATH (the reference prints "Not support!" there).  When split_k > 1
+ * the library uses a per-device workspace that it grows on demand and keeps until
+ * nmspmm_release(); calls sharing a device must then be issued on one stream at a time. */
+int nmspmm_gemm_low_sparsity(int tile, const float* A, const float* B, const int32_t* D, float* C,
+                             int M, int N, int K, int W, float sparsity, int split_k, void* stream);
+int nmspmm_gemm_high_sparsity(int tile, const float* A, const float* B, const int32_t* D,
+                              const int32_t* column_info, float* C, int M, int N, int K, int W,
+                              float sparsity, int split_k, void* stream);
+
+/* Frees the cached split-K workspaces of every device. */
+int nmspmm_release(void);
+
+/* Name of the kernel family the last successful nmspmm_spmm call on this thread dispatched to
+ * ("mfma", "simt"), for tests and profiles.  Never NULL. */
+const char* nmspmm_last_kernel(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NMSPMM_C_API_H */

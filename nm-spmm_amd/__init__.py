@@ -1,0 +1,156 @@
+"""ctypes binding of libnmspmm.so, the MI355X N:M sparse x dense fp32 library.
+
+The product is the shared library (C-ABI in include/nmspmm.h, C++ drop-in in include/NM-SpMM.h);
+this module only loads it and forwards torch device pointers, for the Python tests and the
+benchmark.  There is no CPU fallback: if the library has not been built, importing works but
+every call raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libnmspmm.so")
+CSRC_DIR = os.path.join(_HERE, "csrc")
+
+OK = 0
+STATUS_NAMES = {
+    0: "NMSPMM_OK", 1: "NMSPMM_ERR_NULL_POINTER", 2: "NMSPMM_ERR_BAD_SHAPE", 3: "NMSPMM_ERR_BAD_PATTERN",
+    4: "NMSPMM_ERR_WRONG_PATH", 5: "NMSPMM_ERR_BAD_SPLIT", 6: "NMSPMM_ERR_WORKSPACE", 7: "NMSPMM_ERR_HIP",
+    8: "NMSPMM_ERR_ALIGNMENT",
+}
+TILE_SMALL, TILE_MEDIUM, TILE_LARGE, TILE_HUGE = 32, 64, 64, 128
+
+
+class NmSpmmError(RuntimeError):
+    def __init__(self, fn, status):
+        self.status = status
+        super().__init__("%s failed: %s" % (fn, STATUS_NAMES.get(status, status)))
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises if it has not been built (no silent fallback)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libnmspmm.so is not built: run `make -C %s` (or __graft_entry__.build())" % CSRC_DIR)
+        L = ctypes.CDLL(LIB_PATH)
+        c_int, c_void_p, c_float, c_size_t = ctypes.c_int, ctypes.c_void_p, ctypes.c_float, ctypes.c_size_t
+        ip = ctypes.POINTER(ctypes.c_int)
+        L.nmspmm_version.restype = c_int
+        L.nmspmm_status_string.restype = ctypes.c_char_p
+        L.nmspmm_status_string.argtypes = [c_int]
+        L.nmspmm_last_kernel.restype = ctypes.c_char_p
+        L.nmspmm_pattern_from_sparsity.argtypes = [c_float, ip, ip, ip]
+        L.nmspmm_trans_index_host.argtypes = [c_void_p, c_int, c_int, c_int, ip, ip]
+        L.nmspmm_trans_index_device.argtypes = [c_void_p, c_int, c_int, c_int, ip, ip, c_void_p]
+        L.nmspmm_preprocess_low_host.argtypes = [c_void_p] + [c_int] * 4
+        L.nmspmm_preprocess_low_device.argtypes = [c_void_p, c_void_p] + [c_int] * 4 + [c_void_p]
+        L.nmspmm_preprocess_high_host.argtypes = [c_void_p, c_int, c_int, c_void_p] + [c_int] * 5
+        L.nmspmm_preprocess_high_device.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p] + [c_int] * 5 + [c_void_p]
+        L.nmspmm_column_info_ints.restype = c_size_t
+        L.nmspmm_column_info_ints.argtypes = [c_int] * 5
+        L.nmspmm_workspace_bytes.restype = c_size_t
+        L.nmspmm_workspace_bytes.argtypes = [c_int] * 3
+        L.nmspmm_spmm.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, c_void_p]
+        L.nmspmm_gemm_low_sparsity.argtypes = [c_int] + [c_void_p] * 4 + [c_int] * 4 + [c_float, c_int, c_void_p]
+        L.nmspmm_gemm_high_sparsity.argtypes = [c_int] + [c_void_p] * 5 + [c_int] * 4 + [c_float, c_int, c_void_p]
+        L.nmspmm_release.restype = c_int
+        _lib = L
+    return _lib
+
+
+def _check(fn, status):
+    if status != OK:
+        raise NmSpmmError(fn, status)
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def pattern_from_sparsity(sparsity):
+    w, k, h = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    _check("nmspmm_pattern_from_sparsity",
+           lib().nmspmm_pattern_from_sparsity(sparsity, ctypes.byref(w), ctypes.byref(k), ctypes.byref(h)))
+    return w.value, k.value, bool(h.value)
+
+
+def last_kernel():
+    return lib().nmspmm_last_kernel().decode()
+
+
+# ---- device-pointer forms: arguments are torch tensors on the GPU -----------------------------------
+
+def trans_index_device(dDT, W, N, Q, pN, pM):
+    n, m = ctypes.c_int(pN), ctypes.c_int(pM)
+    _check("nmspmm_trans_index_device",
+           lib().nmspmm_trans_index_device(_ptr(dDT), W, N, Q, ctypes.byref(n), ctypes.byref(m), _stream()))
+    return n.value, m.value
+
+
+def preprocess_low_device(dDT_in, dDT_out, W, Q, Ns, vec_len=32):
+    _check("nmspmm_preprocess_low_device",
+           lib().nmspmm_preprocess_low_device(_ptr(dDT_in), _ptr(dDT_out), W, Q, Ns, vec_len, _stream()))
+
+
+def preprocess_high_device(d_cinfo, pM, pN, dDT_in, dDT_out, W, Q, N, Ns, vec_len=32):
+    _check("nmspmm_preprocess_high_device",
+           lib().nmspmm_preprocess_high_device(_ptr(d_cinfo), pM, pN, _ptr(dDT_in), _ptr(dDT_out), W, Q, N, Ns,
+                                               vec_len, _stream()))
+
+
+def column_info_ints(W, pN, pM, N, Ns):
+    return lib().nmspmm_column_info_ints(W, pN, pM, N, Ns)
+
+
+def workspace_bytes(M, N, split_k):
+    return lib().nmspmm_workspace_bytes(M, N, split_k)
+
+
+def spmm(A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len=32, Ns=128, split_k=1, workspace=None):
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _check("nmspmm_spmm",
+           lib().nmspmm_spmm(_ptr(A), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(C), M, N, K, W, window, kept, vec_len,
+                             Ns, split_k, _ptr(workspace), ws_bytes, _stream()))
+
+
+def gemm_low_sparsity(tile, A, B, D, C, M, N, K, W, sparsity, split_k=1):
+    _check("nmspmm_gemm_low_sparsity",
+           lib().nmspmm_gemm_low_sparsity(tile, _ptr(A), _ptr(B), _ptr(D), _ptr(C), M, N, K, W, sparsity, split_k,
+                                          _stream()))
+
+
+def gemm_high_sparsity(tile, A, B, D, cinfo, C, M, N, K, W, sparsity, split_k=1):
+    _check("nmspmm_gemm_high_sparsity",
+           lib().nmspmm_gemm_high_sparsity(tile, _ptr(A), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(C), M, N, K, W,
+                                           sparsity, split_k, _stream()))
+
+
+# ---- host-pointer forms: arguments are C-contiguous numpy int32 arrays, updated in place ----------
+
+def _np_ptr(a):
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+def trans_index_host(DT, W, N, Q, pN, pM):
+    n, m = ctypes.c_int(pN), ctypes.c_int(pM)
+    _check("nmspmm_trans_index_host",
+           lib().nmspmm_trans_index_host(_np_ptr(DT), W, N, Q, ctypes.byref(n), ctypes.byref(m)))
+    return n.value, m.value
+
+
+def preprocess_low_host(DT, W, Q, Ns, vec_len=32):
+    _check("nmspmm_preprocess_low_host", lib().nmspmm_preprocess_low_host(_np_ptr(DT), W, Q, Ns, vec_len))
+
+
+def preprocess_high_host(cinfo, pM, pN, DT, W, Q, N, Ns, vec_len=32):
+    _check("nmspmm_preprocess_high_host",
+           lib().nmspmm_preprocess_high_host(_np_ptr(cinfo), pM, pN, _np_ptr(DT), W, Q, N, Ns, vec_len))

@@ -1,0 +1,397 @@
+// C-ABI layer: argument validation, kernel-family dispatch and the per-device split-K workspace.
+// Validation happens before any HIP call, so the error paths can be exercised without a GPU.
+#include "../../include/nmspmm.h"
+#include "internal.h"
+
+#include <cmath>
+#include <mutex>
+
+using namespace nmspmm;
+
+namespace {
+
+thread_local const char* g_last_kernel = "none";
+
+struct Workspace {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
+constexpr int kMaxDevices = 64;
+Workspace g_workspace[kMaxDevices];
+std::mutex g_workspace_mutex;
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+size_t slice_stride(int M, int N) { return (((size_t)M * N + 3) / 4) * 4; }
+
+int valid_vec_len(int v) { return v == 4 || v == 8 || v == 16 || v == 32; }
+
+int check_index_shape(int W, int Q)
+{
+    return (W > 0 && Q > 0) ? NMSPMM_OK : NMSPMM_ERR_BAD_SHAPE;
+}
+
+// Grows (never shrinks) the calling device's cached workspace.
+int cached_workspace(size_t bytes, void** out)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return NMSPMM_ERR_HIP;
+    std::lock_guard<std::mutex> lock(g_workspace_mutex);
+    Workspace& ws = g_workspace[dev];
+    if (ws.bytes < bytes) {
+        if (ws.ptr) {
+            if (hipDeviceSynchronize() != hipSuccess)
+                return NMSPMM_ERR_HIP;
+            (void)hipFree(ws.ptr);
+            ws.ptr = nullptr;
+            ws.bytes = 0;
+        }
+        if (hipMalloc(&ws.ptr, bytes) != hipSuccess) {
+            ws.ptr = nullptr;
+            return NMSPMM_ERR_HIP;
+        }
+        ws.bytes = bytes;
+    }
+    *out = ws.ptr;
+    return NMSPMM_OK;
+}
+
+// RAII device buffer for the host-pointer preprocessing forms.
+struct DeviceBuf {
+    void* p = nullptr;
+    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes); }
+    ~DeviceBuf()
+    {
+        if (p)
+            (void)hipFree(p);
+    }
+};
+
+} // namespace
+
+extern "C" {
+
+int nmspmm_version(void) { return 100; }
+
+const char* nmspmm_status_string(int status)
+{
+    switch (status) {
+    case NMSPMM_OK: return "ok";
+    case NMSPMM_ERR_NULL_POINTER: return "null pointer";
+    case NMSPMM_ERR_BAD_SHAPE: return "bad shape";
+    case NMSPMM_ERR_BAD_PATTERN: return "unsupported sparsity pattern";
+    case NMSPMM_ERR_WRONG_PATH: return "sparsity belongs to the other (low/high) entry point";
+    case NMSPMM_ERR_BAD_SPLIT: return "bad split_k";
+    case NMSPMM_ERR_WORKSPACE: return "workspace missing or too small";
+    case NMSPMM_ERR_HIP: return "HIP runtime error";
+    case NMSPMM_ERR_ALIGNMENT: return "pointer not 16-byte aligned";
+    }
+    return "unknown status";
+}
+
+const char* nmspmm_last_kernel(void) { return g_last_kernel; }
+
+int nmspmm_pattern_from_sparsity(float sparsity, int* window, int* kept, int* is_high)
+{
+    if (!window || !kept || !is_high)
+        return NMSPMM_ERR_NULL_POINTER;
+    struct Row { float s; int window, kept, high; };
+    static const Row table[] = {
+        {0.0f, 32, 32, 0}, {0.5f, 32, 16, 0}, {0.625f, 32, 12, 0}, {0.75f, 64, 16, 1}, {0.875f, 64, 8, 1},
+    };
+    for (const Row& r : table) {
+        if (std::fabs(sparsity - r.s) < 1e-6f) {
+            *window = r.window;
+            *kept = r.kept;
+            *is_high = r.high;
+            return NMSPMM_OK;
+        }
+    }
+    return NMSPMM_ERR_BAD_PATTERN;
+}
+
+/* ---- preprocessing ------------------------------------------------------------------------- */
+
+static int check_trans(const void* DT, int W, int N, int Q, const int* pN, const int* pM)
+{
+    if (!DT || !pN || !pM)
+        return NMSPMM_ERR_NULL_POINTER;
+    if (check_index_shape(W, Q) != NMSPMM_OK || N <= 0 || N % Q != 0)
+        return NMSPMM_ERR_BAD_SHAPE;
+    if (*pN <= 0 || *pM <= 0 || *pN > *pM)
+        return NMSPMM_ERR_BAD_PATTERN;
+    if (W % (2 * *pN) != 0) /* an odd number of windows has no partner for the last one */
+        return NMSPMM_ERR_BAD_SHAPE;
+    return NMSPMM_OK;
+}
+
+int nmspmm_trans_index_device(int32_t* dDT, int W, int N, int Q, int* pruning_N, int* pruning_M, void* stream)
+{
+    const int st = check_trans(dDT, W, N, Q, pruning_N, pruning_M);
+    if (st != NMSPMM_OK)
+        return st;
+    if (launch_trans_index(dDT, W, Q, *pruning_N, *pruning_M, (hipStream_t)stream) != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    *pruning_N *= 2;
+    *pruning_M *= 2;
+    return NMSPMM_OK;
+}
+
+int nmspmm_trans_index_host(int32_t* DT, int W, int N, int Q, int* pruning_N, int* pruning_M)
+{
+    const int st = check_trans(DT, W, N, Q, pruning_N, pruning_M);
+    if (st != NMSPMM_OK)
+        return st;
+    const size_t bytes = sizeof(int32_t) * (size_t)W * Q;
+    DeviceBuf d;
+    if (d.alloc(bytes) != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    if (hipMemcpy(d.p, DT, bytes, hipMemcpyHostToDevice) != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    const int rc = nmspmm_trans_index_device((int32_t*)d.p, W, N, Q, pruning_N, pruning_M, nullptr);
+    if (rc != NMSPMM_OK)
+        return rc;
+    if (hipMemcpy(DT, d.p, bytes, hipMemcpyDeviceToHost) != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    return NMSPMM_OK;
+}
+
+static int check_reblock(const void* in, const void* out, int W, int Q, int Ns, int vec_len)
+{
+    if (!in || !out)
+        return NMSPMM_ERR_NULL_POINTER;
+    if (!valid_vec_len(vec_len))
+        return NMSPMM_ERR_BAD_PATTERN;
+    if (check_index_shape(W, Q) != NMSPMM_OK || Ns <= 0 || Ns % vec_len != 0 || Q % (Ns / vec_len) != 0)
+        return NMSPMM_ERR_BAD_SHAPE;
+    return NMSPMM_OK;
+}
+
+int nmspmm_preprocess_low_device(const int32_t* dDT_in, int32_t* dDT_out, int W, int Q, int Ns, int vec_len,
+                                 void* stream)
+{
+    const int st = check_reblock(dDT_in, dDT_out, W, Q, Ns, vec_len);
+    if (st != NMSPMM_OK)
+        return st;
+    if (dDT_in == dDT_out)
+        return NMSPMM_ERR_BAD_SHAPE;
+    if (launch_reblock(dDT_in, dDT_out, W, Q, Ns / vec_len, (hipStream_t)stream) != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    return NMSPMM_OK;
+}
+
+int nmspmm_preprocess_low_host(int32_t* DT, int W, int Q, int Ns, int vec_len)
+{
+    const int st = check_reblock(DT, DT, W, Q, Ns, vec_len);
+    if (st != NMSPMM_OK)
+        return st;
+    const size_t bytes = sizeof(int32_t) * (size_t)W * Q;
+    DeviceBuf in, out;
+    if (in.alloc(bytes) != hipSuccess || out.alloc(bytes) != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    if (hipMemcpy(in.p, DT, bytes, hipMemcpyHostToDevice) != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    const int rc = nmspmm_preprocess_low_device((const int32_t*)in.p, (int32_t*)out.p, W, Q, Ns, vec_len, nullptr);
+    if (rc != NMSPMM_OK)
+        return rc;
+    if (hipMemcpy(DT, out.p, bytes, hipMemcpyDeviceToHost) != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    return NMSPMM_OK;
+}
+
+size_t nmspmm_column_info_ints(int W, int pruning_N, int pruning_M, int N, int Ns)
+{
+    if (W <= 0 || pruning_N <= 0 || pruning_M <= 0 || N <= 0 || Ns <= 0 || W % pruning_N != 0 || N % Ns != 0)
+        return 0;
+    return (size_t)(N / Ns) * (size_t)(W / pruning_N) * (size_t)pruning_M;
+}
+
+static int check_high(const void* ci, const void* in, const void* out, int pM, int pN, int W, int Q, int N,
+                      int Ns, int vec_len)
+{
+    if (!ci)
+        return NMSPMM_ERR_NULL_POINTER;
+    const int st = check_reblock(in, out, W, Q, Ns, vec_len);
+    if (st != NMSPMM_OK)
+        return st;
+    if (pN <= 0 || pM <= 0 || pN > pM || pM > 1024)
+        return NMSPMM_ERR_BAD_PATTERN;
+    if (W % pN != 0 || N != Q * vec_len)
+        return NMSPMM_ERR_BAD_SHAPE;
+    return NMSPMM_OK;
+}
+
+int nmspmm_preprocess_high_device(int32_t* d_column_info, int pruning_M, int pruning_N, const int32_t* dDT_in,
+                                  int32_t* dDT_out, int W, int Q, int N, int Ns, int vec_len, void* stream)
+{
+    const int st = check_high(d_column_info, dDT_in, dDT_out, pruning_M, pruning_N, W, Q, N, Ns, vec_len);
+    if (st != NMSPMM_OK)
+        return st;
+    if (dDT_in == dDT_out)
+        return NMSPMM_ERR_BAD_SHAPE;
+    if (launch_preprocess_high(d_column_info, pruning_M, pruning_N, dDT_in, dDT_out, W, Q, Ns / vec_len,
+                               (hipStream_t)stream) != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    return NMSPMM_OK;
+}
+
+int nmspmm_preprocess_high_host(int32_t* column_info, int pruning_M, int pruning_N, int32_t* DT, int W, int Q,
+                                int N, int Ns, int vec_len)
+{
+    const int st = check_high(column_info, DT, DT, pruning_M, pruning_N, W, Q, N, Ns, vec_len);
+    if (st != NMSPMM_OK)
+        return st;
+    const size_t bytes = sizeof(int32_t) * (size_t)W * Q;
+    const size_t ci_bytes = sizeof(int32_t) * nmspmm_column_info_ints(W, pruning_N, pruning_M, N, Ns);
+    DeviceBuf in, out, ci;
+    if (in.alloc(bytes) != hipSuccess || out.alloc(bytes) != hipSuccess || ci.alloc(ci_bytes) != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    if (hipMemcpy(in.p, DT, bytes, hipMemcpyHostToDevice) != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    const int rc = nmspmm_preprocess_high_device((int32_t*)ci.p, pruning_M, pruning_N, (const int32_t*)in.p,
+                                                 (int32_t*)out.p, W, Q, N, Ns, vec_len, nullptr);
+    if (rc != NMSPMM_OK)
+        return rc;
+    if (hipMemcpy(DT, out.p, bytes, hipMemcpyDeviceToHost) != hipSuccess ||
+        hipMemcpy(column_info, ci.p, ci_bytes, hipMemcpyDeviceToHost) != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    return NMSPMM_OK;
+}
+
+/* ---- multiplication ------------------------------------------------------------------------ */
+
+size_t nmspmm_workspace_bytes(int M, int N, int split_k)
+{
+    if (M <= 0 || N <= 0 || split_k <= 1)
+        return 0;
+    return sizeof(float) * slice_stride(M, N) * (size_t)split_k;
+}
+
+int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C, int M,
+                int N, int K, int W, int window, int kept, int vec_len, int Ns, int split_k, void* workspace,
+                size_t workspace_bytes, void* stream)
+{
+    if (!A || !B || !D || !C)
+        return NMSPMM_ERR_NULL_POINTER;
+    if (M <= 0 || N <= 0 || K <= 0 || W <= 0)
+        return NMSPMM_ERR_BAD_SHAPE;
+    if (window <= 0 || kept <= 0 || kept > window || !valid_vec_len(vec_len))
+        return NMSPMM_ERR_BAD_PATTERN;
+    if (Ns <= 0 || Ns % vec_len != 0 || N % Ns != 0 || W % kept != 0)
+        return NMSPMM_ERR_BAD_SHAPE;
+    if ((long long)K * kept != (long long)W * window)
+        return NMSPMM_ERR_BAD_SHAPE;
+    if (split_k < 1 || split_k > W / kept)
+        return NMSPMM_ERR_BAD_SPLIT;
+    if (!aligned16(A) || !aligned16(B) || !aligned16(C))
+        return NMSPMM_ERR_ALIGNMENT;
+    if (split_k > 1) {
+        if (!workspace || workspace_bytes < nmspmm_workspace_bytes(M, N, split_k) || !aligned16(workspace))
+            return NMSPMM_ERR_WORKSPACE;
+    }
+
+    SpmmArgs a;
+    a.A = A;
+    a.B = B;
+    a.D = D;
+    a.cinfo = column_info;
+    a.C = C;
+    a.partial = split_k > 1 ? (float*)workspace : nullptr;
+    a.slice_stride = slice_stride(M, N);
+    a.M = M;
+    a.N = N;
+    a.K = K;
+    a.W = W;
+    a.window = window;
+    a.kept = kept;
+    a.vec_len = vec_len;
+    a.Ns = Ns;
+    a.split_k = split_k;
+    a.stream = (hipStream_t)stream;
+
+    hipError_t e;
+    if (mfma_supported(a)) {
+        e = launch_mfma(a);
+        g_last_kernel = "mfma";
+    } else if (simt_supported(a)) {
+        e = launch_simt(a);
+        g_last_kernel = "simt";
+    } else {
+        return NMSPMM_ERR_BAD_PATTERN;
+    }
+    if (e != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    if (split_k > 1) {
+        e = launch_splitk_reduce(a.partial, C, (size_t)M * N, a.slice_stride, split_k, a.stream);
+        if (e != hipSuccess)
+            return NMSPMM_ERR_HIP;
+    }
+    return NMSPMM_OK;
+}
+
+static int named_gemm(int want_high, int tile, const float* A, const float* B, const int32_t* D,
+                      const int32_t* column_info, float* C, int M, int N, int K, int W, float sparsity,
+                      int split_k, void* stream)
+{
+    int window, kept, is_high;
+    const int st = nmspmm_pattern_from_sparsity(sparsity, &window, &kept, &is_high);
+    if (st != NMSPMM_OK)
+        return st;
+    if (is_high != want_high)
+        return NMSPMM_ERR_WRONG_PATH;
+    if (tile != 32 && tile != 64 && tile != 128)
+        return NMSPMM_ERR_BAD_SHAPE;
+    if (want_high && !column_info)
+        return NMSPMM_ERR_NULL_POINTER;
+    if (!A || !B || !D || !C)
+        return NMSPMM_ERR_NULL_POINTER;
+    if (M <= 0 || N <= 0 || W <= 0 || W % kept != 0)
+        return NMSPMM_ERR_BAD_SHAPE;
+    if (split_k < 1 || split_k > W / kept)
+        return NMSPMM_ERR_BAD_SPLIT;
+    void* ws = nullptr;
+    size_t ws_bytes = 0;
+    if (split_k > 1) {
+        ws_bytes = nmspmm_workspace_bytes(M, N, split_k);
+        const int rc = cached_workspace(ws_bytes, &ws);
+        if (rc != NMSPMM_OK)
+            return rc;
+    }
+    return nmspmm_spmm(A, B, D, want_high ? column_info : nullptr, C, M, N, K, W, window, kept, 32, tile, split_k,
+                       ws, ws_bytes, stream);
+}
+
+int nmspmm_gemm_low_sparsity(int tile, const float* A, const float* B, const int32_t* D, float* C, int M, int N,
+                             int K, int W, float sparsity, int split_k, void* stream)
+{
+    return named_gemm(0, tile, A, B, D, nullptr, C, M, N, K, W, sparsity, split_k, stream);
+}
+
+int nmspmm_gemm_high_sparsity(int tile, const float* A, const float* B, const int32_t* D,
+                              const int32_t* column_info, float* C, int M, int N, int K, int W, float sparsity,
+                              int split_k, void* stream)
+{
+    return named_gemm(1, tile, A, B, D, column_info, C, M, N, K, W, sparsity, split_k, stream);
+}
+
+int nmspmm_release(void)
+{
+    std::lock_guard<std::mutex> lock(g_workspace_mutex);
+    int rc = NMSPMM_OK;
+    int prev = 0;
+    const bool have_dev = hipGetDevice(&prev) == hipSuccess;
+    for (int d = 0; d < kMaxDevices; ++d) {
+        if (!g_workspace[d].ptr)
+            continue;
+        if (hipSetDevice(d) != hipSuccess || hipFree(g_workspace[d].ptr) != hipSuccess)
+            rc = NMSPMM_ERR_HIP;
+        g_workspace[d].ptr = nullptr;
+        g_workspace[d].bytes = 0;
+    }
+    if (have_dev)
+        (void)hipSetDevice(prev);
+    return rc;
+}
+
+} // extern "C"

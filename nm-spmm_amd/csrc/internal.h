@@ -1,0 +1,55 @@
+// Shared declarations between the C-ABI layer and the kernel translation units.
+#ifndef NMSPMM_INTERNAL_H
+#define NMSPMM_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace nmspmm {
+
+// One multiplication, already validated by the C-ABI layer.
+struct SpmmArgs {
+    const float* A;        // column-major M x K
+    const float* B;        // row-major W x N
+    const int32_t* D;      // [N/Ns][W][Ns/vec_len]
+    const int32_t* cinfo;  // [N/Ns][W/kept][window] or nullptr (low-sparsity layout)
+    float* C;              // row-major M x N
+    float* partial;        // split_k slices of slice_stride floats when split_k > 1, else nullptr
+    size_t slice_stride;   // M * N rounded up to a multiple of 4
+    int M, N, K, W;
+    int window, kept, vec_len, Ns;
+    int split_k;
+    hipStream_t stream;
+};
+
+// Windows [begin, begin + count) of reduction slice `z` out of `split_k`: an even split when it
+// divides, otherwise the first (nwin % split_k) slices take one extra window — the partition
+// rule of the reference kernels (src/kernel_64x128_8x8.cu:20-37).
+__host__ __device__ inline void split_windows(int nwin, int split_k, int z, int* begin, int* count)
+{
+    const int p = nwin / split_k, q = nwin % split_k;
+    *begin = z < q ? z * (p + 1) : z * p + q;
+    *count = z < q ? p + 1 : p;
+}
+
+// Matrix-core path (spmm_mfma.hip).  Returns false when the geometry has no instantiation.
+bool mfma_supported(const SpmmArgs& a);
+hipError_t launch_mfma(const SpmmArgs& a);
+
+// Generic SIMT path (spmm_simt.hip): any window/kept, vec_len in {4, 8, 16, 32}, any M.
+bool simt_supported(const SpmmArgs& a);
+hipError_t launch_simt(const SpmmArgs& a);
+
+// Sums split_k slices of `partial` into C in slice order (spmm_simt.hip).
+hipError_t launch_splitk_reduce(const float* partial, float* C, size_t elems, size_t slice_stride,
+                                int split_k, hipStream_t stream);
+
+// Index preprocessing kernels (preprocess.hip).
+hipError_t launch_trans_index(int32_t* dDT, int W, int Q, int pN, int pM, hipStream_t stream);
+hipError_t launch_reblock(const int32_t* in, int32_t* out, int W, int Q, int Qs, hipStream_t stream);
+hipError_t launch_preprocess_high(int32_t* cinfo, int pM, int pN, const int32_t* in, int32_t* out,
+                                  int W, int Q, int Qs, hipStream_t stream);
+
+} // namespace nmspmm
+#endif

@@ -1,0 +1,334 @@
+// Matrix-core kernels for C = A . B with an N:M-sparse B whose index pattern is shared by 32
+// adjacent columns (reference kernels: src/kernel_{64x128_8x8,64x64_8x8,32x64_8x4,32x32_4x4}.cu;
+// this file replaces their role, not their design).
+//
+// Design for gfx950 (64-lane waves, v_mfma_f32_32x32x2_f32):
+//  * A 32-column index vector is exactly the N extent of one 32x32x2 MFMA, so one wave owns one
+//    column vector and RM row blocks of 32 rows.  Its A operand for one MFMA is A[row][k] with
+//    lane = (row % 32, k half): lanes 0-31 take compressed row 2s, lanes 32-63 row 2s+1, and each
+//    half reads the LDS row of A that *its* index selects.  The gather is therefore just a
+//    per-lane LDS row offset; no data is moved to perform it.
+//  * The wave's RM row blocks interleave rows (block b holds rows 4*r + b), so one 128-bit LDS
+//    read yields the A operands of all RM blocks and the B operand is reused RM times.
+//  * A (window rows x Ms, k-major as in global memory) and B (kept rows x Ns) tiles are staged
+//    global -> registers -> LDS with 128-bit accesses, double buffered: the loads of window t+1
+//    are in flight while window t is multiplied, one barrier per window.
+//  * High-sparsity layout: only the rows listed in column_info are staged (the indices are
+//    already ranks into that list); column_info is fetched two windows ahead.
+//  * Workgroup ids are remapped so that the tiles resident on one XCD form a compact patch of
+//    C and share A / B panels in that XCD's L2.
+#include "internal.h"
+
+namespace nmspmm {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kXcds = 8;
+
+struct MfmaParams {
+    const float* A;
+    const float* B;
+    const int32_t* D;
+    const int32_t* cinfo;
+    float* out;          // C, or the first partial slice when split_k > 1
+    size_t slice_elems;  // M * N
+    int M, N, W;
+    int nwin;            // windows in the whole reduction
+    int split_k;
+    int tiles_m, tiles_n;
+};
+
+template <int RM> struct AFrag;
+template <> struct AFrag<4> { typedef float4 type; };
+template <> struct AFrag<2> { typedef float2 type; };
+template <> struct AFrag<1> { typedef float type; };
+
+__device__ inline float frag_get(const float4& v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+__device__ inline float frag_get(const float2& v, int i) { return i == 0 ? v.x : v.y; }
+__device__ inline float frag_get(const float& v, int) { return v; }
+
+// KS: dense rows per window, WS: kept rows per window, QS: column vectors per workgroup tile
+// (Ns = 32*QS, the width the indices were preprocessed for), WR: waves along M, RM: 32-row
+// blocks per wave, HIGH: high-sparsity layout.
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+struct TileCfg {
+    static constexpr int MS = WR * RM * 32;
+    static constexpr int NS = QS * 32;
+    static constexpr int NT = 64 * QS * WR;
+    static constexpr int AROWS = HIGH ? (KS < WS * QS ? KS : WS * QS) : KS;
+    static constexpr int ASTR = MS;       // floats per staged A row
+    static constexpr int BSTR = NS + 32;  // odd rows land in the other half of the banks
+    static constexpr int A_F4_ROW = MS / 4;
+    static constexpr int B_F4_ROW = NS / 4;
+    static constexpr int A_F4 = AROWS * A_F4_ROW;
+    static constexpr int B_F4 = WS * B_F4_ROW;
+    static constexpr int A_SLOTS = (A_F4 + NT - 1) / NT;
+    static constexpr int B_SLOTS = (B_F4 + NT - 1) / NT;
+    static constexpr int KSTEPS = WS / 2;
+    static constexpr size_t LDS_BYTES = sizeof(float) * 2 * (size_t)(AROWS * ASTR + WS * BSTR);
+    static_assert(WS % 2 == 0, "two compressed rows per MFMA");
+};
+
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+__global__ void __launch_bounds__(64 * QS * WR)
+spmm_mfma_kernel(const MfmaParams p)
+{
+    typedef TileCfg<KS, WS, QS, WR, RM, HIGH> T;
+    typedef typename AFrag<RM>::type afrag_t;
+    extern __shared__ __align__(16) float lds[];
+    float* const As = lds;                          // [2][AROWS][ASTR]
+    float* const Bs = lds + 2 * T::AROWS * T::ASTR;  // [2][WS][BSTR]
+
+    // ---- which tile -------------------------------------------------------------------------
+    // Consecutive workgroup ids go to consecutive XCDs; give every XCD a contiguous run of
+    // logical tile ids, then walk the tiles in bands of GROUP tile-rows.
+    const int total = p.tiles_m * p.tiles_n;
+    int logical;
+    {
+        const int id = blockIdx.x;
+        const int q = total / kXcds, r = total % kXcds;
+        const int xcd = id % kXcds, loc = id / kXcds;
+        logical = xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc;
+    }
+    constexpr int GROUP = 8;
+    int tile_m, tile_n;
+    {
+        const int band = logical / (GROUP * p.tiles_n);
+        const int first_m = band * GROUP;
+        const int rows = min(GROUP, p.tiles_m - first_m);
+        const int in_band = logical - band * GROUP * p.tiles_n;
+        tile_m = first_m + in_band % rows;
+        tile_n = in_band / rows;
+    }
+    const int bi = tile_m * T::MS;
+    const int bj = tile_n * T::NS;
+
+    int w_begin, w_count;
+    split_windows(p.nwin, p.split_k, blockIdx.y, &w_begin, &w_count);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int vec = wave % QS;   // column vector inside the tile
+    const int grp = wave / QS;   // row group inside the tile
+    const int h = lane >> 5;     // which of the two compressed rows of a k-step
+    const int j = lane & 31;
+
+    const int M = p.M, N = p.N;
+    const float* const Ablk = p.A + bi;
+    const float* const Bblk = p.B + bj;
+    const int32_t* const Dvec = p.D + (size_t)tile_n * p.W * QS + vec;
+    const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)tile_n * p.nwin * KS : nullptr;
+
+    // ---- per-thread staging slots -----------------------------------------------------------
+    float4 areg[T::A_SLOTS];
+    float4 breg[T::B_SLOTS];
+    int acol[T::A_SLOTS];  // HIGH: source row of each A slot for the window to be loaded next
+
+    auto load_cinfo = [&](int w) {
+#pragma unroll
+        for (int s = 0; s < T::A_SLOTS; ++s) {
+            const int lin = tid + s * T::NT;
+            const int row = lin / T::A_F4_ROW;
+            acol[s] = (lin < T::A_F4) ? Cinfo[(size_t)w * KS + row] : -1;
+        }
+    };
+    auto load_tiles = [&](int w) {
+        const float* Aw = Ablk + (size_t)w * KS * M;
+#pragma unroll
+        for (int s = 0; s < T::A_SLOTS; ++s) {
+            const int lin = tid + s * T::NT;
+            const int row = lin / T::A_F4_ROW;
+            const int c4 = (lin % T::A_F4_ROW) * 4;
+            const int src = HIGH ? acol[s] : row;
+            if (lin < T::A_F4 && src >= 0 && bi + c4 < M)
+                areg[s] = *reinterpret_cast<const float4*>(Aw + (size_t)src * M + c4);
+        }
+        const float* Bw = Bblk + (size_t)w * WS * N;
+#pragma unroll
+        for (int s = 0; s < T::B_SLOTS; ++s) {
+            const int lin = tid + s * T::NT;
+            const int row = lin / T::B_F4_ROW;
+            const int c4 = (lin % T::B_F4_ROW) * 4;
+            if (lin < T::B_F4)
+                breg[s] = *reinterpret_cast<const float4*>(Bw + (size_t)row * N + c4);
+        }
+    };
+    auto store_tiles = [&](int buf) {
+        float* Ab = As + buf * T::AROWS * T::ASTR;
+#pragma unroll
+        for (int s = 0; s < T::A_SLOTS; ++s) {
+            const int lin = tid + s * T::NT;
+            const int row = lin / T::A_F4_ROW;
+            const int c4 = (lin % T::A_F4_ROW) * 4;
+            if (lin < T::A_F4)
+                *reinterpret_cast<float4*>(Ab + row * T::ASTR + c4) = areg[s];
+        }
+        float* Bb = Bs + buf * WS * T::BSTR;
+#pragma unroll
+        for (int s = 0; s < T::B_SLOTS; ++s) {
+            const int lin = tid + s * T::NT;
+            const int row = lin / T::B_F4_ROW;
+            const int c4 = (lin % T::B_F4_ROW) * 4;
+            if (lin < T::B_F4)
+                *reinterpret_cast<float4*>(Bb + row * T::BSTR + c4) = breg[s];
+        }
+    };
+
+    // Index of compressed row (2s + h) of window w for this wave's column vector.
+    int idx_next[T::KSTEPS];
+    auto load_idx = [&](int w) {
+        const int32_t* Dw = Dvec + ((size_t)w * WS + h) * QS;
+#pragma unroll
+        for (int s = 0; s < T::KSTEPS; ++s)
+            idx_next[s] = Dw[(size_t)(2 * s) * QS];
+    };
+
+    const int a_lane = grp * (RM * 32) + j * RM;  // first of this lane's RM adjacent rows
+    const int b_lane = h * T::BSTR + vec * 32 + j;
+    int aoff[T::KSTEPS];
+
+    floatx16 acc[RM];
+#pragma unroll
+    for (int b = 0; b < RM; ++b)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            acc[b][v] = 0.0f;
+
+#pragma unroll
+    for (int s = 0; s < T::A_SLOTS; ++s) {
+        areg[s] = make_float4(0.f, 0.f, 0.f, 0.f);
+        acol[s] = -1;
+    }
+
+    // ---- prologue ---------------------------------------------------------------------------
+    if (w_count > 0) {
+        if (HIGH)
+            load_cinfo(w_begin);
+        load_tiles(w_begin);
+        load_idx(w_begin);
+        if (HIGH && w_count > 1)
+            load_cinfo(w_begin + 1);
+        store_tiles(0);
+#pragma unroll
+        for (int s = 0; s < T::KSTEPS; ++s)
+            aoff[s] = idx_next[s] * T::ASTR + a_lane;
+    }
+    __syncthreads();
+
+    // ---- main loop: one window per iteration --------------------------------------------------
+    for (int t = 0; t < w_count; ++t) {
+        const int w = w_begin + t;
+        const bool more = t + 1 < w_count;
+        if (more) {
+            load_tiles(w + 1);
+            load_idx(w + 1);
+            if (HIGH && t + 2 < w_count)
+                load_cinfo(w + 2);
+        }
+
+        const float* Ab = As + (t & 1) * T::AROWS * T::ASTR;
+        const float* Bb = Bs + (t & 1) * WS * T::BSTR + b_lane;
+#pragma unroll
+        for (int s = 0; s < T::KSTEPS; ++s) {
+            const afrag_t av = *reinterpret_cast<const afrag_t*>(Ab + aoff[s]);
+            const float bv = Bb[2 * s * T::BSTR];
+#pragma unroll
+            for (int b = 0; b < RM; ++b)
+                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_get(av, b), bv, acc[b], 0, 0, 0);
+        }
+
+        if (more) {
+            store_tiles((t + 1) & 1);
+#pragma unroll
+            for (int s = 0; s < T::KSTEPS; ++s)
+                aoff[s] = idx_next[s] * T::ASTR + a_lane;
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue -----------------------------------------------------------------------------
+    // MFMA result register v of lane (h, j) is row 8*(v/4) + 4*h + v%4, column j of the 32x32
+    // block; block b holds tile rows RM*row + b of this wave's row group.
+    float* out = p.out + (size_t)blockIdx.y * p.slice_elems;
+    const int col = bj + vec * 32 + j;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int r32 = 8 * (v / 4) + 4 * h + (v % 4);
+#pragma unroll
+        for (int b = 0; b < RM; ++b) {
+            const int row = bi + grp * (RM * 32) + r32 * RM + b;
+            if (row < M)
+                out[(size_t)row * N + col] = acc[b][v];
+        }
+    }
+}
+
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+static hipError_t launch_cfg(const SpmmArgs& a)
+{
+    typedef TileCfg<KS, WS, QS, WR, RM, HIGH> T;
+    MfmaParams p;
+    p.A = a.A;
+    p.B = a.B;
+    p.D = a.D;
+    p.cinfo = a.cinfo;
+    p.out = a.split_k > 1 ? a.partial : a.C;
+    p.slice_elems = a.slice_stride;
+    p.M = a.M;
+    p.N = a.N;
+    p.W = a.W;
+    p.nwin = a.W / WS;
+    p.split_k = a.split_k;
+    p.tiles_m = (a.M + T::MS - 1) / T::MS;
+    p.tiles_n = a.N / T::NS;
+    auto kern = spmm_mfma_kernel<KS, WS, QS, WR, RM, HIGH>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)T::LDS_BYTES);
+    if (e != hipSuccess)
+        return e;
+    dim3 grid(p.tiles_m * p.tiles_n, a.split_k, 1);
+    hipLaunchKernelGGL(kern, grid, dim3(T::NT), T::LDS_BYTES, a.stream, p);
+    return hipGetLastError();
+}
+
+// Four waves and 128 rows per workgroup tile for every column-block width: 1 x 4, 2 x 2 or
+// 4 x 1 waves (rows x column vectors), each wave 128, 64 or 32 rows tall.
+template <int KS, int WS, bool HIGH>
+static hipError_t launch_ns(const SpmmArgs& a)
+{
+    switch (a.Ns) {
+    case 128: return launch_cfg<KS, WS, 4, 1, 4, HIGH>(a);
+    case 64: return launch_cfg<KS, WS, 2, 2, 2, HIGH>(a);
+    case 32: return launch_cfg<KS, WS, 1, 4, 1, HIGH>(a);
+    }
+    return hipErrorInvalidValue;
+}
+
+bool mfma_supported(const SpmmArgs& a)
+{
+    if (a.vec_len != 32 || (a.Ns != 32 && a.Ns != 64 && a.Ns != 128))
+        return false;
+    if (a.M % 4 != 0 || a.M < 32)
+        return false;
+    const bool high = a.cinfo != nullptr;
+    if (!high)
+        return a.window == 32 && (a.kept == 32 || a.kept == 16 || a.kept == 12);
+    return a.window == 64 && (a.kept == 16 || a.kept == 8);
+}
+
+hipError_t launch_mfma(const SpmmArgs& a)
+{
+    const bool high = a.cinfo != nullptr;
+    if (!high) {
+        if (a.kept == 32) return launch_ns<32, 32, false>(a);
+        if (a.kept == 16) return launch_ns<32, 16, false>(a);
+        if (a.kept == 12) return launch_ns<32, 12, false>(a);
+    } else {
+        if (a.kept == 16) return launch_ns<64, 16, true>(a);
+        if (a.kept == 8) return launch_ns<64, 8, true>(a);
+    }
+    return hipErrorInvalidValue;
+}
+
+} // namespace nmspmm

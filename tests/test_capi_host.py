@@ -1,0 +1,123 @@
+"""CPU-only checks of the C-ABI: the library loads, exports every symbol include/nmspmm.h
+declares and every C++ drop-in function of include/NM-SpMM.h, and rejects bad arguments with the
+documented status codes before touching the GPU."""
+import ctypes
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+from conftest import ROOT, nmspmm
+
+
+def declared_c_symbols():
+    text = open(os.path.join(ROOT, "include", "nmspmm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(nmspmm_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = nmspmm.lib()
+    names = declared_c_symbols()
+    assert len(names) >= 16
+    for name in names:
+        assert hasattr(lib, name), name
+    assert lib.nmspmm_version() >= 100
+
+
+def test_library_exports_the_cxx_drop_in_functions():
+    out = subprocess.run(["nm", "-DC", nmspmm.LIB_PATH], check=True, capture_output=True, text=True).stdout
+    wanted = ["transIndex(int*, int, int, int, int&, int&)", "PreProcessing_low_sparsity(int*, int, int, int)",
+              "PreProcessing_high_sparsity(int*, int, int, int*, int, int, int, int)"]
+    for size in ("huge", "large", "medium", "small"):
+        wanted.append("nmGEMM_%s_matrices_low_sparsity(float*, float*, int*, float*, int, int, int, int, float, int)" % size)
+        wanted.append("nmGEMM_%s_matrices_high_sparsity(float*, float*, int*, int*, float*, int, int, int, int, float, int)" % size)
+    for w in wanted:
+        assert " T " + w in out, w
+
+
+def test_pattern_table():
+    assert nmspmm.pattern_from_sparsity(0.0) == (32, 32, False)
+    assert nmspmm.pattern_from_sparsity(0.5) == (32, 16, False)
+    assert nmspmm.pattern_from_sparsity(0.625) == (32, 12, False)
+    assert nmspmm.pattern_from_sparsity(0.75) == (64, 16, True)
+    assert nmspmm.pattern_from_sparsity(0.875) == (64, 8, True)
+    with pytest.raises(nmspmm.NmSpmmError) as e:
+        nmspmm.pattern_from_sparsity(0.3)
+    assert e.value.status == 3
+
+
+def test_sizes():
+    assert nmspmm.workspace_bytes(64, 128, 1) == 0
+    assert nmspmm.workspace_bytes(64, 128, 4) == 4 * 64 * 128 * 4
+    assert nmspmm.workspace_bytes(3, 3, 2) == 2 * 12 * 4  # slices padded to 4 floats
+    # payload of the reference's allocation rule (tests/test_nmspmm.cu:23) without its slack window
+    assert nmspmm.column_info_ints(1024, 16, 64, 4096, 128) == 32 * 64 * 64
+    assert nmspmm.column_info_ints(1024, 16, 64, 4096, 96) == 0
+
+
+FAKE = 0x1000  # an aligned non-NULL address that is never dereferenced on the error paths
+
+
+def spmm_status(**kw):
+    a = dict(A=FAKE, B=FAKE, D=FAKE, ci=None, C=FAKE, M=128, N=128, K=128, W=64, window=32, kept=16, vl=32, Ns=128,
+             split=1, ws=None, wsb=0)
+    a.update(kw)
+    return nmspmm.lib().nmspmm_spmm(a["A"], a["B"], a["D"], a["ci"], a["C"], a["M"], a["N"], a["K"], a["W"],
+                                    a["window"], a["kept"], a["vl"], a["Ns"], a["split"], a["ws"], a["wsb"], None)
+
+
+def test_spmm_rejects_bad_arguments_without_a_gpu():
+    assert spmm_status(A=None) == 1
+    assert spmm_status(C=None) == 1
+    assert spmm_status(M=0) == 2
+    assert spmm_status(N=96) == 2           # N % Ns
+    assert spmm_status(W=60) == 2           # W % kept
+    assert spmm_status(K=256) == 2          # K * kept != W * window
+    assert spmm_status(vl=5) == 3
+    assert spmm_status(kept=40) == 3        # kept > window
+    assert spmm_status(split=0) == 5
+    assert spmm_status(split=5) == 5        # more slices than windows (W / kept = 4)
+    assert spmm_status(split=2) == 6        # no workspace
+    assert spmm_status(split=2, ws=FAKE, wsb=16) == 6
+    assert spmm_status(A=FAKE + 4) == 8
+
+
+def test_named_entry_points_reject_the_other_family():
+    L = nmspmm.lib()
+    low = lambda s, tile=128: L.nmspmm_gemm_low_sparsity(tile, FAKE, FAKE, FAKE, FAKE, 128, 128, 128, 64, s, 1, None)
+    high = lambda s, ci=FAKE: L.nmspmm_gemm_high_sparsity(128, FAKE, FAKE, FAKE, ci, FAKE, 128, 128, 128, 32, s, 1, None)
+    assert low(0.75) == 4 and low(0.875) == 4
+    assert high(0.5) == 4 and high(0.625) == 4 and high(0.0) == 4
+    assert low(0.3) == 3 and high(0.3) == 3
+    assert low(0.5, tile=48) == 2
+    assert high(0.75, ci=None) == 1
+
+
+def test_preprocess_rejects_bad_arguments_without_a_gpu():
+    L = nmspmm.lib()
+    n, m = ctypes.c_int(2), ctypes.c_int(4)
+    assert L.nmspmm_trans_index_host(None, 8, 64, 2, ctypes.byref(n), ctypes.byref(m)) == 1
+    assert L.nmspmm_trans_index_host(FAKE, 6, 64, 2, ctypes.byref(n), ctypes.byref(m)) == 2  # odd window count
+    assert (n.value, m.value) == (2, 4)
+    assert L.nmspmm_preprocess_low_host(FAKE, 8, 3, 64, 32) == 2       # Q % Qs
+    assert L.nmspmm_preprocess_low_host(FAKE, 8, 4, 64, 7) == 3
+    assert L.nmspmm_preprocess_low_device(FAKE, FAKE, 8, 4, 64, 32, None) == 2  # in == out
+    assert L.nmspmm_preprocess_high_host(None, 64, 16, FAKE, 32, 4, 128, 128, 32) == 1
+    assert L.nmspmm_preprocess_high_host(FAKE, 2048, 16, FAKE, 32, 4, 128, 128, 32) == 3
+    assert L.nmspmm_preprocess_high_host(FAKE, 64, 16, FAKE, 40, 4, 128, 128, 32) == 2  # W % pN
+    assert L.nmspmm_status_string(4).decode().startswith("sparsity belongs")
+
+
+def test_split_rule_matches_reference_partition():
+    """The reference kernels give the first (windows % SPLIT_K) slices one extra window
+    (src/kernel_64x128_8x8.cu:20-37, '20 tasks over 8 slices: 3 3 3 3 2 2 2 2')."""
+    src = open(os.path.join(ROOT, "nm-spmm_amd", "csrc", "internal.h")).read()
+    assert "split_windows" in src
+    p, q = divmod(20, 8)
+    counts = [p + 1 if z < q else p for z in range(8)]
+    begins = [z * (p + 1) if z < q else z * p + q for z in range(8)]
+    assert counts == [3, 3, 3, 3, 2, 2, 2, 2]
+    assert begins == list(np.cumsum([0] + counts[:-1]))

@@ -1,0 +1,160 @@
+"""GPU parity of the multiplication, through the C-ABI, against the CPU checker (the restatement
+of the reference's nmGEMM_on_cpu) on the same seeded inputs.
+
+Tolerance: scaled max error  max|c - c_ref| / max(|c_ref|, rms(c_ref)) <= 1e-4  (the north-star
+bound for fp32 with reordered accumulation; the rms floor keeps it meaningful for signed data)."""
+import numpy as np
+import pytest
+
+from conftest import REL_TOL, datagen, kernel_geometry, nmspmm, preprocess_with_oracle, scaled_max_error, widen
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def run_gpu(oracle, d, Ns, split_k=1, fill=float("nan")):
+    """Preprocess on the checker, multiply on the GPU; returns (C, kernel family)."""
+    M, N, K, W = d["M"], d["N"], d["K"], d["W"]
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, Ns)
+    C = torch.full((M, N), fill, dtype=torch.float32, device="cuda")
+    ws = None
+    if split_k > 1:
+        ws = torch.empty(nmspmm.workspace_bytes(M, N, split_k) // 4, dtype=torch.float32, device="cuda")
+    nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), None if cinfo is None else dev(cinfo), C, M, N, K, W,
+                window, kept, d["vec_len"], Ns, split_k, ws)
+    torch.cuda.synchronize()
+    return C.cpu().numpy(), nmspmm.last_kernel()
+
+
+def check(oracle, d, got):
+    want = oracle.gemm_cpu(d["A_km"].reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), d["M"], d["N"],
+                           d["W"], d["vec_len"]).reshape(d["M"], d["N"])
+    assert np.isfinite(got).all()
+    err = scaled_max_error(got, want)
+    assert err <= REL_TOL, err
+
+
+PATTERNS = [(2, 4), (3, 8), (2, 8), (1, 8), (16, 32), (12, 32), (8, 32), (4, 32), (32, 32)]
+
+
+@pytest.mark.parametrize("n,m", PATTERNS)
+@pytest.mark.parametrize("Ns", [128, 64, 32])
+def test_matrix_core_tiles_every_pattern(oracle, n, m, Ns):
+    d = datagen.init_data(256, 256, 512, n, m, seed=100 * n + m + Ns)
+    got, fam = run_gpu(oracle, d, Ns)
+    assert fam == "mfma"
+    check(oracle, d, got)
+
+
+def test_config1_512_cubed_2of4(oracle):
+    """BASELINE config 1: M = Ncols = K = 512, 2:4, uniform(-1,1); also checked against the dense
+    product with the decompressed operand in fp64."""
+    d = datagen.init_data(512, 512, 512, 2, 4, seed=1001)
+    got, fam = run_gpu(oracle, d, 128)
+    assert fam == "mfma"
+    check(oracle, d, got)
+    dense = oracle.decompress(d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), 512, 512, d["W"])
+    want = d["A_km"].T.astype(np.float64) @ dense.astype(np.float64)
+    assert scaled_max_error(got, want) <= REL_TOL
+
+
+@pytest.mark.parametrize("M", [32, 36, 64, 100, 192, 328])
+@pytest.mark.parametrize("n,m,Ns", [(2, 4, 128), (1, 8, 128), (2, 8, 64), (3, 8, 32)])
+def test_ragged_row_counts(oracle, M, n, m, Ns):
+    d = datagen.init_data(M, 256, 256, n, m, seed=M + n)
+    got, fam = run_gpu(oracle, d, Ns)
+    assert fam == "mfma"
+    check(oracle, d, got)
+
+
+@pytest.mark.parametrize("split_k", [2, 3, 4, 8, 16])
+@pytest.mark.parametrize("n,m,Ns", [(2, 4, 128), (1, 8, 128), (2, 8, 32)])
+def test_split_k_through_workspace(oracle, split_k, n, m, Ns):
+    d = datagen.init_data(128, 256, 1280, n, m, seed=split_k)  # 40 or 20 windows: uneven splits included
+    got, _ = run_gpu(oracle, d, Ns, split_k)
+    check(oracle, d, got)
+    one, _ = run_gpu(oracle, d, Ns, 1)
+    assert scaled_max_error(got, one) <= REL_TOL
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 30])
+@pytest.mark.parametrize("n,m", [(1, 8), (2, 8)])
+def test_skinny_rows_take_the_simt_path(oracle, M, n, m):
+    d = datagen.init_data(M, 512, 1024, n, m, seed=M, dist="normal", b_scale=0.02)
+    for split_k in (1, 4):
+        got, fam = run_gpu(oracle, d, 128, split_k)
+        assert fam == "simt"
+        check(oracle, d, got)
+
+
+@pytest.mark.parametrize("vl,n,m", [(4, 2, 4), (8, 1, 8), (16, 3, 8)])
+def test_short_vectors_take_the_simt_path(oracle, vl, n, m):
+    """Per-vector length below 32: indices are used as generated (no widening), any window."""
+    M, N, K = 64, 128, 256
+    d = datagen.init_data(M, N, K, n, m, vec_len=vl, seed=vl)
+    W, Q = d["W"], d["Q"]
+    D = d["DT"].reshape(-1).copy()
+    oracle.preprocess_low(D, W, Q, 64, vl)
+    C = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), None, C, M, N, K, W, m, n, vl, 64)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == "simt"
+    check(oracle, d, C.cpu().numpy())
+
+
+@pytest.mark.parametrize("sparsity,n,m", [(0.5, 16, 32), (0.625, 12, 32), (0.0, 32, 32), (0.75, 8, 32), (0.875, 4, 32)])
+@pytest.mark.parametrize("tile", [128, 64, 32])
+def test_named_entry_points_with_gpu_preprocessing(oracle, sparsity, n, m, tile):
+    """The reference driver's sequence (tests/test_nmspmm.cu:72-97) with pruning_M = 32: preprocess
+    (here on the GPU), then the named launcher chosen by sparsity."""
+    M, N, K = 128, 256, 256
+    d = datagen.init_data(M, N, K, n, m, seed=int(sparsity * 1000) + tile)
+    W, Q = d["W"], d["Q"]
+    A, B, C = dev(d["A_km"]), dev(d["BT"]), torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    DT = dev(d["DT"].reshape(-1))
+    Dp = torch.empty_like(DT)
+    if sparsity < 0.7:
+        nmspmm.preprocess_low_device(DT, Dp, W, Q, tile)
+        nmspmm.gemm_low_sparsity(tile, A, B, Dp, C, M, N, K, W, sparsity, 1)
+    else:
+        pn, pm = nmspmm.trans_index_device(DT, W, N, Q, n, m)
+        ci = torch.empty(nmspmm.column_info_ints(W, pn, pm, N, tile), dtype=torch.int32, device="cuda")
+        nmspmm.preprocess_high_device(ci, pm, pn, DT, Dp, W, Q, N, tile)
+        nmspmm.gemm_high_sparsity(tile, A, B, Dp, ci, C, M, N, K, W, sparsity, 2)  # split 2 via cached workspace
+    torch.cuda.synchronize()
+    check(oracle, d, C.cpu().numpy())
+
+
+def test_llm_layer_shape_2of8(oracle):
+    """One BASELINE config-3 shape (M = 512, K = 4096, Ncols = 11008, 2:8, N(0,1) x N(0,0.02^2))."""
+    d = datagen.init_data(512, 11008, 4096, 2, 8, seed=3001, dist="normal", b_scale=0.02)
+    got, fam = run_gpu(oracle, d, 128)
+    assert fam == "mfma"
+    check(oracle, d, got)
+
+
+@pytest.mark.parametrize("n,m", [(2, 4), (2, 8), (1, 8)])
+def test_full_size_4096_cubed_checksums_and_row_sample(oracle, n, m):
+    """BASELINE config 2 at full size.  The checker would need minutes for all of C, so: (1) rows
+    [0,32) and [4064,4096) are compared with the checker; (2) checksums that hold for any size:
+    C . 1 = A . (B_dense . 1) and 1^T . C = (1^T . A) . B_dense, evaluated in fp64 from the inputs."""
+    M = N = K = 4096
+    d = datagen.init_data(M, N, K, n, m, seed=2000 + n * 10 + m)
+    got, fam = run_gpu(oracle, d, 128)
+    assert fam == "mfma" and np.isfinite(got).all()
+    A, B, D = d["A_km"].reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1)
+    for rows in ((0, 32), (M - 32, M)):
+        want = oracle.gemm_cpu(A, B, D, M, N, d["W"], rows=rows).reshape(M, N)[rows[0]:rows[1]]
+        assert scaled_max_error(got[rows[0]:rows[1]], want) <= REL_TOL
+    dense = oracle.decompress(B, D, K, N, d["W"]).astype(np.float64)
+    A64 = d["A_km"].T.astype(np.float64)  # M x K
+    row_sums = A64 @ dense.sum(axis=1)
+    col_sums = A64.sum(axis=0) @ dense
+    g64 = got.astype(np.float64)
+    scale = np.sqrt(d["W"] * N / 9.0)  # std of a row/column sum of C for uniform(-1,1) operands
+    assert np.max(np.abs(g64.sum(axis=1) - row_sums)) <= 1e-4 * scale
+    assert np.max(np.abs(g64.sum(axis=0) - col_sums)) <= 1e-4 * scale
