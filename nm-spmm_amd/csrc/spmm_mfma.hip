@@ -69,6 +69,19 @@ struct TileCfg {
     static_assert(WS % 2 == 0, "two compressed rows per MFMA");
 };
 
+// Buffer descriptors give branch-free guarded loads: an offset at or beyond num_records reads 0
+// without touching memory, so "this slot has nothing to load" is just an out-of-range offset.
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+__device__ inline float4 buffer_load_f4(__amdgpu_buffer_rsrc_t r, uint32_t byte_off)
+{
+    auto v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
+    return *reinterpret_cast<float4*>(&v);
+}
+constexpr uint32_t kNoLoad = 0x80000000u;  // beyond any window's num_records
+
 template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
 __global__ void __launch_bounds__(64 * QS * WR)
 spmm_mfma_kernel(const MfmaParams p)
@@ -119,40 +132,55 @@ spmm_mfma_kernel(const MfmaParams p)
     const float* const Bblk = p.B + bj;
     const int32_t* const Dvec = p.D + (size_t)tile_n * p.W * QS + vec;
     const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)tile_n * p.nwin * KS : nullptr;
+    // Bytes addressable from the first element of a window's A / B tile.  Columns past M in a
+    // row that is not the last one alias the next row (finite garbage that only reaches C rows
+    // >= M, which are never stored); the descriptor bound keeps the last row inside the matrix.
+    const uint32_t a_bytes = (uint32_t)(((size_t)(KS - 1) * M + (M - bi)) * sizeof(float));
+    const uint32_t b_bytes = (uint32_t)(((size_t)(WS - 1) * N + (N - bj)) * sizeof(float));
 
     // ---- per-thread staging slots -----------------------------------------------------------
     float4 areg[T::A_SLOTS];
     float4 breg[T::B_SLOTS];
-    int acol[T::A_SLOTS];  // HIGH: source row of each A slot for the window to be loaded next
-
-    auto load_cinfo = [&](int w) {
+    uint32_t a_off[T::A_SLOTS];  // byte offset of each A slot inside the window (kNoLoad: none)
+    uint32_t b_off[T::B_SLOTS];
 #pragma unroll
-        for (int s = 0; s < T::A_SLOTS; ++s) {
-            const int lin = tid + s * T::NT;
-            const int row = lin / T::A_F4_ROW;
-            acol[s] = (lin < T::A_F4) ? Cinfo[(size_t)w * KS + row] : -1;
-        }
-    };
-    auto load_tiles = [&](int w) {
-        const float* Aw = Ablk + (size_t)w * KS * M;
+    for (int s = 0; s < T::B_SLOTS; ++s) {
+        const int lin = tid + s * T::NT;
+        const int row = lin / T::B_F4_ROW;
+        const int c4 = (lin % T::B_F4_ROW) * 4;
+        b_off[s] = lin < T::B_F4 ? (uint32_t)(((size_t)row * N + c4) * sizeof(float)) : kNoLoad;
+    }
+    if (!HIGH) {
 #pragma unroll
         for (int s = 0; s < T::A_SLOTS; ++s) {
             const int lin = tid + s * T::NT;
             const int row = lin / T::A_F4_ROW;
             const int c4 = (lin % T::A_F4_ROW) * 4;
-            const int src = HIGH ? acol[s] : row;
-            if (lin < T::A_F4 && src >= 0 && bi + c4 < M)
-                areg[s] = *reinterpret_cast<const float4*>(Aw + (size_t)src * M + c4);
+            a_off[s] = lin < T::A_F4 ? (uint32_t)(((size_t)row * M + c4) * sizeof(float)) : kNoLoad;
         }
-        const float* Bw = Bblk + (size_t)w * WS * N;
+    }
+
+    // HIGH: the A rows of window w are the ones column_info lists; -1 means "no such row".
+    auto load_cinfo = [&](int w) {
 #pragma unroll
-        for (int s = 0; s < T::B_SLOTS; ++s) {
-            const int lin = tid + s * T::NT;
-            const int row = lin / T::B_F4_ROW;
-            const int c4 = (lin % T::B_F4_ROW) * 4;
-            if (lin < T::B_F4)
-                breg[s] = *reinterpret_cast<const float4*>(Bw + (size_t)row * N + c4);
+        for (int s = 0; s < T::A_SLOTS; ++s) {
+            const int lin = min(tid + s * T::NT, T::A_F4 - 1);
+            const int row = lin / T::A_F4_ROW;
+            const int c4 = (lin % T::A_F4_ROW) * 4;
+            const int src = Cinfo[(size_t)w * KS + row];
+            a_off[s] = (src >= 0 && tid + s * T::NT < T::A_F4)
+                           ? (uint32_t)(((size_t)src * M + c4) * sizeof(float)) : kNoLoad;
         }
+    };
+    auto load_tiles = [&](int w) {
+        const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w * KS * M, a_bytes);
+#pragma unroll
+        for (int s = 0; s < T::A_SLOTS; ++s)
+            areg[s] = buffer_load_f4(ra, a_off[s]);
+        const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bblk + (size_t)w * WS * N, b_bytes);
+#pragma unroll
+        for (int s = 0; s < T::B_SLOTS; ++s)
+            breg[s] = buffer_load_f4(rb, b_off[s]);
     };
     auto store_tiles = [&](int buf) {
         float* Ab = As + buf * T::AROWS * T::ASTR;
@@ -161,7 +189,7 @@ spmm_mfma_kernel(const MfmaParams p)
             const int lin = tid + s * T::NT;
             const int row = lin / T::A_F4_ROW;
             const int c4 = (lin % T::A_F4_ROW) * 4;
-            if (lin < T::A_F4)
+            if (T::A_F4 % T::NT == 0 || s + 1 < T::A_SLOTS || lin < T::A_F4)
                 *reinterpret_cast<float4*>(Ab + row * T::ASTR + c4) = areg[s];
         }
         float* Bb = Bs + buf * WS * T::BSTR;
@@ -170,7 +198,7 @@ spmm_mfma_kernel(const MfmaParams p)
             const int lin = tid + s * T::NT;
             const int row = lin / T::B_F4_ROW;
             const int c4 = (lin % T::B_F4_ROW) * 4;
-            if (lin < T::B_F4)
+            if (T::B_F4 % T::NT == 0 || s + 1 < T::B_SLOTS || lin < T::B_F4)
                 *reinterpret_cast<float4*>(Bb + row * T::BSTR + c4) = breg[s];
         }
     };
@@ -194,12 +222,6 @@ spmm_mfma_kernel(const MfmaParams p)
 #pragma unroll
         for (int v = 0; v < 16; ++v)
             acc[b][v] = 0.0f;
-
-#pragma unroll
-    for (int s = 0; s < T::A_SLOTS; ++s) {
-        areg[s] = make_float4(0.f, 0.f, 0.f, 0.f);
-        acol[s] = -1;
-    }
 
     // ---- prologue ---------------------------------------------------------------------------
     if (w_count > 0) {
@@ -227,15 +249,22 @@ spmm_mfma_kernel(const MfmaParams p)
                 load_cinfo(w + 2);
         }
 
+        // All operand fragments of the window are requested before the first MFMA, so LDS
+        // latency is paid once per window and overlaps the matrix pipe.
         const float* Ab = As + (t & 1) * T::AROWS * T::ASTR;
         const float* Bb = Bs + (t & 1) * WS * T::BSTR + b_lane;
+        afrag_t av[T::KSTEPS];
+        float bv[T::KSTEPS];
 #pragma unroll
         for (int s = 0; s < T::KSTEPS; ++s) {
-            const afrag_t av = *reinterpret_cast<const afrag_t*>(Ab + aoff[s]);
-            const float bv = Bb[2 * s * T::BSTR];
+            av[s] = *reinterpret_cast<const afrag_t*>(Ab + aoff[s]);
+            bv[s] = Bb[2 * s * T::BSTR];
+        }
+#pragma unroll
+        for (int s = 0; s < T::KSTEPS; ++s) {
 #pragma unroll
             for (int b = 0; b < RM; ++b)
-                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_get(av, b), bv, acc[b], 0, 0, 0);
+                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_get(av[s], b), bv[s], acc[b], 0, 0, 0);
         }
 
         if (more) {
