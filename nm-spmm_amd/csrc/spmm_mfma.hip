@@ -10,9 +10,12 @@
 //    per-lane LDS row offset; no data is moved to perform it.
 //  * The wave's RM row blocks interleave rows (block b holds rows 4*r + b), so one 128-bit LDS
 //    read yields the A operands of all RM blocks and the B operand is reused RM times.
-//  * A (window rows x Ms, k-major as in global memory) and B (kept rows x Ns) tiles are staged
-//    global -> registers -> LDS with 128-bit accesses, double buffered: the loads of window t+1
-//    are in flight while window t is multiplied, one barrier per window.
+//  * The A tile (window rows x Ms, k-major as in global memory) is shared by the tile's column
+//    vectors, so it is staged global -> registers -> LDS with 128-bit accesses, double
+//    buffered: the loads of window t+1 are in flight while window t is multiplied, one barrier
+//    per window.  A B element is consumed by exactly one wave, so B never touches LDS: each
+//    lane loads its MFMA operands (two 128-byte row segments per wave and k-step) straight
+//    from global memory one window ahead.
 //  * High-sparsity layout: only the rows listed in column_info are staged (the indices are
 //    already ranks into that list); column_info is fetched two windows ahead.
 //  * Workgroup ids are remapped so that the tiles resident on one XCD form a compact patch of
@@ -57,15 +60,11 @@ struct TileCfg {
     static constexpr int NT = 64 * QS * WR;
     static constexpr int AROWS = HIGH ? (KS < WS * QS ? KS : WS * QS) : KS;
     static constexpr int ASTR = MS;       // floats per staged A row
-    static constexpr int BSTR = NS + 32;  // odd rows land in the other half of the banks
     static constexpr int A_F4_ROW = MS / 4;
-    static constexpr int B_F4_ROW = NS / 4;
     static constexpr int A_F4 = AROWS * A_F4_ROW;
-    static constexpr int B_F4 = WS * B_F4_ROW;
     static constexpr int A_SLOTS = (A_F4 + NT - 1) / NT;
-    static constexpr int B_SLOTS = (B_F4 + NT - 1) / NT;
     static constexpr int KSTEPS = WS / 2;
-    static constexpr size_t LDS_BYTES = sizeof(float) * 2 * (size_t)(AROWS * ASTR + WS * BSTR);
+    static constexpr size_t LDS_BYTES = sizeof(float) * 2 * (size_t)(AROWS * ASTR);
     static_assert(WS % 2 == 0, "two compressed rows per MFMA");
 };
 
@@ -80,6 +79,10 @@ __device__ inline float4 buffer_load_f4(__amdgpu_buffer_rsrc_t r, uint32_t byte_
     auto v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
     return *reinterpret_cast<float4*>(&v);
 }
+__device__ inline float buffer_load_f1(__amdgpu_buffer_rsrc_t r, uint32_t byte_off, uint32_t s_off)
+{
+    return __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, byte_off, s_off, 0));
+}
 constexpr uint32_t kNoLoad = 0x80000000u;  // beyond any window's num_records
 
 template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
@@ -89,8 +92,7 @@ spmm_mfma_kernel(const MfmaParams p)
     typedef TileCfg<KS, WS, QS, WR, RM, HIGH> T;
     typedef typename AFrag<RM>::type afrag_t;
     extern __shared__ __align__(16) float lds[];
-    float* const As = lds;                          // [2][AROWS][ASTR]
-    float* const Bs = lds + 2 * T::AROWS * T::ASTR;  // [2][WS][BSTR]
+    float* const As = lds;  // [2][AROWS][ASTR]
 
     // ---- which tile -------------------------------------------------------------------------
     // Consecutive workgroup ids go to consecutive XCDs; give every XCD a contiguous run of
@@ -121,7 +123,7 @@ spmm_mfma_kernel(const MfmaParams p)
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int vec = wave % QS;   // column vector inside the tile
     const int grp = wave / QS;   // row group inside the tile
     const int h = lane >> 5;     // which of the two compressed rows of a k-step
@@ -129,27 +131,19 @@ spmm_mfma_kernel(const MfmaParams p)
 
     const int M = p.M, N = p.N;
     const float* const Ablk = p.A + bi;
-    const float* const Bblk = p.B + bj;
+    const float* const Bvec = p.B + bj + vec * 32;
     const int32_t* const Dvec = p.D + (size_t)tile_n * p.W * QS + vec;
     const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)tile_n * p.nwin * KS : nullptr;
-    // Bytes addressable from the first element of a window's A / B tile.  Columns past M in a
-    // row that is not the last one alias the next row (finite garbage that only reaches C rows
-    // >= M, which are never stored); the descriptor bound keeps the last row inside the matrix.
+    // Bytes addressable from the first element of a window's A tile / B vector.  Columns past
+    // M in an A row that is not the last one alias the next row (finite garbage that only
+    // reaches C rows >= M, which are never stored); the descriptor bound keeps the last row
+    // inside the matrix.
     const uint32_t a_bytes = (uint32_t)(((size_t)(KS - 1) * M + (M - bi)) * sizeof(float));
-    const uint32_t b_bytes = (uint32_t)(((size_t)(WS - 1) * N + (N - bj)) * sizeof(float));
+    const uint32_t b_bytes = (uint32_t)(((size_t)(WS - 1) * N + 32) * sizeof(float));
 
-    // ---- per-thread staging slots -----------------------------------------------------------
+    // ---- A staging: slot s of thread tid is float4 number tid + s*NT of the [AROWS][MS] tile ----
     float4 areg[T::A_SLOTS];
-    float4 breg[T::B_SLOTS];
-    uint32_t a_off[T::A_SLOTS];  // byte offset of each A slot inside the window (kNoLoad: none)
-    uint32_t b_off[T::B_SLOTS];
-#pragma unroll
-    for (int s = 0; s < T::B_SLOTS; ++s) {
-        const int lin = tid + s * T::NT;
-        const int row = lin / T::B_F4_ROW;
-        const int c4 = (lin % T::B_F4_ROW) * 4;
-        b_off[s] = lin < T::B_F4 ? (uint32_t)(((size_t)row * N + c4) * sizeof(float)) : kNoLoad;
-    }
+    uint32_t a_off[T::A_SLOTS];  // byte offset inside the window (kNoLoad: nothing to load)
     if (!HIGH) {
 #pragma unroll
         for (int s = 0; s < T::A_SLOTS; ++s) {
@@ -159,8 +153,7 @@ spmm_mfma_kernel(const MfmaParams p)
             a_off[s] = lin < T::A_F4 ? (uint32_t)(((size_t)row * M + c4) * sizeof(float)) : kNoLoad;
         }
     }
-
-    // HIGH: the A rows of window w are the ones column_info lists; -1 means "no such row".
+    // HIGH: staged row r of window w is A row column_info[w][r]; -1 means "no such row".
     auto load_cinfo = [&](int w) {
 #pragma unroll
         for (int s = 0; s < T::A_SLOTS; ++s) {
@@ -172,17 +165,13 @@ spmm_mfma_kernel(const MfmaParams p)
                            ? (uint32_t)(((size_t)src * M + c4) * sizeof(float)) : kNoLoad;
         }
     };
-    auto load_tiles = [&](int w) {
+    auto load_a = [&](int w) {
         const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w * KS * M, a_bytes);
 #pragma unroll
         for (int s = 0; s < T::A_SLOTS; ++s)
             areg[s] = buffer_load_f4(ra, a_off[s]);
-        const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bblk + (size_t)w * WS * N, b_bytes);
-#pragma unroll
-        for (int s = 0; s < T::B_SLOTS; ++s)
-            breg[s] = buffer_load_f4(rb, b_off[s]);
     };
-    auto store_tiles = [&](int buf) {
+    auto store_a = [&](int buf) {
         float* Ab = As + buf * T::AROWS * T::ASTR;
 #pragma unroll
         for (int s = 0; s < T::A_SLOTS; ++s) {
@@ -192,29 +181,25 @@ spmm_mfma_kernel(const MfmaParams p)
             if (T::A_F4 % T::NT == 0 || s + 1 < T::A_SLOTS || lin < T::A_F4)
                 *reinterpret_cast<float4*>(Ab + row * T::ASTR + c4) = areg[s];
         }
-        float* Bb = Bs + buf * WS * T::BSTR;
+    };
+
+    // ---- per-wave operands that bypass LDS: B values and indices of compressed rows 2s + h ------
+    float b_next[T::KSTEPS];
+    int idx_next[T::KSTEPS];
+    const uint32_t b_lane = (uint32_t)(((size_t)h * N + j) * sizeof(float));
+    auto load_b_idx = [&](int w) {
+        const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)w * WS * N, b_bytes);
+        const int32_t* Dw = Dvec + ((size_t)w * WS + h) * QS;
 #pragma unroll
-        for (int s = 0; s < T::B_SLOTS; ++s) {
-            const int lin = tid + s * T::NT;
-            const int row = lin / T::B_F4_ROW;
-            const int c4 = (lin % T::B_F4_ROW) * 4;
-            if (T::B_F4 % T::NT == 0 || s + 1 < T::B_SLOTS || lin < T::B_F4)
-                *reinterpret_cast<float4*>(Bb + row * T::BSTR + c4) = breg[s];
+        for (int s = 0; s < T::KSTEPS; ++s) {
+            b_next[s] = buffer_load_f1(rb, b_lane, (uint32_t)(2 * s * N * sizeof(float)));
+            idx_next[s] = Dw[(size_t)(2 * s) * QS];
         }
     };
 
-    // Index of compressed row (2s + h) of window w for this wave's column vector.
-    int idx_next[T::KSTEPS];
-    auto load_idx = [&](int w) {
-        const int32_t* Dw = Dvec + ((size_t)w * WS + h) * QS;
-#pragma unroll
-        for (int s = 0; s < T::KSTEPS; ++s)
-            idx_next[s] = Dw[(size_t)(2 * s) * QS];
-    };
-
     const int a_lane = grp * (RM * 32) + j * RM;  // first of this lane's RM adjacent rows
-    const int b_lane = h * T::BSTR + vec * 32 + j;
     int aoff[T::KSTEPS];
+    float bv[T::KSTEPS];
 
     floatx16 acc[RM];
 #pragma unroll
@@ -227,14 +212,16 @@ spmm_mfma_kernel(const MfmaParams p)
     if (w_count > 0) {
         if (HIGH)
             load_cinfo(w_begin);
-        load_tiles(w_begin);
-        load_idx(w_begin);
+        load_a(w_begin);
+        load_b_idx(w_begin);
         if (HIGH && w_count > 1)
             load_cinfo(w_begin + 1);
-        store_tiles(0);
+        store_a(0);
 #pragma unroll
-        for (int s = 0; s < T::KSTEPS; ++s)
+        for (int s = 0; s < T::KSTEPS; ++s) {
             aoff[s] = idx_next[s] * T::ASTR + a_lane;
+            bv[s] = b_next[s];
+        }
     }
     __syncthreads();
 
@@ -243,23 +230,17 @@ spmm_mfma_kernel(const MfmaParams p)
         const int w = w_begin + t;
         const bool more = t + 1 < w_count;
         if (more) {
-            load_tiles(w + 1);
-            load_idx(w + 1);
+            load_a(w + 1);
+            load_b_idx(w + 1);
             if (HIGH && t + 2 < w_count)
                 load_cinfo(w + 2);
         }
 
-        // All operand fragments of the window are requested before the first MFMA, so LDS
-        // latency is paid once per window and overlaps the matrix pipe.
         const float* Ab = As + (t & 1) * T::AROWS * T::ASTR;
-        const float* Bb = Bs + (t & 1) * WS * T::BSTR + b_lane;
         afrag_t av[T::KSTEPS];
-        float bv[T::KSTEPS];
 #pragma unroll
-        for (int s = 0; s < T::KSTEPS; ++s) {
+        for (int s = 0; s < T::KSTEPS; ++s)
             av[s] = *reinterpret_cast<const afrag_t*>(Ab + aoff[s]);
-            bv[s] = Bb[2 * s * T::BSTR];
-        }
 #pragma unroll
         for (int s = 0; s < T::KSTEPS; ++s) {
 #pragma unroll
@@ -268,10 +249,12 @@ spmm_mfma_kernel(const MfmaParams p)
         }
 
         if (more) {
-            store_tiles((t + 1) & 1);
+            store_a((t + 1) & 1);
 #pragma unroll
-            for (int s = 0; s < T::KSTEPS; ++s)
+            for (int s = 0; s < T::KSTEPS; ++s) {
                 aoff[s] = idx_next[s] * T::ASTR + a_lane;
+                bv[s] = b_next[s];
+            }
         }
         __syncthreads();
     }
