@@ -68,6 +68,25 @@ struct TileCfg {
     static_assert(WS % 2 == 0, "two compressed rows per MFMA");
 };
 
+// The two halves of the double-buffered A tile are separate LDS objects (not one array indexed
+// by t & 1): the compiler can then prove that the fragment reads of one buffer do not alias the
+// asynchronous global->LDS writes into the other and does not serialise them with a vmcnt(0)
+// wait.  They live at namespace scope, one pair per tile size in floats; a kernel is charged
+// only for the pair it references.
+#define NMSPMM_LDS_PAIR(FLOATS)                                          \
+    __shared__ __align__(16) float g_lds_a0_##FLOATS[FLOATS];           \
+    __shared__ __align__(16) float g_lds_a1_##FLOATS[FLOATS];           \
+    template <> struct LdsPair<FLOATS> {                                 \
+        __device__ static float* first() { return g_lds_a0_##FLOATS; }  \
+        __device__ static float* second() { return g_lds_a1_##FLOATS; } \
+    };
+template <int FLOATS> struct LdsPair;
+NMSPMM_LDS_PAIR(1024)
+NMSPMM_LDS_PAIR(2048)
+NMSPMM_LDS_PAIR(4096)
+NMSPMM_LDS_PAIR(8192)
+NMSPMM_LDS_PAIR(16384)
+
 // Buffer descriptors give branch-free guarded loads: an offset at or beyond num_records reads 0
 // without touching memory, so "this slot has nothing to load" is just an out-of-range offset.
 __device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes)
@@ -79,20 +98,50 @@ __device__ inline float4 buffer_load_f4(__amdgpu_buffer_rsrc_t r, uint32_t byte_
     auto v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
     return *reinterpret_cast<float4*>(&v);
 }
+typedef __attribute__((address_space(3))) float lds_f32;
 __device__ inline float buffer_load_f1(__amdgpu_buffer_rsrc_t r, uint32_t byte_off, uint32_t s_off)
 {
     return __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, byte_off, s_off, 0));
 }
+// 128-bit global -> LDS load without a register stop-over: lane l's 16 bytes land at
+// dst + 16*l (dst is wave-uniform).  Completion is tracked by vmcnt.  Kept out of the kernel
+// template: the host pass drops a kernel template that names this builtin directly.
+__device__ inline void buffer_load_f4_to_lds(__amdgpu_buffer_rsrc_t r, lds_f32* dst, uint32_t byte_off)
+{
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, dst, 16, byte_off, 0, 0, 0);
+}
 constexpr uint32_t kNoLoad = 0x80000000u;  // beyond any window's num_records
+constexpr int kWaitVm0 = 0x0F70;           // s_waitcnt vmcnt(0), other counters untouched
+
+// Tuning knobs (compile-time): minimum waves per SIMD the register allocation must allow, the
+// tile-walk band height, and the (waves along M, 32-row blocks per wave) of each tile width.
+#ifndef NMSPMM_OCC
+#define NMSPMM_OCC 1
+#endif
+#ifndef NMSPMM_LDS_MIN
+#define NMSPMM_LDS_MIN 0  // extra dynamic LDS bytes to claim (caps workgroups per CU)
+#endif
+#ifndef NMSPMM_GROUP
+#define NMSPMM_GROUP 8
+#endif
+#ifndef NMSPMM_CFG128
+#define NMSPMM_CFG128 1, 4
+#endif
+#ifndef NMSPMM_CFG64
+#define NMSPMM_CFG64 2, 2
+#endif
+#ifndef NMSPMM_CFG32
+#define NMSPMM_CFG32 4, 1
+#endif
 
 template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
-__global__ void __launch_bounds__(64 * QS * WR)
+__global__ void __launch_bounds__(64 * QS * WR, NMSPMM_OCC)
 spmm_mfma_kernel(const MfmaParams p)
 {
     typedef TileCfg<KS, WS, QS, WR, RM, HIGH> T;
     typedef typename AFrag<RM>::type afrag_t;
-    extern __shared__ __align__(16) float lds[];
-    float* const As = lds;  // [2][AROWS][ASTR]
+    float* const As0 = LdsPair<T::AROWS * T::ASTR>::first();
+    float* const As1 = LdsPair<T::AROWS * T::ASTR>::second();
 
     // ---- which tile -------------------------------------------------------------------------
     // Consecutive workgroup ids go to consecutive XCDs; give every XCD a contiguous run of
@@ -105,7 +154,7 @@ spmm_mfma_kernel(const MfmaParams p)
         const int xcd = id % kXcds, loc = id / kXcds;
         logical = xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc;
     }
-    constexpr int GROUP = 8;
+    constexpr int GROUP = NMSPMM_GROUP;
     int tile_m, tile_n;
     {
         const int band = logical / (GROUP * p.tiles_n);
@@ -115,6 +164,10 @@ spmm_mfma_kernel(const MfmaParams p)
         tile_m = first_m + in_band % rows;
         tile_n = in_band / rows;
     }
+#ifdef NMSPMM_EXP_SAMETILE
+    tile_m = 0;
+    tile_n = 0;
+#endif
     const int bi = tile_m * T::MS;
     const int bj = tile_n * T::NS;
 
@@ -141,8 +194,10 @@ spmm_mfma_kernel(const MfmaParams p)
     const uint32_t a_bytes = (uint32_t)(((size_t)(KS - 1) * M + (M - bi)) * sizeof(float));
     const uint32_t b_bytes = (uint32_t)(((size_t)(WS - 1) * N + 32) * sizeof(float));
 
-    // ---- A staging: slot s of thread tid is float4 number tid + s*NT of the [AROWS][MS] tile ----
-    float4 areg[T::A_SLOTS];
+    // ---- A staging: global -> LDS without passing through registers -------------------------------
+    // Slot s of wave `wave` is the 1 KiB chunk number wave + s*NW of the [AROWS][MS] tile: float4
+    // number 64*chunk + lane, which is also where an LDS-direct 128-bit load puts lane's data.
+    constexpr int NW = T::NT / 64;
     uint32_t a_off[T::A_SLOTS];  // byte offset inside the window (kNoLoad: nothing to load)
     if (!HIGH) {
 #pragma unroll
@@ -155,31 +210,23 @@ spmm_mfma_kernel(const MfmaParams p)
     }
     // HIGH: staged row r of window w is A row column_info[w][r]; -1 means "no such row".
     auto load_cinfo = [&](int w) {
-#pragma unroll
-        for (int s = 0; s < T::A_SLOTS; ++s) {
-            const int lin = min(tid + s * T::NT, T::A_F4 - 1);
-            const int row = lin / T::A_F4_ROW;
-            const int c4 = (lin % T::A_F4_ROW) * 4;
-            const int src = Cinfo[(size_t)w * KS + row];
-            a_off[s] = (src >= 0 && tid + s * T::NT < T::A_F4)
-                           ? (uint32_t)(((size_t)src * M + c4) * sizeof(float)) : kNoLoad;
-        }
-    };
-    auto load_a = [&](int w) {
-        const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w * KS * M, a_bytes);
-#pragma unroll
-        for (int s = 0; s < T::A_SLOTS; ++s)
-            areg[s] = buffer_load_f4(ra, a_off[s]);
-    };
-    auto store_a = [&](int buf) {
-        float* Ab = As + buf * T::AROWS * T::ASTR;
+        const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cinfo + (size_t)w * KS, KS * sizeof(int32_t));
 #pragma unroll
         for (int s = 0; s < T::A_SLOTS; ++s) {
             const int lin = tid + s * T::NT;
             const int row = lin / T::A_F4_ROW;
             const int c4 = (lin % T::A_F4_ROW) * 4;
-            if (T::A_F4 % T::NT == 0 || s + 1 < T::A_SLOTS || lin < T::A_F4)
-                *reinterpret_cast<float4*>(Ab + row * T::ASTR + c4) = areg[s];
+            const int src = __builtin_amdgcn_raw_buffer_load_b32(rc, row * (int)sizeof(int32_t), 0, 0);
+            a_off[s] = (src >= 0 && lin < T::A_F4) ? (uint32_t)(((size_t)src * M + c4) * sizeof(float)) : kNoLoad;
+        }
+    };
+    auto load_a = [&](int w, float* dst) {
+        const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w * KS * M, a_bytes);
+        lds_f32* Ab = (lds_f32*)dst + wave * 256;
+#pragma unroll
+        for (int s = 0; s < T::A_SLOTS; ++s) {
+            if (T::A_F4 % T::NT == 0 || s + 1 < T::A_SLOTS || (wave + s * NW) * 64 < T::A_F4)
+                buffer_load_f4_to_lds(ra, Ab + s * NW * 256, a_off[s]);
         }
     };
 
@@ -187,13 +234,14 @@ spmm_mfma_kernel(const MfmaParams p)
     float b_next[T::KSTEPS];
     int idx_next[T::KSTEPS];
     const uint32_t b_lane = (uint32_t)(((size_t)h * N + j) * sizeof(float));
+    const uint32_t d_lane = (uint32_t)(h * QS * sizeof(int32_t));
     auto load_b_idx = [&](int w) {
         const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)w * WS * N, b_bytes);
-        const int32_t* Dw = Dvec + ((size_t)w * WS + h) * QS;
+        const __amdgpu_buffer_rsrc_t rd = make_rsrc(Dvec + (size_t)w * WS * QS, ((WS - 1) * QS + 1) * sizeof(int32_t));
 #pragma unroll
         for (int s = 0; s < T::KSTEPS; ++s) {
             b_next[s] = buffer_load_f1(rb, b_lane, (uint32_t)(2 * s * N * sizeof(float)));
-            idx_next[s] = Dw[(size_t)(2 * s) * QS];
+            idx_next[s] = __builtin_amdgcn_raw_buffer_load_b32(rd, d_lane, 2 * s * QS * (int)sizeof(int32_t), 0);
         }
     };
 
@@ -209,38 +257,42 @@ spmm_mfma_kernel(const MfmaParams p)
             acc[b][v] = 0.0f;
 
     // ---- prologue ---------------------------------------------------------------------------
+    const int w_last = w_begin + w_count - 1;
     if (w_count > 0) {
         if (HIGH)
             load_cinfo(w_begin);
-        load_a(w_begin);
+        load_a(w_begin, As0);
         load_b_idx(w_begin);
-        if (HIGH && w_count > 1)
-            load_cinfo(w_begin + 1);
-        store_a(0);
+        if (HIGH)
+            load_cinfo(min(w_begin + 1, w_last));
 #pragma unroll
         for (int s = 0; s < T::KSTEPS; ++s) {
             aoff[s] = idx_next[s] * T::ASTR + a_lane;
             bv[s] = b_next[s];
         }
     }
+    __builtin_amdgcn_s_waitcnt(kWaitVm0);
     __syncthreads();
 
     // ---- main loop: one window per iteration --------------------------------------------------
-    for (int t = 0; t < w_count; ++t) {
+    // The body is one basic block: loads for the next window are always issued (the last
+    // iteration re-reads its own window into the idle buffer, which is harmless).  The A tile of
+    // window t+1 streams into the other LDS buffer while window t is multiplied; the wave waits
+    // for its own loads, then the barrier publishes the buffer to the other waves.
+    auto window = [&](int t, const float* cur, float* nxt) {
         const int w = w_begin + t;
-        const bool more = t + 1 < w_count;
-        if (more) {
-            load_a(w + 1);
-            load_b_idx(w + 1);
-            if (HIGH && t + 2 < w_count)
-                load_cinfo(w + 2);
-        }
+        const int w1 = min(w + 1, w_last);
+        load_a(w1, nxt);
+        load_b_idx(w1);
+        if (HIGH)
+            load_cinfo(min(w + 2, w_last));
+        // Keep the loads ahead of the multiplication: they need the whole MFMA phase to land.
+        __builtin_amdgcn_sched_barrier(0);
 
-        const float* Ab = As + (t & 1) * T::AROWS * T::ASTR;
         afrag_t av[T::KSTEPS];
 #pragma unroll
         for (int s = 0; s < T::KSTEPS; ++s)
-            av[s] = *reinterpret_cast<const afrag_t*>(Ab + aoff[s]);
+            av[s] = *reinterpret_cast<const afrag_t*>(cur + aoff[s]);
 #pragma unroll
         for (int s = 0; s < T::KSTEPS; ++s) {
 #pragma unroll
@@ -248,15 +300,19 @@ spmm_mfma_kernel(const MfmaParams p)
                 acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_get(av[s], b), bv[s], acc[b], 0, 0, 0);
         }
 
-        if (more) {
-            store_a((t + 1) & 1);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int s = 0; s < T::KSTEPS; ++s) {
-                aoff[s] = idx_next[s] * T::ASTR + a_lane;
-                bv[s] = b_next[s];
-            }
+        for (int s = 0; s < T::KSTEPS; ++s) {
+            aoff[s] = idx_next[s] * T::ASTR + a_lane;
+            bv[s] = b_next[s];
         }
+        __builtin_amdgcn_s_waitcnt(kWaitVm0);
         __syncthreads();
+    };
+    for (int t = 0; t < w_count; t += 2) {
+        window(t, As0, As1);
+        if (t + 1 < w_count)
+            window(t + 1, As1, As0);
     }
 
     // ---- epilogue -----------------------------------------------------------------------------
@@ -270,7 +326,11 @@ spmm_mfma_kernel(const MfmaParams p)
 #pragma unroll
         for (int b = 0; b < RM; ++b) {
             const int row = bi + grp * (RM * 32) + r32 * RM + b;
+#ifdef NMSPMM_EXP_NOSTORE
+            if (row < M && acc[b][v] == 12345.f)
+#else
             if (row < M)
+#endif
                 out[(size_t)row * N + col] = acc[b][v];
         }
     }
@@ -294,13 +354,8 @@ static hipError_t launch_cfg(const SpmmArgs& a)
     p.split_k = a.split_k;
     p.tiles_m = (a.M + T::MS - 1) / T::MS;
     p.tiles_n = a.N / T::NS;
-    auto kern = spmm_mfma_kernel<KS, WS, QS, WR, RM, HIGH>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)T::LDS_BYTES);
-    if (e != hipSuccess)
-        return e;
     dim3 grid(p.tiles_m * p.tiles_n, a.split_k, 1);
-    hipLaunchKernelGGL(kern, grid, dim3(T::NT), T::LDS_BYTES, a.stream, p);
+    spmm_mfma_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, dim3(T::NT), (size_t)NMSPMM_LDS_MIN, a.stream>>>(p);
     return hipGetLastError();
 }
 
@@ -310,9 +365,9 @@ template <int KS, int WS, bool HIGH>
 static hipError_t launch_ns(const SpmmArgs& a)
 {
     switch (a.Ns) {
-    case 128: return launch_cfg<KS, WS, 4, 1, 4, HIGH>(a);
-    case 64: return launch_cfg<KS, WS, 2, 2, 2, HIGH>(a);
-    case 32: return launch_cfg<KS, WS, 1, 4, 1, HIGH>(a);
+    case 128: return launch_cfg<KS, WS, 4, NMSPMM_CFG128, HIGH>(a);
+    case 64: return launch_cfg<KS, WS, 2, NMSPMM_CFG64, HIGH>(a);
+    case 32: return launch_cfg<KS, WS, 1, NMSPMM_CFG32, HIGH>(a);
     }
     return hipErrorInvalidValue;
 }
