@@ -208,16 +208,25 @@ spmm_mfma_kernel(const MfmaParams p)
             a_off[s] = lin < T::A_F4 ? (uint32_t)(((size_t)row * M + c4) * sizeof(float)) : kNoLoad;
         }
     }
-    // HIGH: staged row r of window w is A row column_info[w][r]; -1 means "no such row".
+    // HIGH: staged row r of window w is A row column_info[w][r]; -1 means "no such row".  The
+    // list is fetched raw two windows ahead and only turned into load offsets after the
+    // multiplication, so that its latency never sits in front of anything.
+    int ci_raw[T::A_SLOTS];
     auto load_cinfo = [&](int w) {
         const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cinfo + (size_t)w * KS, KS * sizeof(int32_t));
 #pragma unroll
         for (int s = 0; s < T::A_SLOTS; ++s) {
+            const int row = (tid + s * T::NT) / T::A_F4_ROW;
+            ci_raw[s] = __builtin_amdgcn_raw_buffer_load_b32(rc, row * (int)sizeof(int32_t), 0, 0);
+        }
+    };
+    auto cinfo_to_offsets = [&]() {
+#pragma unroll
+        for (int s = 0; s < T::A_SLOTS; ++s) {
             const int lin = tid + s * T::NT;
-            const int row = lin / T::A_F4_ROW;
             const int c4 = (lin % T::A_F4_ROW) * 4;
-            const int src = __builtin_amdgcn_raw_buffer_load_b32(rc, row * (int)sizeof(int32_t), 0, 0);
-            a_off[s] = (src >= 0 && lin < T::A_F4) ? (uint32_t)(((size_t)src * M + c4) * sizeof(float)) : kNoLoad;
+            a_off[s] = (ci_raw[s] >= 0 && lin < T::A_F4)
+                           ? (uint32_t)(((size_t)ci_raw[s] * M + c4) * sizeof(float)) : kNoLoad;
         }
     };
     auto load_a = [&](int w, float* dst) {
@@ -259,12 +268,16 @@ spmm_mfma_kernel(const MfmaParams p)
     // ---- prologue ---------------------------------------------------------------------------
     const int w_last = w_begin + w_count - 1;
     if (w_count > 0) {
-        if (HIGH)
+        if (HIGH) {
             load_cinfo(w_begin);
+            cinfo_to_offsets();
+        }
         load_a(w_begin, As0);
         load_b_idx(w_begin);
-        if (HIGH)
+        if (HIGH) {
             load_cinfo(min(w_begin + 1, w_last));
+            cinfo_to_offsets();
+        }
 #pragma unroll
         for (int s = 0; s < T::KSTEPS; ++s) {
             aoff[s] = idx_next[s] * T::ASTR + a_lane;
@@ -306,6 +319,8 @@ spmm_mfma_kernel(const MfmaParams p)
             aoff[s] = idx_next[s] * T::ASTR + a_lane;
             bv[s] = b_next[s];
         }
+        if (HIGH)
+            cinfo_to_offsets();
         __builtin_amdgcn_s_waitcnt(kWaitVm0);
         __syncthreads();
     };
