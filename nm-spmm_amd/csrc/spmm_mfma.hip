@@ -116,7 +116,7 @@ constexpr int kWaitVm0 = 0x0F70;           // s_waitcnt vmcnt(0), other counters
 // Tuning knobs (compile-time): minimum waves per SIMD the register allocation must allow, the
 // tile-walk band height, and the (waves along M, 32-row blocks per wave) of each tile width.
 #ifndef NMSPMM_OCC
-#define NMSPMM_OCC 1
+#define NMSPMM_OCC 3
 #endif
 #ifndef NMSPMM_LDS_MIN
 #define NMSPMM_LDS_MIN 0  // extra dynamic LDS bytes to claim (caps workgroups per CU)
@@ -185,7 +185,6 @@ spmm_mfma_kernel(const MfmaParams p)
     const int M = p.M, N = p.N;
     const float* const Ablk = p.A + bi;
     const float* const Bvec = p.B + bj + vec * 32;
-    const int32_t* const Dvec = p.D + (size_t)tile_n * p.W * QS + vec;
     const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)tile_n * p.nwin * KS : nullptr;
     // Bytes addressable from the first element of a window's A tile / B vector.  Columns past
     // M in an A row that is not the last one alias the next row (finite garbage that only
@@ -197,66 +196,80 @@ spmm_mfma_kernel(const MfmaParams p)
     // ---- A staging: global -> LDS without passing through registers -------------------------------
     // Slot s of wave `wave` is the 1 KiB chunk number wave + s*NW of the [AROWS][MS] tile: float4
     // number 64*chunk + lane, which is also where an LDS-direct 128-bit load puts lane's data.
+    // HIGH: staged row r of window w is A row column_info[w][r]; -1 means "no such row".  One
+    // wave-wide load brings the whole list (KS = 64 entries, lane l holds entry l) two windows
+    // ahead; readlane hands every lane the entry of the row its load slot covers.  Load offsets
+    // are formed right before use so that nothing per slot stays live across the multiplication.
     constexpr int NW = T::NT / 64;
-    uint32_t a_off[T::A_SLOTS];  // byte offset inside the window (kNoLoad: nothing to load)
-    if (!HIGH) {
-#pragma unroll
-        for (int s = 0; s < T::A_SLOTS; ++s) {
-            const int lin = tid + s * T::NT;
-            const int row = lin / T::A_F4_ROW;
-            const int c4 = (lin % T::A_F4_ROW) * 4;
-            a_off[s] = lin < T::A_F4 ? (uint32_t)(((size_t)row * M + c4) * sizeof(float)) : kNoLoad;
-        }
-    }
-    // HIGH: staged row r of window w is A row column_info[w][r]; -1 means "no such row".  The
-    // list is fetched raw two windows ahead and only turned into load offsets after the
-    // multiplication, so that its latency never sits in front of anything.
-    int ci_raw[T::A_SLOTS];
+    constexpr int RPC = T::A_F4_ROW < 64 ? 64 / T::A_F4_ROW : 1;  // tile rows per 1 KiB chunk
+    int ci_vec = -1;  // HIGH: column_info of the window whose A tile is loaded next
     auto load_cinfo = [&](int w) {
         const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cinfo + (size_t)w * KS, KS * sizeof(int32_t));
-#pragma unroll
-        for (int s = 0; s < T::A_SLOTS; ++s) {
-            const int row = (tid + s * T::NT) / T::A_F4_ROW;
-            ci_raw[s] = __builtin_amdgcn_raw_buffer_load_b32(rc, row * (int)sizeof(int32_t), 0, 0);
-        }
-    };
-    auto cinfo_to_offsets = [&]() {
-#pragma unroll
-        for (int s = 0; s < T::A_SLOTS; ++s) {
-            const int lin = tid + s * T::NT;
-            const int c4 = (lin % T::A_F4_ROW) * 4;
-            a_off[s] = (ci_raw[s] >= 0 && lin < T::A_F4)
-                           ? (uint32_t)(((size_t)ci_raw[s] * M + c4) * sizeof(float)) : kNoLoad;
-        }
+        ci_vec = __builtin_amdgcn_raw_buffer_load_b32(rc, lane * (int)sizeof(int32_t), 0, 0);
     };
     auto load_a = [&](int w, float* dst) {
         const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w * KS * M, a_bytes);
         lds_f32* Ab = (lds_f32*)dst + wave * 256;
 #pragma unroll
         for (int s = 0; s < T::A_SLOTS; ++s) {
-            if (T::A_F4 % T::NT == 0 || s + 1 < T::A_SLOTS || (wave + s * NW) * 64 < T::A_F4)
-                buffer_load_f4_to_lds(ra, Ab + s * NW * 256, a_off[s]);
+            const int chunk = wave + s * NW;
+            const int r0 = chunk * 64 / T::A_F4_ROW;  // first tile row of the chunk (wave-uniform)
+            const int f4 = lane % T::A_F4_ROW + (T::A_F4_ROW > 64 ? (chunk * 64) % T::A_F4_ROW : 0);
+            const bool in_tile = T::A_F4 % T::NT == 0 || s + 1 < T::A_SLOTS || chunk * 64 < T::A_F4;
+            // No branch here: a skipped slot is an out-of-range load (reads nothing, stores zeros).
+            // Control flow inside the loop body makes the register allocator shuttle the
+            // accumulators between VGPRs and AGPRs every iteration.
+            if (in_tile) {
+                int src = r0 + lane / T::A_F4_ROW;
+                if (HIGH) {
+                    src = __builtin_amdgcn_readlane(ci_vec, r0 & 63);
+#pragma unroll
+                    for (int g = 1; g < RPC; ++g) {
+                        const int v = __builtin_amdgcn_readlane(ci_vec, (r0 + g) & 63);
+                        src = (lane / T::A_F4_ROW == g) ? v : src;
+                    }
+                }
+                const uint32_t off = src >= 0 ? (uint32_t)(((size_t)src * M + f4 * 4) * sizeof(float)) : kNoLoad;
+                buffer_load_f4_to_lds(ra, Ab + s * NW * 256, off);
+            }
         }
     };
 
-    // ---- per-wave operands that bypass LDS: B values and indices of compressed rows 2s + h ------
+    // ---- per-wave operands that bypass LDS ---------------------------------------------------------
+    // B values of compressed rows 2s + h come one dword per lane.  The window's index block
+    // ([WS][QS] ints, contiguous) comes as one wave-wide load per 64 entries; readlane then
+    // gives lane (h, j) the index of row 2s + h of this wave's column vector.
+    constexpr int ND = (WS * QS + 63) / 64;
     float b_next[T::KSTEPS];
-    int idx_next[T::KSTEPS];
+    int d_next[ND];
     const uint32_t b_lane = (uint32_t)(((size_t)h * N + j) * sizeof(float));
-    const uint32_t d_lane = (uint32_t)(h * QS * sizeof(int32_t));
+    const uint32_t b_step = (uint32_t)(2 * (size_t)N * sizeof(float));
+    const int32_t* const Dblk = p.D + (size_t)tile_n * p.W * QS;
     auto load_b_idx = [&](int w) {
         const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)w * WS * N, b_bytes);
-        const __amdgpu_buffer_rsrc_t rd = make_rsrc(Dvec + (size_t)w * WS * QS, ((WS - 1) * QS + 1) * sizeof(int32_t));
+        const __amdgpu_buffer_rsrc_t rd = make_rsrc(Dblk + (size_t)w * WS * QS, WS * QS * sizeof(int32_t));
+        uint32_t off = b_lane;
 #pragma unroll
-        for (int s = 0; s < T::KSTEPS; ++s) {
-            b_next[s] = buffer_load_f1(rb, b_lane, (uint32_t)(2 * s * N * sizeof(float)));
-            idx_next[s] = __builtin_amdgcn_raw_buffer_load_b32(rd, d_lane, 2 * s * QS * (int)sizeof(int32_t), 0);
-        }
+        for (int s = 0; s < T::KSTEPS; ++s, off += b_step)
+            b_next[s] = buffer_load_f1(rb, off, 0);
+#pragma unroll
+        for (int q = 0; q < ND; ++q)
+            d_next[q] = __builtin_amdgcn_raw_buffer_load_b32(rd, (lane + 64 * q) * (int)sizeof(int32_t), 0, 0);
     };
 
-    const int a_lane = grp * (RM * 32) + j * RM;  // first of this lane's RM adjacent rows
     int aoff[T::KSTEPS];
     float bv[T::KSTEPS];
+    const int a_lane = grp * (RM * 32) + j * RM;  // first of this lane's RM adjacent rows
+    auto take_b_idx = [&]() {
+#pragma unroll
+        for (int s = 0; s < T::KSTEPS; ++s) {
+            const int e0 = 2 * s * QS, e1 = (2 * s + 1) * QS;  // entries of rows 2s, 2s+1, vector 0
+            const int lo = __builtin_amdgcn_readlane(d_next[e0 / 64], e0 % 64 + vec);
+            const int hi = __builtin_amdgcn_readlane(d_next[e1 / 64], e1 % 64 + vec);
+            aoff[s] = (h ? hi : lo) * T::ASTR + a_lane;
+            bv[s] = b_next[s];
+        }
+    };
 
     floatx16 acc[RM];
 #pragma unroll
@@ -268,21 +281,13 @@ spmm_mfma_kernel(const MfmaParams p)
     // ---- prologue ---------------------------------------------------------------------------
     const int w_last = w_begin + w_count - 1;
     if (w_count > 0) {
-        if (HIGH) {
+        if (HIGH)
             load_cinfo(w_begin);
-            cinfo_to_offsets();
-        }
         load_a(w_begin, As0);
         load_b_idx(w_begin);
-        if (HIGH) {
+        if (HIGH)
             load_cinfo(min(w_begin + 1, w_last));
-            cinfo_to_offsets();
-        }
-#pragma unroll
-        for (int s = 0; s < T::KSTEPS; ++s) {
-            aoff[s] = idx_next[s] * T::ASTR + a_lane;
-            bv[s] = b_next[s];
-        }
+        take_b_idx();
     }
     __builtin_amdgcn_s_waitcnt(kWaitVm0);
     __syncthreads();
@@ -295,10 +300,16 @@ spmm_mfma_kernel(const MfmaParams p)
     auto window = [&](int t, const float* cur, float* nxt) {
         const int w = w_begin + t;
         const int w1 = min(w + 1, w_last);
+#ifndef NMSPMM_EXP_NODMA
         load_a(w1, nxt);
+#endif
+#ifndef NMSPMM_EXP_NOBIDX
         load_b_idx(w1);
+#endif
+#ifndef NMSPMM_EXP_NOCI
         if (HIGH)
             load_cinfo(min(w + 2, w_last));
+#endif
         // Keep the loads ahead of the multiplication: they need the whole MFMA phase to land.
         __builtin_amdgcn_sched_barrier(0);
 
@@ -314,15 +325,11 @@ spmm_mfma_kernel(const MfmaParams p)
         }
 
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s = 0; s < T::KSTEPS; ++s) {
-            aoff[s] = idx_next[s] * T::ASTR + a_lane;
-            bv[s] = b_next[s];
-        }
-        if (HIGH)
-            cinfo_to_offsets();
+        take_b_idx();
         __builtin_amdgcn_s_waitcnt(kWaitVm0);
+#ifndef NMSPMM_EXP_NOBAR
         __syncthreads();
+#endif
     };
     for (int t = 0; t < w_count; t += 2) {
         window(t, As0, As1);
