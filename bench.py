@@ -112,12 +112,22 @@ def cpu_baseline(case, rows):
     orc = Oracle()
     A_sub = np.ascontiguousarray(d["A_km"][:, :rows]).reshape(-1)
     B, D = d["B_cm"].reshape(-1), d["D_cm"].reshape(-1)
-    t0 = time.perf_counter()
-    if ref is not None:
-        C = ref.gemm_cpu(A_sub, B, D, rows, N, K, case.W)
-    else:
-        C = orc.gemm_cpu(A_sub, B, D, rows, N, case.W)
-    dt = time.perf_counter() - t0
+    # The reference prints its thread count with printf; keep stdout for the one JSON line.
+    sys.stdout.flush()
+    saved = os.dup(1)
+    os.dup2(2, 1)
+    try:
+        t0 = time.perf_counter()
+        if ref is not None:
+            C = ref.gemm_cpu(A_sub, B, D, rows, N, K, case.W)
+        else:
+            C = orc.gemm_cpu(A_sub, B, D, rows, N, case.W)
+        dt = time.perf_counter() - t0
+        import ctypes
+        ctypes.CDLL(None).fflush(None)
+    finally:
+        os.dup2(saved, 1)
+        os.close(saved)
     return C.reshape(rows, N), {
         "value": 2.0 * rows * N * case.W / dt / 1e12, "unit": "TFLOP/s (useful)", "cores": orc.threads(), "kind": kind,
         "sample": "rows [0,%d) of the M=%d 2:4 workload (rows are independent), %.1f s wall" % (rows, M, dt),

@@ -22,6 +22,14 @@
 //    C and share A / B panels in that XCD's L2.
 #include "internal.h"
 
+#ifdef NMSPMM_TRACE
+__device__ unsigned long long g_trace[4 * 64 * 8];  // [wave][iteration][stamp]
+extern "C" int nmspmm_debug_trace(void* dst) { return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_trace), sizeof(g_trace)); }
+#define TRACE_STAMP(k) do { if (blockIdx.x == 264 && lane == 0 && t < 64) g_trace[(wave * 64 + t) * 8 + (k)] = __builtin_readcyclecounter(); } while (0)
+#else
+#define TRACE_STAMP(k) do { } while (0)
+#endif
+
 namespace nmspmm {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -41,11 +49,15 @@ struct MfmaParams {
     int tiles_m, tiles_n;
 };
 
+struct float8 { float4 lo, hi; };
 template <int RM> struct AFrag;
+template <> struct AFrag<8> { typedef float8 type; };
 template <> struct AFrag<4> { typedef float4 type; };
 template <> struct AFrag<2> { typedef float2 type; };
 template <> struct AFrag<1> { typedef float type; };
 
+__device__ inline float frag_get(const float4& v, int i);
+__device__ inline float frag_get(const float8& v, int i) { return i < 4 ? frag_get(v.lo, i) : frag_get(v.hi, i - 4); }
 __device__ inline float frag_get(const float4& v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
 __device__ inline float frag_get(const float2& v, int i) { return i == 0 ? v.x : v.y; }
 __device__ inline float frag_get(const float& v, int) { return v; }
@@ -86,6 +98,7 @@ NMSPMM_LDS_PAIR(2048)
 NMSPMM_LDS_PAIR(4096)
 NMSPMM_LDS_PAIR(8192)
 NMSPMM_LDS_PAIR(16384)
+NMSPMM_LDS_PAIR(32768)
 
 // Buffer descriptors give branch-free guarded loads: an offset at or beyond num_records reads 0
 // without touching memory, so "this slot has nothing to load" is just an out-of-range offset.
@@ -120,6 +133,12 @@ constexpr int kWaitVm0 = 0x0F70;           // s_waitcnt vmcnt(0), other counters
 #endif
 #ifndef NMSPMM_LDS_MIN
 #define NMSPMM_LDS_MIN 0  // extra dynamic LDS bytes to claim (caps workgroups per CU)
+#endif
+#ifndef NMSPMM_SKIP_ROWS
+#define NMSPMM_SKIP_ROWS 0  // HIGH: branch around load slots behind the end of the row list
+#endif
+#ifndef NMSPMM_INTERLEAVE
+#define NMSPMM_INTERLEAVE 0  // k-steps over which the next window's loads are spread (0: all up front)
 #endif
 #ifndef NMSPMM_GROUP
 #define NMSPMM_GROUP 8
@@ -210,16 +229,20 @@ spmm_mfma_kernel(const MfmaParams p)
     auto load_a = [&](int w, float* dst) {
         const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w * KS * M, a_bytes);
         lds_f32* Ab = (lds_f32*)dst + wave * 256;
+#if NMSPMM_SKIP_ROWS
+        const int a_rows = HIGH ? __builtin_popcountll(__ballot(ci_vec >= 0)) : T::AROWS;
+#endif
 #pragma unroll
         for (int s = 0; s < T::A_SLOTS; ++s) {
             const int chunk = wave + s * NW;
             const int r0 = chunk * 64 / T::A_F4_ROW;  // first tile row of the chunk (wave-uniform)
             const int f4 = lane % T::A_F4_ROW + (T::A_F4_ROW > 64 ? (chunk * 64) % T::A_F4_ROW : 0);
             const bool in_tile = T::A_F4 % T::NT == 0 || s + 1 < T::A_SLOTS || chunk * 64 < T::A_F4;
-            // No branch here: a skipped slot is an out-of-range load (reads nothing, stores zeros).
-            // Control flow inside the loop body makes the register allocator shuttle the
-            // accumulators between VGPRs and AGPRs every iteration.
+#if NMSPMM_SKIP_ROWS
+            if (in_tile && (!HIGH || r0 < a_rows)) {
+#else
             if (in_tile) {
+#endif
                 int src = r0 + lane / T::A_F4_ROW;
                 if (HIGH) {
                     src = __builtin_amdgcn_readlane(ci_vec, r0 & 63);
@@ -300,6 +323,7 @@ spmm_mfma_kernel(const MfmaParams p)
     auto window = [&](int t, const float* cur, float* nxt) {
         const int w = w_begin + t;
         const int w1 = min(w + 1, w_last);
+        TRACE_STAMP(0);
 #ifndef NMSPMM_EXP_NODMA
         load_a(w1, nxt);
 #endif
@@ -310,8 +334,12 @@ spmm_mfma_kernel(const MfmaParams p)
         if (HIGH)
             load_cinfo(min(w + 2, w_last));
 #endif
+#if NMSPMM_INTERLEAVE == 0
         // Keep the loads ahead of the multiplication: they need the whole MFMA phase to land.
         __builtin_amdgcn_sched_barrier(0);
+        TRACE_STAMP(1);
+        __builtin_amdgcn_sched_barrier(0);
+#endif
 
         afrag_t av[T::KSTEPS];
 #pragma unroll
@@ -323,13 +351,37 @@ spmm_mfma_kernel(const MfmaParams p)
             for (int b = 0; b < RM; ++b)
                 acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_get(av[s], b), bv[s], acc[b], 0, 0, 0);
         }
+#if NMSPMM_INTERLEAVE
+        // Issue order inside the block: two fragment reads, then per k-step its RM MFMAs, one
+        // more fragment read, and (during the first NMSPMM_INTERLEAVE k-steps) a share of the next
+        // window's global loads, so that a stalled memory issue overlaps running MFMAs.
+        {
+            constexpr int VMEM = T::A_SLOTS + T::KSTEPS + ND + (HIGH ? 1 : 0);
+            constexpr int SPREAD = NMSPMM_INTERLEAVE < T::KSTEPS ? NMSPMM_INTERLEAVE : T::KSTEPS;
+            constexpr int VPS = (VMEM + SPREAD - 1) / SPREAD;
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+            for (int s = 0; s < T::KSTEPS; ++s) {
+                __builtin_amdgcn_sched_group_barrier(0x008, RM, 0);
+                if (s < SPREAD)
+                    __builtin_amdgcn_sched_group_barrier(0x020, VPS, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+        }
+#endif
 
         __builtin_amdgcn_sched_barrier(0);
+        TRACE_STAMP(2);
+        __builtin_amdgcn_sched_barrier(0);
         take_b_idx();
+        __builtin_amdgcn_sched_barrier(0);
+        TRACE_STAMP(3);
         __builtin_amdgcn_s_waitcnt(kWaitVm0);
+        TRACE_STAMP(4);
 #ifndef NMSPMM_EXP_NOBAR
         __syncthreads();
 #endif
+        TRACE_STAMP(5);
     };
     for (int t = 0; t < w_count; t += 2) {
         window(t, As0, As1);
@@ -381,13 +433,20 @@ static hipError_t launch_cfg(const SpmmArgs& a)
     return hipGetLastError();
 }
 
-// Four waves and 128 rows per workgroup tile for every column-block width: 1 x 4, 2 x 2 or
-// 4 x 1 waves (rows x column vectors), each wave 128, 64 or 32 rows tall.
+// Row extent of the workgroup tile.  Every tile has four waves: 1 x 4, 2 x 2 or 4 x 1 (rows x
+// column vectors).  For 128-wide column blocks a wave is 128 rows tall, or 256 rows when the
+// matrix is large enough that 256-row tiles still give every CU at least two workgroups: the
+// taller wave amortises its per-window loads and barrier over twice the MFMAs.
+constexpr int kCus = 256;
+
 template <int KS, int WS, bool HIGH>
 static hipError_t launch_ns(const SpmmArgs& a)
 {
     switch (a.Ns) {
-    case 128: return launch_cfg<KS, WS, 4, NMSPMM_CFG128, HIGH>(a);
+    case 128:
+        if ((long long)((a.M + 255) / 256) * (a.N / 128) * a.split_k >= 2 * kCus)
+            return launch_cfg<KS, WS, 4, 1, 8, HIGH>(a);
+        return launch_cfg<KS, WS, 4, NMSPMM_CFG128, HIGH>(a);
     case 64: return launch_cfg<KS, WS, 2, NMSPMM_CFG64, HIGH>(a);
     case 32: return launch_cfg<KS, WS, 1, NMSPMM_CFG32, HIGH>(a);
     }
