@@ -128,7 +128,7 @@ int nmspmm_gemm_high_sparsity(int tile, const float* A, const float* B, const in
 int nmspmm_release(void);
 
 /* Name of the kernel family the last successful nmspmm_spmm call on this thread dispatched to
- * ("mfma", "simt"), for tests and profiles.  Never NULL. */
+ * ("mfma", "skinny", "simt"), for tests and profiles.  Never NULL. */
 const char* nmspmm_last_kernel(void);
 
 #ifdef __cplusplus

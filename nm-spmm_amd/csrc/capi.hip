@@ -311,6 +311,12 @@ int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t*
     a.stream = (hipStream_t)stream;
 
     hipError_t e;
+    if (skinny_supported(a)) {
+        // one launch, reduction inside the workgroup: split_k and the workspace are not needed
+        e = launch_skinny(a);
+        g_last_kernel = "skinny";
+        return e == hipSuccess ? NMSPMM_OK : NMSPMM_ERR_HIP;
+    }
     if (mfma_supported(a)) {
         e = launch_mfma(a);
         g_last_kernel = "mfma";

@@ -37,6 +37,10 @@ __host__ __device__ inline void split_windows(int nwin, int split_k, int z, int*
 bool mfma_supported(const SpmmArgs& a);
 hipError_t launch_mfma(const SpmmArgs& a);
 
+// Decode-sized path (spmm_skinny.hip): M <= 32, the reference geometries, no workspace needed.
+bool skinny_supported(const SpmmArgs& a);
+hipError_t launch_skinny(const SpmmArgs& a);
+
 // Generic SIMT path (spmm_simt.hip): any window/kept, vec_len in {4, 8, 16, 32}, any M.
 bool simt_supported(const SpmmArgs& a);
 hipError_t launch_simt(const SpmmArgs& a);
