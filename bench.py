@@ -141,6 +141,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the CPU baseline sample (0 = skip)")
     ap.add_argument("--headline-only", action="store_true", help="time only the 2:4 kernel (for profiling runs)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy 5 times (known traffic, to scale rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this library is a single-GPU kernel library; run with --gpus 1", file=sys.stderr)
@@ -181,6 +184,14 @@ def main():
         sweep["%d:%d" % (n, m)] = entry
         if idx > 0:
             del case
+
+    if args.calibrate_copy:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     case, ms, wall_ms = head
     achieved = case.useful_flops() / (ms * 1e-3) / 1e12

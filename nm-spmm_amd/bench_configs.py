@@ -1,0 +1,145 @@
+#!/usr/bin/env python3
+"""Measurement of the baseline's other workloads (bench.py at the repository root covers the
+square sweep): LLM-layer shapes, decode-sized M, and the fine-grained / short-vector patterns.
+Prints one markdown table row per case.
+
+    python nm-spmm_amd/bench_configs.py [llm] [decode] [fine]
+
+useful TFLOP/s = 2*M*Ncols*W / t; GB/s = algorithmic bytes
+4*(M*K + W*Ncols + W*Ncols/L + M*Ncols) (+ column_info) / t.
+"""
+import importlib
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+
+import torch  # noqa: E402
+
+pkg = importlib.import_module("nm-spmm_amd")
+datagen = importlib.import_module("nm-spmm_amd.datagen")
+
+GEOMETRY = {(2, 4): (32, 16), (3, 8): (32, 12), (2, 8): (64, 16), (1, 8): (64, 8),
+            (16, 32): (32, 16), (12, 32): (32, 12), (8, 32): (64, 16), (4, 32): (64, 8)}
+
+
+def timed(fn, steps=50, warmup=10):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    best = 1e9
+    for _ in range(3):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        best = min(best, e0.elapsed_time(e1) / steps)
+    return best
+
+
+class Operands:
+    def __init__(self, M, N, K, n, m, vec_len=32, Ns=128, dist="uniform", b_scale=1.0, seed=0):
+        d = datagen.init_data(M, N, K, n, m, vec_len=vec_len, seed=seed, dist=dist, b_scale=b_scale)
+        self.M, self.N, self.K, self.W, self.Q, self.vl, self.Ns = M, N, K, d["W"], d["Q"], vec_len, Ns
+        self.A = torch.from_numpy(d["A_km"]).cuda()
+        self.B = torch.from_numpy(d["BT"]).cuda()
+        self.C = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        DT0 = torch.from_numpy(d["DT"].reshape(-1).copy()).cuda()
+        DT, self.D = torch.empty_like(DT0), torch.empty_like(DT0)
+        if vec_len == 32:
+            self.window, self.kept = GEOMETRY[(n, m)]
+        else:
+            self.window, self.kept = m, n
+        self.cinfo = None
+        if self.window == 64:
+            self.cinfo = torch.empty(pkg.column_info_ints(self.W, self.kept, self.window, N, Ns), dtype=torch.int32,
+                                     device="cuda")
+
+        def preprocess():
+            DT.copy_(DT0)
+            pn, pm = n, m
+            while pm < self.window:
+                pn, pm = pkg.trans_index_device(DT, self.W, N, self.Q, pn, pm)
+            if self.cinfo is None:
+                pkg.preprocess_low_device(DT, self.D, self.W, self.Q, Ns, vec_len)
+            else:
+                pkg.preprocess_high_device(self.cinfo, pm, pn, DT, self.D, self.W, self.Q, N, Ns, vec_len)
+
+        self.preprocess_ms = timed(preprocess, 5, 1)
+
+    def launch(self, split_k=1, ws=None):
+        pkg.spmm(self.A, self.B, self.D, self.cinfo, self.C, self.M, self.N, self.K, self.W, self.window, self.kept,
+                 self.vl, self.Ns, split_k, ws)
+
+    def flops(self):
+        return 2.0 * self.M * self.N * self.W
+
+    def bytes(self):
+        b = 4.0 * (self.M * self.K + self.W * self.N + self.W * self.N / self.vl + self.M * self.N)
+        if self.cinfo is not None:
+            b += 4.0 * self.cinfo.numel()
+        return b
+
+
+def dense_ms(M, N, K):
+    a = torch.randn((M, K), dtype=torch.float32, device="cuda")
+    b = torch.randn((K, N), dtype=torch.float32, device="cuda")
+    c = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    return timed(lambda: torch.mm(a, b, out=c))
+
+
+def llm():
+    print("| M | K x Ncols | pattern | kernel | ms | useful TFLOP/s | dense fp32 GEMM ms | speedup | of ideal 4x | preprocess ms |")
+    print("|---|---|---|---|---|---|---|---|---|---|")
+    for (K, N) in ((4096, 4096), (4096, 11008), (11008, 4096)):
+        for M in (512, 2048, 8192):
+            op = Operands(M, N, K, 2, 8, dist="normal", b_scale=0.02, seed=M + K)
+            best = (1e9, 1)
+            for split in (1, 2, 4):
+                if split > 1 and (M // 128) * (N // 128) * split > 4096:
+                    continue
+                ws = None if split == 1 else torch.empty(pkg.workspace_bytes(M, N, split) // 4, dtype=torch.float32,
+                                                         device="cuda")
+                best = min(best, (timed(lambda: op.launch(split, ws)), split))
+            ms, split = best
+            dms = dense_ms(M, N, K)
+            print("| %d | %dx%d | 2:8 | %s sk%d | %.4f | %.1f | %.4f | %.2f | %.2f | %.3f |" % (
+                M, K, N, pkg.last_kernel(), split, ms, op.flops() / ms / 1e9, dms, dms / ms, dms / ms / 4, op.preprocess_ms),
+                flush=True)
+            del op
+
+
+def decode():
+    print("| M | K x Ncols | pattern | kernel | us | GB/s (algorithmic) | of 8 TB/s |")
+    print("|---|---|---|---|---|---|---|")
+    for (K, N) in ((8192, 8192), (4096, 14336)):
+        for (n, m) in ((1, 8), (2, 8)):
+            for M in (1, 8, 16, 32):
+                op = Operands(M, N, K, n, m, dist="normal", b_scale=0.02, seed=M)
+                ms = timed(lambda: op.launch())
+                print("| %d | %dx%d | %d:%d | %s | %.1f | %.0f | %.3f |" % (
+                    M, K, N, n, m, pkg.last_kernel(), ms * 1e3, op.bytes() / ms / 1e6, op.bytes() / ms / 1e6 / 8000), flush=True)
+                del op
+
+
+def fine():
+    print("| pattern | vector length | kernel | ms | useful TFLOP/s | of fp32 MFMA peak | preprocess ms | index bytes |")
+    print("|---|---|---|---|---|---|---|---|")
+    for (n, m, vl) in ((4, 32, 32), (8, 32, 32), (16, 32, 32), (2, 4, 4)):
+        op = Operands(4096, 4096, 4096, n, m, vec_len=vl, seed=n)
+        ms = timed(lambda: op.launch(), 20 if vl == 32 else 3, 2)
+        print("| %d:%d | %d | %s | %.4f | %.1f | %.3f | %.3f | %d |" % (
+            n, m, vl, pkg.last_kernel(), ms, op.flops() / ms / 1e9, op.flops() / ms / 1e9 / 157.3, op.preprocess_ms,
+            op.D.numel() * 4), flush=True)
+        del op
+
+
+if __name__ == "__main__":
+    which = sys.argv[1:] or ["llm", "decode", "fine"]
+    pkg.lib()
+    for name in which:
+        print("\n### %s" % name)
+        {"llm": llm, "decode": decode, "fine": fine}[name]()

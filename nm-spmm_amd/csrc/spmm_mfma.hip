@@ -8,8 +8,9 @@
 //    lane = (row % 32, k half): lanes 0-31 take compressed row 2s, lanes 32-63 row 2s+1, and each
 //    half reads the LDS row of A that *its* index selects.  The gather is therefore just a
 //    per-lane LDS row offset; no data is moved to perform it.
-//  * The wave's RM row blocks interleave rows (block b holds rows 4*r + b), so one 128-bit LDS
-//    read yields the A operands of all RM blocks and the B operand is reused RM times.
+//  * The wave's RM row blocks interleave rows (block b holds rows 4*r + b, a 256-row wave two
+//    such groups), so one 128-bit LDS read yields the A operands of four blocks and the B
+//    operand is reused RM times.
 //  * The A tile (window rows x Ms, k-major as in global memory) is shared by the tile's column
 //    vectors, so it is staged global -> registers -> LDS with 128-bit accesses, double
 //    buffered: the loads of window t+1 are in flight while window t is multiplied, one barrier
@@ -56,6 +57,14 @@ template <> struct AFrag<4> { typedef float4 type; };
 template <> struct AFrag<2> { typedef float2 type; };
 template <> struct AFrag<1> { typedef float type; };
 
+template <typename F> __device__ inline F load_frag(const float* p) { return *reinterpret_cast<const F*>(p); }
+template <> __device__ inline float8 load_frag<float8>(const float* p)
+{
+    float8 f;
+    f.lo = *reinterpret_cast<const float4*>(p);
+    f.hi = *reinterpret_cast<const float4*>(p + 128);
+    return f;
+}
 __device__ inline float frag_get(const float4& v, int i);
 __device__ inline float frag_get(const float8& v, int i) { return i < 4 ? frag_get(v.lo, i) : frag_get(v.hi, i - 4); }
 __device__ inline float frag_get(const float4& v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
@@ -282,7 +291,10 @@ spmm_mfma_kernel(const MfmaParams p)
 
     int aoff[T::KSTEPS];
     float bv[T::KSTEPS];
-    const int a_lane = grp * (RM * 32) + j * RM;  // first of this lane's RM adjacent rows
+    // A lane owns runs of up to four adjacent rows, so that the 64 lanes of one 128-bit read cover
+    // contiguous LDS; a 256-row wave tile (RM = 8) is two such runs 128 rows apart.
+    constexpr int RUN = RM < 4 ? RM : 4;
+    const int a_lane = grp * (RM * 32) + j * RUN;
     auto take_b_idx = [&]() {
 #pragma unroll
         for (int s = 0; s < T::KSTEPS; ++s) {
@@ -344,7 +356,7 @@ spmm_mfma_kernel(const MfmaParams p)
         afrag_t av[T::KSTEPS];
 #pragma unroll
         for (int s = 0; s < T::KSTEPS; ++s)
-            av[s] = *reinterpret_cast<const afrag_t*>(cur + aoff[s]);
+            av[s] = load_frag<afrag_t>(cur + aoff[s]);
 #pragma unroll
         for (int s = 0; s < T::KSTEPS; ++s) {
 #pragma unroll
@@ -391,7 +403,7 @@ spmm_mfma_kernel(const MfmaParams p)
 
     // ---- epilogue -----------------------------------------------------------------------------
     // MFMA result register v of lane (h, j) is row 8*(v/4) + 4*h + v%4, column j of the 32x32
-    // block; block b holds tile rows RM*row + b of this wave's row group.
+    // block; block b holds tile rows 128*(b/4) + RUN*row + b%4 of this wave's row group.
     float* out = p.out + (size_t)blockIdx.y * p.slice_elems;
     const int col = bj + vec * 32 + j;
 #pragma unroll
@@ -399,7 +411,7 @@ spmm_mfma_kernel(const MfmaParams p)
         const int r32 = 8 * (v / 4) + 4 * h + (v % 4);
 #pragma unroll
         for (int b = 0; b < RM; ++b) {
-            const int row = bi + grp * (RM * 32) + r32 * RM + b;
+            const int row = bi + grp * (RM * 32) + (b / 4) * 128 + r32 * RUN + (b % 4);
 #ifdef NMSPMM_EXP_NOSTORE
             if (row < M && acc[b][v] == 12345.f)
 #else
