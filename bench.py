@@ -213,7 +213,11 @@ def main():
         "config": {"workload": "square sweep M=Ncols=K=4096 fp32, uniform(-1,1), seeded n:m patterns per 32-column "
                                "vector; value at 2:4, others under sweep", "tile": "Ns=128", "split_k": 1},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
+                     # bytes behind L2 per launch: rocprofv3 FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the
+                     # factors coming from a plain 256 MiB copy in the same runs
+                     # (profiles/spmm_mfma_kernel_4096cubed_2of4.md)
+                     "traffic": 652.4e6, "traffic_unit": "bytes per launch", "algorithmic_bytes": 168.8e6,
                      "kernel": "spmm_mfma_kernel<32,16,4,...>", "flops_per_launch": case.useful_flops(),
                      "launch_ms_events": round(ms, 5), "launch_ms_wall": round(wall_ms, 5)},
         "cpu_baseline": cpu,
