@@ -1,0 +1,173 @@
+// Self-checking driver for the C++ drop-in API (include/NM-SpMM.h), in the manner of the
+// reference's tests/test_nmspmm.cu: same positional arguments, same call sequence (host-side
+// preprocessing in place, copy, launch by tile name), one run per tile whose divisibility holds.
+// Differences: operands are seeded and signed, the CPU check is the checker library
+// (oracle/libnm_oracle.so), the comparison is the scaled max error bound 1e-4, and the exit code
+// reports failure.
+//
+//   test_nmspmm_dropin M N K [pruning_M sparsity [SPLIT_K]]
+#include "NM-SpMM.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+extern "C" void nm_oracle_gemm_cpu(const float* A, const float* B, const int32_t* D, float* C, int M, int N, int W,
+                                   int vec_len, int row_begin, int row_end);
+
+typedef void (*LowFn)(float*, float*, int*, float*, int, int, int, int, float, int);
+typedef void (*HighFn)(float*, float*, int*, int*, float*, int, int, int, int, float, int);
+
+static uint64_t g_state = 0x9E3779B97F4A7C15ull;
+static uint32_t next_u32()
+{
+    g_state = g_state * 6364136223846793005ull + 1442695040888963407ull;
+    return (uint32_t)(g_state >> 33);
+}
+static float next_unit() { return (float)(next_u32() & 0xFFFFFF) / 8388608.0f - 1.0f; }  // [-1, 1)
+
+#define HIP_OK(x)                                                          \
+    do {                                                                   \
+        hipError_t e_ = (x);                                               \
+        if (e_ != hipSuccess) {                                            \
+            std::printf("%s failed: %s\n", #x, hipGetErrorString(e_));     \
+            return false;                                                  \
+        }                                                                  \
+    } while (0)
+
+static bool run_tile(const char* name, LowFn low, HighFn high, int Ns, int M, int N, int K, int pruning_M,
+                     float sparsity, int split_k)
+{
+    const bool is_high = std::fabs(sparsity - 0.75f) < 1e-6f || std::fabs(sparsity - 0.875f) < 1e-6f;
+    const int W = (int)(K * (1.0f - sparsity));
+    const int Q = N / VEC_LEN;
+    int pruning_N = (int)(pruning_M * (1.0f - sparsity));
+    const int nwin = K / pruning_M;
+    std::printf("\n** %s: Ns = %d\n", name, Ns);
+
+    std::vector<float> A((size_t)M * K), B((size_t)W * N), BT((size_t)W * N), Cref((size_t)M * N, 0.0f), Cgpu((size_t)M * N);
+    std::vector<int> D((size_t)W * Q), DT((size_t)W * Q);
+    for (float& x : A) x = next_unit();
+    for (int k = 0; k < W; ++k)
+        for (int j = 0; j < N; ++j)
+            BT[(size_t)k * N + j] = B[(size_t)k + (size_t)j * W] = next_unit();
+    std::vector<int> perm(pruning_M);
+    for (int a = 0; a < Q; ++a)
+        for (int w = 0; w < nwin; ++w) {
+            for (int x = 0; x < pruning_M; ++x) perm[x] = x;
+            for (int x = 0; x < pruning_N; ++x) std::swap(perm[x], perm[x + next_u32() % (pruning_M - x)]);
+            std::sort(perm.begin(), perm.begin() + pruning_N);
+            for (int u = 0; u < pruning_N; ++u) {
+                const size_t k = (size_t)w * pruning_N + u;
+                D[k + (size_t)a * W] = perm[u] + w * pruning_M;  // column-major, global K index
+                DT[k * Q + a] = perm[u];                         // row-major, window-local
+            }
+        }
+
+    const size_t ci_ints = (size_t)((W / pruning_N) * (N / Ns) + 1) * pruning_M;  // the reference's sizing rule
+    std::vector<int> column_info(ci_ints, -7);
+    int pM = pruning_M, pN = pruning_N;
+    if (!is_high) {
+        PreProcessing_low_sparsity(DT.data(), W, Q, Ns);
+    } else {
+        transIndex(DT.data(), W, N, Q, pN, pM);
+        PreProcessing_high_sparsity(column_info.data(), pM, pN, DT.data(), W, Q, N, Ns);
+    }
+
+    float *dA, *dB, *dC;
+    int *dD, *dci;
+    HIP_OK(hipMalloc(&dA, A.size() * 4));
+    HIP_OK(hipMalloc(&dB, BT.size() * 4));
+    HIP_OK(hipMalloc(&dC, Cgpu.size() * 4));
+    HIP_OK(hipMalloc(&dD, DT.size() * 4));
+    HIP_OK(hipMalloc(&dci, ci_ints * 4));
+    HIP_OK(hipMemcpy(dA, A.data(), A.size() * 4, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dB, BT.data(), BT.size() * 4, hipMemcpyHostToDevice));
+    HIP_OK(hipMemset(dC, 0, Cgpu.size() * 4));
+    HIP_OK(hipMemcpy(dD, DT.data(), DT.size() * 4, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dci, column_info.data(), ci_ints * 4, hipMemcpyHostToDevice));
+
+    nm_oracle_gemm_cpu(A.data(), B.data(), D.data(), Cref.data(), M, N, W, VEC_LEN, 0, M);
+
+    if (!is_high)
+        low(dA, dB, dD, dC, M, N, K, W, sparsity, split_k);
+    else
+        high(dA, dB, dD, dci, dC, M, N, K, W, sparsity, split_k);
+    HIP_OK(hipDeviceSynchronize());
+    HIP_OK(hipMemcpy(Cgpu.data(), dC, Cgpu.size() * 4, hipMemcpyDeviceToHost));
+
+    double sq = 0.0;
+    for (float x : Cref) sq += (double)x * x;
+    const double rms = std::sqrt(sq / Cref.size());
+    double worst = 0.0;
+    for (size_t i = 0; i < Cref.size(); ++i) {
+        const double err = std::fabs((double)Cgpu[i] - Cref[i]) / std::max(std::fabs((double)Cref[i]), rms);
+        if (!(err <= worst)) worst = err;  // also catches NaN
+    }
+    const bool ok = worst <= 1e-4;
+    std::printf(ok ? "The result is right! (scaled max error %.3g)\n" : "The result is wrong !!!!!!!!!! (scaled max error %.3g)\n", worst);
+
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0));
+    HIP_OK(hipEventCreate(&e1));
+    const int iters = 20;
+    HIP_OK(hipEventRecord(e0));
+    for (int i = 0; i < iters; ++i) {
+        if (!is_high)
+            low(dA, dB, dD, dC, M, N, K, W, sparsity, split_k);
+        else
+            high(dA, dB, dD, dci, dC, M, N, K, W, sparsity, split_k);
+    }
+    HIP_OK(hipEventRecord(e1));
+    HIP_OK(hipEventSynchronize(e1));
+    float ms = 0.0f;
+    HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+    ms /= iters;
+    std::printf("Time elapsed: %f ms, %f TFLOPS (dense-equivalent), %f useful TFLOPS\n", ms,
+                2.0 * M * N * K / 1e12 / (ms / 1e3), 2.0 * M * N * W / 1e12 / (ms / 1e3));
+    (void)hipFree(dA);
+    (void)hipFree(dB);
+    (void)hipFree(dC);
+    (void)hipFree(dD);
+    (void)hipFree(dci);
+    return ok;
+}
+
+int main(int argc, char** argv)
+{
+    int M = 512, N = 512, K = 512, pruning_M = 32, split_k = 1;
+    float sparsity = 0.5f;
+    if (argc != 1 && argc != 4 && argc != 6 && argc != 7) {
+        std::printf("Usage: %s M N K [pruning_M sparsity [SPLIT_K]]\n", argv[0]);
+        return -1;
+    }
+    if (argc >= 4) { M = std::atoi(argv[1]); N = std::atoi(argv[2]); K = std::atoi(argv[3]); }
+    if (argc >= 6) { pruning_M = std::atoi(argv[4]); sparsity = (float)std::atof(argv[5]); }
+    if (argc >= 7) split_k = std::atoi(argv[6]);
+    std::printf("M = %d, N = %d, K = %d, pruning_M = %d, sparsity = %f, SPLIT_K = %d\n", M, N, K, pruning_M, sparsity, split_k);
+    const float allowed[] = {0.0f, 0.5f, 0.625f, 0.75f, 0.875f};
+    bool known = false;
+    for (float s : allowed) known = known || std::fabs(sparsity - s) < 1e-6f;
+    if (!known) { std::printf("sparsity not in {0, 0.5, 0.625, 0.75, 0.875}!!!\n"); return -2; }
+    if (K % pruning_M != 0) { std::printf("K is not an integer multiple of pruning_M!!!\n"); return -3; }
+
+    int failures = 0, runs = 0;
+    struct Tile { const char* name; LowFn low; HighFn high; int Ns; } tiles[] = {
+        {"small", &nmGEMM_small_matrices_low_sparsity, &nmGEMM_small_matrices_high_sparsity, 32},
+        {"medium", &nmGEMM_medium_matrices_low_sparsity, &nmGEMM_medium_matrices_high_sparsity, 64},
+        {"large", &nmGEMM_large_matrices_low_sparsity, &nmGEMM_large_matrices_high_sparsity, 64},
+        {"huge", &nmGEMM_huge_matrices_low_sparsity, &nmGEMM_huge_matrices_high_sparsity, 128},
+    };
+    for (const Tile& t : tiles) {
+        if (N % t.Ns != 0) continue;
+        ++runs;
+        if (!run_tile(t.name, t.low, t.high, t.Ns, M, N, K, pruning_M, sparsity, split_k)) ++failures;
+    }
+    std::printf("\n%d tile runs, %d failures\n", runs, failures);
+    return failures == 0 && runs > 0 ? 0 : 1;
+}
