@@ -23,14 +23,6 @@
 //    C and share A / B panels in that XCD's L2.
 #include "internal.h"
 
-#ifdef NMSPMM_TRACE
-__device__ unsigned long long g_trace[4 * 64 * 8];  // [wave][iteration][stamp]
-extern "C" int nmspmm_debug_trace(void* dst) { return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_trace), sizeof(g_trace)); }
-#define TRACE_STAMP(k) do { if (blockIdx.x == 264 && lane == 0 && t < 64) g_trace[(wave * 64 + t) * 8 + (k)] = __builtin_readcyclecounter(); } while (0)
-#else
-#define TRACE_STAMP(k) do { } while (0)
-#endif
-
 namespace nmspmm {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -89,25 +81,27 @@ struct TileCfg {
     static_assert(WS % 2 == 0, "two compressed rows per MFMA");
 };
 
-// The two halves of the double-buffered A tile are separate LDS objects (not one array indexed
-// by t & 1): the compiler can then prove that the fragment reads of one buffer do not alias the
-// asynchronous global->LDS writes into the other and does not serialise them with a vmcnt(0)
-// wait.  They live at namespace scope, one pair per tile size in floats; a kernel is charged
-// only for the pair it references.
-#define NMSPMM_LDS_PAIR(FLOATS)                                          \
-    __shared__ __align__(16) float g_lds_a0_##FLOATS[FLOATS];           \
-    __shared__ __align__(16) float g_lds_a1_##FLOATS[FLOATS];           \
-    template <> struct LdsPair<FLOATS> {                                 \
-        __device__ static float* first() { return g_lds_a0_##FLOATS; }  \
-        __device__ static float* second() { return g_lds_a1_##FLOATS; } \
+// The buffers of the multi-buffered A tile are separate LDS objects (not one array indexed by
+// t % NBUF): the compiler can then prove that the fragment reads of one buffer do not alias the
+// asynchronous global->LDS writes into another and does not serialise them with a vmcnt(0)
+// wait.  They live at namespace scope, one set per tile size in floats; a kernel is charged
+// only for the buffers it references.
+#define NMSPMM_LDS_SET(FLOATS)                                                  \
+    __shared__ __align__(16) float g_lds_a0_##FLOATS[FLOATS];                  \
+    __shared__ __align__(16) float g_lds_a1_##FLOATS[FLOATS];                  \
+    __shared__ __align__(16) float g_lds_a2_##FLOATS[FLOATS];                  \
+    template <> struct LdsSet<FLOATS> {                                         \
+        __device__ static float* buf0() { return g_lds_a0_##FLOATS; }          \
+        __device__ static float* buf1() { return g_lds_a1_##FLOATS; }          \
+        __device__ static float* buf2() { return g_lds_a2_##FLOATS; }          \
     };
-template <int FLOATS> struct LdsPair;
-NMSPMM_LDS_PAIR(1024)
-NMSPMM_LDS_PAIR(2048)
-NMSPMM_LDS_PAIR(4096)
-NMSPMM_LDS_PAIR(8192)
-NMSPMM_LDS_PAIR(16384)
-NMSPMM_LDS_PAIR(32768)
+template <int FLOATS> struct LdsSet;
+NMSPMM_LDS_SET(1024)
+NMSPMM_LDS_SET(2048)
+NMSPMM_LDS_SET(4096)
+NMSPMM_LDS_SET(8192)
+NMSPMM_LDS_SET(16384)
+NMSPMM_LDS_SET(32768)
 
 // Buffer descriptors give branch-free guarded loads: an offset at or beyond num_records reads 0
 // without touching memory, so "this slot has nothing to load" is just an out-of-range offset.
@@ -143,11 +137,14 @@ constexpr int kWaitVm0 = 0x0F70;           // s_waitcnt vmcnt(0), other counters
 #ifndef NMSPMM_LDS_MIN
 #define NMSPMM_LDS_MIN 0  // extra dynamic LDS bytes to claim (caps workgroups per CU)
 #endif
-#ifndef NMSPMM_SKIP_ROWS
-#define NMSPMM_SKIP_ROWS 0  // HIGH: branch around load slots behind the end of the row list
+#ifndef NMSPMM_NBUF
+#define NMSPMM_NBUF 2       // LDS buffers of the A tile, 128-row waves
 #endif
-#ifndef NMSPMM_INTERLEAVE
-#define NMSPMM_INTERLEAVE 0  // k-steps over which the next window's loads are spread (0: all up front)
+#ifndef NMSPMM_NBUF_TALL
+#define NMSPMM_NBUF_TALL 2  // same for 256-row waves
+#endif
+#ifndef NMSPMM_TALL
+#define NMSPMM_TALL 1  // allow 256-row waves
 #endif
 #ifndef NMSPMM_GROUP
 #define NMSPMM_GROUP 8
@@ -162,14 +159,21 @@ constexpr int kWaitVm0 = 0x0F70;           // s_waitcnt vmcnt(0), other counters
 #define NMSPMM_CFG32 4, 1
 #endif
 
-template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+// NBUF: LDS buffers of the A tile.  2: the tile of window t+1 is loaded while window t is
+// multiplied and must have landed when the iteration ends.  3: the tile of window t+2 is loaded
+// during window t, its loads are spread between the MFMAs and have a whole further iteration to
+// land, so memory issue and the matrix pipe overlap inside one wave.
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH, int NBUF>
 __global__ void __launch_bounds__(64 * QS * WR, NMSPMM_OCC)
 spmm_mfma_kernel(const MfmaParams p)
 {
     typedef TileCfg<KS, WS, QS, WR, RM, HIGH> T;
+    static_assert(NBUF == 2 || NBUF == 3, "double or triple buffering");
+    static_assert(T::A_F4 % T::NT == 0, "every wave issues the same number of A loads");
     typedef typename AFrag<RM>::type afrag_t;
-    float* const As0 = LdsPair<T::AROWS * T::ASTR>::first();
-    float* const As1 = LdsPair<T::AROWS * T::ASTR>::second();
+    float* const As0 = LdsSet<T::AROWS * T::ASTR>::buf0();
+    float* const As1 = LdsSet<T::AROWS * T::ASTR>::buf1();
+    float* const As2 = NBUF == 3 ? LdsSet<T::AROWS * T::ASTR>::buf2() : nullptr;
 
     // ---- which tile -------------------------------------------------------------------------
     // Consecutive workgroup ids go to consecutive XCDs; give every XCD a contiguous run of
@@ -192,10 +196,6 @@ spmm_mfma_kernel(const MfmaParams p)
         tile_m = first_m + in_band % rows;
         tile_n = in_band / rows;
     }
-#ifdef NMSPMM_EXP_SAMETILE
-    tile_m = 0;
-    tile_n = 0;
-#endif
     const int bi = tile_m * T::MS;
     const int bj = tile_n * T::NS;
 
@@ -231,27 +231,21 @@ spmm_mfma_kernel(const MfmaParams p)
     constexpr int NW = T::NT / 64;
     constexpr int RPC = T::A_F4_ROW < 64 ? 64 / T::A_F4_ROW : 1;  // tile rows per 1 KiB chunk
     int ci_vec = -1;  // HIGH: column_info of the window whose A tile is loaded next
+    int ci_nxt = -1;  //       and of the one after it (in flight)
     auto load_cinfo = [&](int w) {
         const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cinfo + (size_t)w * KS, KS * sizeof(int32_t));
-        ci_vec = __builtin_amdgcn_raw_buffer_load_b32(rc, lane * (int)sizeof(int32_t), 0, 0);
+        ci_nxt = __builtin_amdgcn_raw_buffer_load_b32(rc, lane * (int)sizeof(int32_t), 0, 0);
     };
     auto load_a = [&](int w, float* dst) {
         const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w * KS * M, a_bytes);
         lds_f32* Ab = (lds_f32*)dst + wave * 256;
-#if NMSPMM_SKIP_ROWS
-        const int a_rows = HIGH ? __builtin_popcountll(__ballot(ci_vec >= 0)) : T::AROWS;
-#endif
 #pragma unroll
         for (int s = 0; s < T::A_SLOTS; ++s) {
             const int chunk = wave + s * NW;
             const int r0 = chunk * 64 / T::A_F4_ROW;  // first tile row of the chunk (wave-uniform)
             const int f4 = lane % T::A_F4_ROW + (T::A_F4_ROW > 64 ? (chunk * 64) % T::A_F4_ROW : 0);
             const bool in_tile = T::A_F4 % T::NT == 0 || s + 1 < T::A_SLOTS || chunk * 64 < T::A_F4;
-#if NMSPMM_SKIP_ROWS
-            if (in_tile && (!HIGH || r0 < a_rows)) {
-#else
             if (in_tile) {
-#endif
                 int src = r0 + lane / T::A_F4_ROW;
                 if (HIGH) {
                     src = __builtin_amdgcn_readlane(ci_vec, r0 & 63);
@@ -313,92 +307,106 @@ spmm_mfma_kernel(const MfmaParams p)
         for (int v = 0; v < 16; ++v)
             acc[b][v] = 0.0f;
 
-    // ---- prologue ---------------------------------------------------------------------------
+    // ---- prologue: windows 0 .. DA-1 of the slice into their buffers ---------------------------------
+    constexpr int DA = NBUF - 1;  // how many windows ahead of the multiplication the A tile is loaded
     const int w_last = w_begin + w_count - 1;
     if (w_count > 0) {
-        if (HIGH)
+        if (HIGH) {
             load_cinfo(w_begin);
+            ci_vec = ci_nxt;
+        }
         load_a(w_begin, As0);
+        if (NBUF == 3) {
+            if (HIGH) {
+                load_cinfo(min(w_begin + 1, w_last));
+                ci_vec = ci_nxt;
+            }
+            load_a(min(w_begin + 1, w_last), As1);
+        }
         load_b_idx(w_begin);
-        if (HIGH)
-            load_cinfo(min(w_begin + 1, w_last));
+        if (HIGH) {
+            load_cinfo(min(w_begin + DA, w_last));
+            ci_vec = ci_nxt;
+        }
         take_b_idx();
     }
     __builtin_amdgcn_s_waitcnt(kWaitVm0);
     __syncthreads();
 
     // ---- main loop: one window per iteration --------------------------------------------------
-    // The body is one basic block: loads for the next window are always issued (the last
-    // iteration re-reads its own window into the idle buffer, which is harmless).  The A tile of
-    // window t+1 streams into the other LDS buffer while window t is multiplied; the wave waits
-    // for its own loads, then the barrier publishes the buffer to the other waves.
-    auto window = [&](int t, const float* cur, float* nxt) {
+    // The body is one basic block: loads for later windows are always issued (past the end of the
+    // slice they re-read its last window into an idle buffer, which is harmless).  Per iteration:
+    // B, index and column_info loads for the next window first (few bytes, they have the whole
+    // iteration to land), then the MFMAs of this window with the LDS-direct loads of the A tile DA
+    // windows ahead; the wave waits for what the next iteration needs, then the barrier publishes
+    // it to the other waves.
+    constexpr int kWaitTile = NBUF == 2 ? 0 : T::A_SLOTS;  // NBUF 3: this iteration's A loads may stay in flight
+    // s_waitcnt vmcnt(kWaitTile) lgkmcnt(0): the loads the next iteration depends on have landed and
+    // every LDS read of this wave has executed, so after the barrier the buffer it read may be
+    // overwritten.  The barrier is the bare instruction: __syncthreads() carries a release fence
+    // that waits for ALL outstanding loads, including the tile loads meant to stay in flight.
+    constexpr int kWaitImm = (kWaitTile & 15) | (7 << 4) | (0 << 8) | ((kWaitTile >> 4) << 14);
+    auto window = [&](int t, const float* cur, float* dst) {
         const int w = w_begin + t;
-        const int w1 = min(w + 1, w_last);
-        TRACE_STAMP(0);
-#ifndef NMSPMM_EXP_NODMA
-        load_a(w1, nxt);
-#endif
-#ifndef NMSPMM_EXP_NOBIDX
-        load_b_idx(w1);
-#endif
-#ifndef NMSPMM_EXP_NOCI
+        load_b_idx(min(w + 1, w_last));
         if (HIGH)
-            load_cinfo(min(w + 2, w_last));
-#endif
-#if NMSPMM_INTERLEAVE == 0
-        // Keep the loads ahead of the multiplication: they need the whole MFMA phase to land.
-        __builtin_amdgcn_sched_barrier(0);
-        TRACE_STAMP(1);
-        __builtin_amdgcn_sched_barrier(0);
-#endif
+            load_cinfo(min(w + DA + 1, w_last));
+        if (NBUF == 2) {
+            load_a(min(w + 1, w_last), dst);
+            // Keep the loads ahead of the multiplication: they need the whole MFMA phase to land.
+            __builtin_amdgcn_sched_barrier(0);
+        }
 
         afrag_t av[T::KSTEPS];
 #pragma unroll
         for (int s = 0; s < T::KSTEPS; ++s)
             av[s] = load_frag<afrag_t>(cur + aoff[s]);
+        if (NBUF == 3)
+            load_a(min(w + DA, w_last), dst);
 #pragma unroll
         for (int s = 0; s < T::KSTEPS; ++s) {
 #pragma unroll
             for (int b = 0; b < RM; ++b)
                 acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_get(av[s], b), bv[s], acc[b], 0, 0, 0);
         }
-#if NMSPMM_INTERLEAVE
-        // Issue order inside the block: two fragment reads, then per k-step its RM MFMAs, one
-        // more fragment read, and (during the first NMSPMM_INTERLEAVE k-steps) a share of the next
-        // window's global loads, so that a stalled memory issue overlaps running MFMAs.
-        {
-            constexpr int VMEM = T::A_SLOTS + T::KSTEPS + ND + (HIGH ? 1 : 0);
-            constexpr int SPREAD = NMSPMM_INTERLEAVE < T::KSTEPS ? NMSPMM_INTERLEAVE : T::KSTEPS;
-            constexpr int VPS = (VMEM + SPREAD - 1) / SPREAD;
-            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        if (NBUF == 3) {
+            // Issue order: the small loads, two fragment reads, then per k-step its MFMAs, a share
+            // of the A-tile loads and the fragment reads of a later k-step.
+            constexpr int FR = RM == 8 ? 2 : 1;  // LDS reads per fragment
+            constexpr int DPS = (T::A_SLOTS + T::KSTEPS - 1) / T::KSTEPS;
+            __builtin_amdgcn_sched_group_barrier(0x020, T::KSTEPS + ND + (HIGH ? 1 : 0), 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * FR, 0);
 #pragma unroll
             for (int s = 0; s < T::KSTEPS; ++s) {
                 __builtin_amdgcn_sched_group_barrier(0x008, RM, 0);
-                if (s < SPREAD)
-                    __builtin_amdgcn_sched_group_barrier(0x020, VPS, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                if (s * DPS < T::A_SLOTS)
+                    __builtin_amdgcn_sched_group_barrier(0x020, DPS, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, FR, 0);
             }
         }
-#endif
 
-        __builtin_amdgcn_sched_barrier(0);
-        TRACE_STAMP(2);
+        // Nothing below may drift up: it consumes what was loaded at the top of this iteration.
         __builtin_amdgcn_sched_barrier(0);
         take_b_idx();
+        ci_vec = ci_nxt;
+        __builtin_amdgcn_s_waitcnt(kWaitImm);
+        __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        TRACE_STAMP(3);
-        __builtin_amdgcn_s_waitcnt(kWaitVm0);
-        TRACE_STAMP(4);
-#ifndef NMSPMM_EXP_NOBAR
-        __syncthreads();
-#endif
-        TRACE_STAMP(5);
     };
-    for (int t = 0; t < w_count; t += 2) {
-        window(t, As0, As1);
-        if (t + 1 < w_count)
-            window(t + 1, As1, As0);
+    if (NBUF == 2) {
+        for (int t = 0; t < w_count; t += 2) {
+            window(t, As0, As1);
+            if (t + 1 < w_count)
+                window(t + 1, As1, As0);
+        }
+    } else {
+        for (int t = 0; t < w_count; t += 3) {
+            window(t, As0, As2);
+            if (t + 1 < w_count)
+                window(t + 1, As1, As0);
+            if (t + 2 < w_count)
+                window(t + 2, As2, As1);
+        }
     }
 
     // ---- epilogue -----------------------------------------------------------------------------
@@ -412,17 +420,13 @@ spmm_mfma_kernel(const MfmaParams p)
 #pragma unroll
         for (int b = 0; b < RM; ++b) {
             const int row = bi + grp * (RM * 32) + (b / 4) * 128 + r32 * RUN + (b % 4);
-#ifdef NMSPMM_EXP_NOSTORE
-            if (row < M && acc[b][v] == 12345.f)
-#else
             if (row < M)
-#endif
                 out[(size_t)row * N + col] = acc[b][v];
         }
     }
 }
 
-template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH, int NBUF>
 static hipError_t launch_cfg(const SpmmArgs& a)
 {
     typedef TileCfg<KS, WS, QS, WR, RM, HIGH> T;
@@ -441,7 +445,7 @@ static hipError_t launch_cfg(const SpmmArgs& a)
     p.tiles_m = (a.M + T::MS - 1) / T::MS;
     p.tiles_n = a.N / T::NS;
     dim3 grid(p.tiles_m * p.tiles_n, a.split_k, 1);
-    spmm_mfma_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, dim3(T::NT), (size_t)NMSPMM_LDS_MIN, a.stream>>>(p);
+    spmm_mfma_kernel<KS, WS, QS, WR, RM, HIGH, NBUF><<<grid, dim3(T::NT), (size_t)NMSPMM_LDS_MIN, a.stream>>>(p);
     return hipGetLastError();
 }
 
@@ -456,11 +460,15 @@ static hipError_t launch_ns(const SpmmArgs& a)
 {
     switch (a.Ns) {
     case 128:
-        if ((long long)((a.M + 255) / 256) * (a.N / 128) * a.split_k >= 2 * kCus)
-            return launch_cfg<KS, WS, 4, 1, 8, HIGH>(a);
-        return launch_cfg<KS, WS, 4, NMSPMM_CFG128, HIGH>(a);
-    case 64: return launch_cfg<KS, WS, 2, NMSPMM_CFG64, HIGH>(a);
-    case 32: return launch_cfg<KS, WS, 1, NMSPMM_CFG32, HIGH>(a);
+        if (NMSPMM_TALL && (long long)((a.M + 255) / 256) * (a.N / 128) * a.split_k >= 2 * kCus) {
+            // three buffers only where they fit the 160 KiB of LDS
+            constexpr int nbuf = TileCfg<KS, WS, 4, 1, 8, HIGH>::LDS_BYTES / 2 * NMSPMM_NBUF_TALL <= 160 * 1024
+                                     ? NMSPMM_NBUF_TALL : 2;
+            return launch_cfg<KS, WS, 4, 1, 8, HIGH, nbuf>(a);
+        }
+        return launch_cfg<KS, WS, 4, NMSPMM_CFG128, HIGH, NMSPMM_NBUF>(a);
+    case 64: return launch_cfg<KS, WS, 2, NMSPMM_CFG64, HIGH, NMSPMM_NBUF>(a);
+    case 32: return launch_cfg<KS, WS, 1, NMSPMM_CFG32, HIGH, NMSPMM_NBUF>(a);
     }
     return hipErrorInvalidValue;
 }
