@@ -236,29 +236,40 @@ spmm_mfma_kernel(const MfmaParams p)
         const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cinfo + (size_t)w * KS, KS * sizeof(int32_t));
         ci_nxt = __builtin_amdgcn_raw_buffer_load_b32(rc, lane * (int)sizeof(int32_t), 0, 0);
     };
+    // Byte offset of every load slot inside its window.  LOW: fixed.  HIGH: formed from ci_vec;
+    // with few slots at the end of an iteration, where the readlanes and integer ops run under
+    // the tail of the MFMA phase instead of in front of the next iteration's loads (EARLY); with
+    // many slots right before each load, so that they do not all stay live across the MFMAs.
+    constexpr bool EARLY = !HIGH || T::A_SLOTS <= 8;
+    uint32_t a_off[EARLY ? T::A_SLOTS : 1];
+    auto slot_offset = [&](int s) -> uint32_t {
+        const int chunk = wave + s * NW;
+        const int r0 = chunk * 64 / T::A_F4_ROW;  // first tile row of the chunk (wave-uniform)
+        const int f4 = lane % T::A_F4_ROW + (T::A_F4_ROW > 64 ? (chunk * 64) % T::A_F4_ROW : 0);
+        int src = r0 + lane / T::A_F4_ROW;
+        if (HIGH) {
+            src = __builtin_amdgcn_readlane(ci_vec, r0 & 63);
+#pragma unroll
+            for (int g = 1; g < RPC; ++g) {
+                const int v = __builtin_amdgcn_readlane(ci_vec, (r0 + g) & 63);
+                src = (lane / T::A_F4_ROW == g) ? v : src;
+            }
+        }
+        return src >= 0 ? (uint32_t)(((size_t)src * M + f4 * 4) * sizeof(float)) : kNoLoad;
+    };
+    auto form_a_offsets = [&]() {
+        if (EARLY) {
+#pragma unroll
+            for (int s = 0; s < T::A_SLOTS; ++s)
+                a_off[s] = slot_offset(s);
+        }
+    };
     auto load_a = [&](int w, float* dst) {
         const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w * KS * M, a_bytes);
         lds_f32* Ab = (lds_f32*)dst + wave * 256;
 #pragma unroll
-        for (int s = 0; s < T::A_SLOTS; ++s) {
-            const int chunk = wave + s * NW;
-            const int r0 = chunk * 64 / T::A_F4_ROW;  // first tile row of the chunk (wave-uniform)
-            const int f4 = lane % T::A_F4_ROW + (T::A_F4_ROW > 64 ? (chunk * 64) % T::A_F4_ROW : 0);
-            const bool in_tile = T::A_F4 % T::NT == 0 || s + 1 < T::A_SLOTS || chunk * 64 < T::A_F4;
-            if (in_tile) {
-                int src = r0 + lane / T::A_F4_ROW;
-                if (HIGH) {
-                    src = __builtin_amdgcn_readlane(ci_vec, r0 & 63);
-#pragma unroll
-                    for (int g = 1; g < RPC; ++g) {
-                        const int v = __builtin_amdgcn_readlane(ci_vec, (r0 + g) & 63);
-                        src = (lane / T::A_F4_ROW == g) ? v : src;
-                    }
-                }
-                const uint32_t off = src >= 0 ? (uint32_t)(((size_t)src * M + f4 * 4) * sizeof(float)) : kNoLoad;
-                buffer_load_f4_to_lds(ra, Ab + s * NW * 256, off);
-            }
-        }
+        for (int s = 0; s < T::A_SLOTS; ++s)
+            buffer_load_f4_to_lds(ra, Ab + s * NW * 256, EARLY ? a_off[s] : slot_offset(s));
     };
 
     // ---- per-wave operands that bypass LDS ---------------------------------------------------------
@@ -315,11 +326,13 @@ spmm_mfma_kernel(const MfmaParams p)
             load_cinfo(w_begin);
             ci_vec = ci_nxt;
         }
+        form_a_offsets();
         load_a(w_begin, As0);
         if (NBUF == 3) {
             if (HIGH) {
                 load_cinfo(min(w_begin + 1, w_last));
                 ci_vec = ci_nxt;
+                form_a_offsets();
             }
             load_a(min(w_begin + 1, w_last), As1);
         }
@@ -327,6 +340,7 @@ spmm_mfma_kernel(const MfmaParams p)
         if (HIGH) {
             load_cinfo(min(w_begin + DA, w_last));
             ci_vec = ci_nxt;
+            form_a_offsets();
         }
         take_b_idx();
     }
@@ -348,11 +362,12 @@ spmm_mfma_kernel(const MfmaParams p)
     constexpr int kWaitImm = (kWaitTile & 15) | (7 << 4) | (0 << 8) | ((kWaitTile >> 4) << 14);
     auto window = [&](int t, const float* cur, float* dst) {
         const int w = w_begin + t;
+        if (NBUF == 2)
+            load_a(min(w + 1, w_last), dst);
         load_b_idx(min(w + 1, w_last));
         if (HIGH)
             load_cinfo(min(w + DA + 1, w_last));
         if (NBUF == 2) {
-            load_a(min(w + 1, w_last), dst);
             // Keep the loads ahead of the multiplication: they need the whole MFMA phase to land.
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -388,7 +403,10 @@ spmm_mfma_kernel(const MfmaParams p)
         // Nothing below may drift up: it consumes what was loaded at the top of this iteration.
         __builtin_amdgcn_sched_barrier(0);
         take_b_idx();
-        ci_vec = ci_nxt;
+        if (HIGH) {
+            ci_vec = ci_nxt;
+            form_a_offsets();
+        }
         __builtin_amdgcn_s_waitcnt(kWaitImm);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);

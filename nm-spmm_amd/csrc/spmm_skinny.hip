@@ -36,7 +36,14 @@ __device__ inline float sk_load(__amdgpu_buffer_rsrc_t r, uint32_t off)
     return __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
 }
 
-constexpr int kSkinnyWaves = 16;
+#ifndef NMSPMM_SK_WAVES
+#define NMSPMM_SK_WAVES 16
+#endif
+#ifndef NMSPMM_SK_UMUL
+#define NMSPMM_SK_UMUL 1
+#endif
+#define NMSPMM_SK_U(u) ((u) * NMSPMM_SK_UMUL)
+constexpr int kSkinnyWaves = NMSPMM_SK_WAVES;
 constexpr uint32_t kSkNoLoad = 0x80000000u;
 
 // KS: dense rows per window, WS: kept rows per window, QS: column vectors per preprocessed column
@@ -83,8 +90,8 @@ spmm_skinny_kernel(const SkinnyParams p)
     int civec[U];
     float a_nxt[STEPS], b_nxt[STEPS];
 
-    // metadata of the U windows starting at w (windows past the end are clamped; their B loads
-    // are suppressed below, so whatever they index contributes nothing)
+    // metadata of the U windows starting at w (windows past the end are clamped; their operand
+    // loads are suppressed below, so whatever they index contributes nothing)
     auto load_meta = [&](int w) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -99,20 +106,29 @@ spmm_skinny_kernel(const SkinnyParams p)
             }
         }
     };
-    // operands of the U windows starting at w, from the metadata currently in dvec / civec
-    auto load_operands = [&](int w) {
+    // B operands of the U windows starting at w: addresses depend on nothing, so these go out first
+    // and the HBM stream starts with the kernel.  A window past this wave's share loads nothing
+    // (zero-sized descriptor) and so adds exact zeros.
+    auto load_b = [&](int w) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int wu = w + u;
-            const bool live = wu < w_end;
             const __amdgpu_buffer_rsrc_t rb =
-                sk_rsrc(Bvec + (size_t)min(wu, p.nwin - 1) * WS * N, live ? b_bytes : 0u);
-            // a window past this wave's share loads nothing at all (zero-sized descriptors), so it
-            // adds exact zeros whatever the operands hold
-            const __amdgpu_buffer_rsrc_t ra_u = sk_rsrc(p.A, live ? a_bytes : 0u);
+                sk_rsrc(Bvec + (size_t)min(wu, p.nwin - 1) * WS * N, wu < w_end ? b_bytes : 0u);
             uint32_t boff = b_lane;
 #pragma unroll
-            for (int s = 0; s < KSTEPS; ++s, boff += b_step) {
+            for (int s = 0; s < KSTEPS; ++s, boff += b_step)
+                b_nxt[u * KSTEPS + s] = sk_load(rb, boff);
+        }
+    };
+    // A operands of the same windows, from the metadata currently in dvec / civec
+    auto load_a = [&](int w) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int wu = w + u;
+            const __amdgpu_buffer_rsrc_t ra_u = sk_rsrc(p.A, wu < w_end ? a_bytes : 0u);
+#pragma unroll
+            for (int s = 0; s < KSTEPS; ++s) {
                 const int e0 = 2 * s * QS, e1 = (2 * s + 1) * QS;
                 int lo = __builtin_amdgcn_readlane(dvec[u][e0 / 64], e0 % 64 + vec);
                 int hi = __builtin_amdgcn_readlane(dvec[u][e1 / 64], e1 % 64 + vec);
@@ -121,15 +137,17 @@ spmm_skinny_kernel(const SkinnyParams p)
                     hi = __builtin_amdgcn_readlane(civec[u], hi & 63);
                 }
                 const int k = min(wu, p.nwin - 1) * KS + (h ? hi : lo);
-                b_nxt[u * KSTEPS + s] = sk_load(rb, boff);
                 a_nxt[u * KSTEPS + s] = sk_load(ra_u, a_lane + (uint32_t)((size_t)k * M * sizeof(float)));
             }
         }
     };
 
+    // Load order per chunk: metadata, B, then (once the metadata has landed) A.  Loads return in
+    // order, so waiting for the metadata never waits for the B stream issued after it.
     if (w_count > 0) {
         load_meta(w_begin);
-        load_operands(w_begin);
+        load_b(w_begin);
+        load_a(w_begin);
         if (U < w_count)
             load_meta(w_begin + U);
     }
@@ -141,7 +159,8 @@ spmm_skinny_kernel(const SkinnyParams p)
             b_cur[s] = b_nxt[s];
         }
         if (w + U < w_end) {
-            load_operands(w + U);
+            load_b(w + U);
+            load_a(w + U);
             if (w + 2 * U < w_end)
                 load_meta(w + 2 * U);
         }
@@ -156,8 +175,7 @@ spmm_skinny_kernel(const SkinnyParams p)
         red[wave][v][lane] = acc[v];
     __syncthreads();
     // wave v finishes result register v: rows 8*(v/4) + 4*h + v%4 (h = lane half), column j
-    {
-        const int v = wave;
+    for (int v = wave; v < 16; v += kSkinnyWaves) {
         float s = red[0][v][lane];
 #pragma unroll
         for (int x = 1; x < kSkinnyWaves; ++x)
@@ -208,12 +226,12 @@ hipError_t launch_skinny(const SpmmArgs& a)
 {
     const bool high = a.cinfo != nullptr;
     if (!high) {
-        if (a.kept == 32) return launch_qs<32, 32, false, 1>(a);
-        if (a.kept == 16) return launch_qs<32, 16, false, 2>(a);
-        if (a.kept == 12) return launch_qs<32, 12, false, 2>(a);
+        if (a.kept == 32) return launch_qs<32, 32, false, NMSPMM_SK_U(1)>(a);
+        if (a.kept == 16) return launch_qs<32, 16, false, NMSPMM_SK_U(2)>(a);
+        if (a.kept == 12) return launch_qs<32, 12, false, NMSPMM_SK_U(2)>(a);
     } else {
-        if (a.kept == 16) return launch_qs<64, 16, true, 2>(a);
-        if (a.kept == 8) return launch_qs<64, 8, true, 4>(a);
+        if (a.kept == 16) return launch_qs<64, 16, true, NMSPMM_SK_U(2)>(a);
+        if (a.kept == 8) return launch_qs<64, 8, true, NMSPMM_SK_U(4)>(a);
     }
     return hipErrorInvalidValue;
 }
