@@ -146,6 +146,12 @@ constexpr int kWaitVm0 = 0x0F70;           // s_waitcnt vmcnt(0), other counters
 #ifndef NMSPMM_TALL
 #define NMSPMM_TALL 1  // allow 256-row waves
 #endif
+#ifndef NMSPMM_GATHER
+#define NMSPMM_GATHER 1          // high-sparsity layout: wave-private gather kernel
+#endif
+#ifndef NMSPMM_GATHER_RM_TALL
+#define NMSPMM_GATHER_RM_TALL 8  // its wave height (32-row blocks) for large problems
+#endif
 #ifndef NMSPMM_GROUP
 #define NMSPMM_GROUP 8
 #endif
@@ -444,6 +450,233 @@ spmm_mfma_kernel(const MfmaParams p)
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Wave-private gather kernel for the high-sparsity layout.
+//
+// At 75 % sparsity and above a column vector touches only WS of a window's 64 rows, so the rows one
+// wave needs (WS per window) are about as many bytes as its quarter share of the workgroup's
+// compacted tile.  Each wave therefore stages ITS OWN rows: the gather happens in the global
+// address of the LDS-direct load (row = column_info[rank]), the rows land in kept order in a
+// region of LDS that only this wave reads, the MFMA operand reads use fixed addresses, and the
+// window loop needs no barrier and no cross-wave wait at all: waves drift apart and their memory
+// and matrix phases overlap on the CU.
+//
+// One workgroup = QS waves = one 32-column vector each, RM*32 rows tall.  Two LDS objects (window
+// parity) so that the compiler can tell the reads of one from the asynchronous writes into the other.
+template <int FLOATS> struct LdsPairG;
+#define NMSPMM_LDS_PAIRG(FLOATS)                                                \
+    __shared__ __align__(16) float g_lds_g0_##FLOATS[FLOATS];                  \
+    __shared__ __align__(16) float g_lds_g1_##FLOATS[FLOATS];                  \
+    template <> struct LdsPairG<FLOATS> {                                       \
+        __device__ static float* even() { return g_lds_g0_##FLOATS; }          \
+        __device__ static float* odd() { return g_lds_g1_##FLOATS; }           \
+    };
+NMSPMM_LDS_PAIRG(1024)
+NMSPMM_LDS_PAIRG(2048)
+NMSPMM_LDS_PAIRG(4096)
+NMSPMM_LDS_PAIRG(8192)
+NMSPMM_LDS_PAIRG(16384)
+
+__device__ inline void buffer_load_f4_to_lds_s(__amdgpu_buffer_rsrc_t r, lds_f32* dst, uint32_t v_off, uint32_t s_off)
+{
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, dst, 16, v_off, s_off, 0, 0);
+}
+
+template <int KS, int WS, int QS, int RM>
+__global__ void __launch_bounds__(64 * QS, NMSPMM_OCC)
+spmm_gather_kernel(const MfmaParams p)
+{
+    static_assert(RM == 4 || RM == 8, "128- or 256-row waves");
+    typedef typename AFrag<RM>::type afrag_t;
+    constexpr int MS = RM * 32;
+    constexpr int NS = QS * 32;
+    constexpr int KSTEPS = WS / 2;
+    constexpr int RPI = 256 / MS;            // rows per 1 KiB load: 1 (256-row waves) or 2
+    constexpr int A_SLOTS = WS / RPI;
+    constexpr int ND = (WS * QS + 63) / 64;
+    constexpr int WAVE_FLOATS = WS * MS;     // one window of one wave
+    float* const L0 = LdsPairG<QS * WAVE_FLOATS>::even();
+    float* const L1 = LdsPairG<QS * WAVE_FLOATS>::odd();
+
+    // ---- which tile (same walk as the shared-tile kernel) ---------------------------------------
+    const int total = p.tiles_m * p.tiles_n;
+    int logical;
+    {
+        const int id = blockIdx.x;
+        const int q = total / kXcds, r = total % kXcds;
+        const int xcd = id % kXcds, loc = id / kXcds;
+        logical = xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc;
+    }
+    constexpr int GROUP = NMSPMM_GROUP;
+    int tile_m, tile_n;
+    {
+        const int band = logical / (GROUP * p.tiles_n);
+        const int first_m = band * GROUP;
+        const int rows = min(GROUP, p.tiles_m - first_m);
+        const int in_band = logical - band * GROUP * p.tiles_n;
+        tile_m = first_m + in_band % rows;
+        tile_n = in_band / rows;
+    }
+    const int bi = tile_m * MS;
+    const int bj = tile_n * NS;
+    int w_begin, w_count;
+    split_windows(p.nwin, p.split_k, blockIdx.y, &w_begin, &w_count);
+    const int w_last = w_begin + w_count - 1;
+
+    const int lane = threadIdx.x & 63;
+    const int vec = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave = column vector
+    const int h = lane >> 5;
+    const int j = lane & 31;
+    const int M = p.M, N = p.N;
+    const float* const Ablk = p.A + bi;
+    const float* const Bvec = p.B + bj + vec * 32;
+    const int32_t* const Dblk = p.D + (size_t)tile_n * p.W * QS;
+    const int32_t* const Cinfo = p.cinfo + (size_t)tile_n * p.nwin * KS;
+    const uint32_t a_bytes = (uint32_t)(((size_t)(KS - 1) * M + (M - bi)) * sizeof(float));
+    const uint32_t b_bytes = (uint32_t)(((size_t)(WS - 1) * N + 32) * sizeof(float));
+    const uint32_t b_lane = (uint32_t)(((size_t)h * N + j) * sizeof(float));
+    const uint32_t b_step = (uint32_t)(2 * (size_t)N * sizeof(float));
+    const uint32_t row_bytes = (uint32_t)((size_t)M * sizeof(float));
+    const uint32_t a_vlane = (uint32_t)((lane % (MS / 4)) * 16);  // this lane's 16 bytes inside a row
+
+    // metadata one window ahead of the loads that use it: ranks of this block's vectors and the
+    // block's row list, one wave-wide load each
+    int d_vec[ND], d_nxt[ND], ci_vec = -1, ci_nxt = -1;
+    auto load_meta = [&](int w) {
+        const __amdgpu_buffer_rsrc_t rd = make_rsrc(Dblk + (size_t)w * WS * QS, WS * QS * sizeof(int32_t));
+#pragma unroll
+        for (int q = 0; q < ND; ++q)
+            d_nxt[q] = __builtin_amdgcn_raw_buffer_load_b32(rd, (lane + 64 * q) * (int)sizeof(int32_t), 0, 0);
+        const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cinfo + (size_t)w * KS, KS * sizeof(int32_t));
+        ci_nxt = __builtin_amdgcn_raw_buffer_load_b32(rc, lane * (int)sizeof(int32_t), 0, 0);
+    };
+    auto take_meta = [&]() {
+#pragma unroll
+        for (int q = 0; q < ND; ++q)
+            d_vec[q] = d_nxt[q];
+        ci_vec = ci_nxt;
+    };
+    // window-local A row of kept row p of this wave's vector (wave-uniform)
+    auto row_of = [&](int pp) -> int {
+        const int e = pp * QS;
+        const int rank = __builtin_amdgcn_readlane(d_vec[e / 64], e % 64 + vec);
+        return __builtin_amdgcn_readlane(ci_vec, rank & 63);
+    };
+    // the wave's WS rows of window w -> dst (kept order), gathered by the load addresses
+    auto load_rows = [&](int w, float* dst) {
+        const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w * KS * M, a_bytes);
+        lds_f32* Ab = (lds_f32*)dst + vec * WAVE_FLOATS;
+#pragma unroll
+        for (int s = 0; s < A_SLOTS; ++s) {
+            if (RPI == 1) {
+                buffer_load_f4_to_lds_s(ra, Ab + s * 256, a_vlane, (uint32_t)row_of(s) * row_bytes);
+            } else {
+                const int r0 = row_of(2 * s), r1 = row_of(2 * s + 1);
+                buffer_load_f4_to_lds(ra, Ab + s * 256, (uint32_t)(h ? r1 : r0) * row_bytes + a_vlane);
+            }
+        }
+    };
+    float b_next[KSTEPS], bv[KSTEPS];
+    auto load_b = [&](int w) {
+        const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)w * WS * N, b_bytes);
+        uint32_t off = b_lane;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s, off += b_step)
+            b_next[s] = buffer_load_f1(rb, off, 0);
+    };
+
+    floatx16 acc[RM];
+#pragma unroll
+    for (int b = 0; b < RM; ++b)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            acc[b][v] = 0.0f;
+
+    // fixed operand address: kept row 2s + h, this lane's runs of four rows
+    const int a_lane = vec * WAVE_FLOATS + h * MS + j * 4;
+
+    if (w_count > 0) {
+        load_meta(w_begin);
+        take_meta();
+        load_rows(w_begin, L0);
+        load_b(w_begin);
+        load_meta(min(w_begin + 1, w_last));
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+            bv[s] = b_next[s];
+        take_meta();
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitVm0);
+
+    auto window = [&](int t, const float* cur, float* nxt) {
+        const int w = w_begin + t;
+        load_rows(min(w + 1, w_last), nxt);
+        load_b(min(w + 1, w_last));
+        load_meta(min(w + 2, w_last));
+        __builtin_amdgcn_sched_barrier(0);
+
+        afrag_t av[KSTEPS];
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+            av[s] = load_frag<afrag_t>(cur + a_lane + 2 * s * MS);
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+#pragma unroll
+            for (int b = 0; b < RM; ++b)
+                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_get(av[s], b), bv[s], acc[b], 0, 0, 0);
+        }
+
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+            bv[s] = b_next[s];
+        take_meta();
+        // own loads landed, own LDS reads executed: the other buffer may be read, this one refilled
+        __builtin_amdgcn_s_waitcnt(0x0070);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    for (int t = 0; t < w_count; t += 2) {
+        window(t, L0, L1);
+        if (t + 1 < w_count)
+            window(t + 1, L1, L0);
+    }
+
+    float* out = p.out + (size_t)blockIdx.y * p.slice_elems;
+    const int col = bj + vec * 32 + j;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int r32 = 8 * (v / 4) + 4 * h + (v % 4);
+#pragma unroll
+        for (int b = 0; b < RM; ++b) {
+            const int row = bi + (b / 4) * 128 + r32 * 4 + (b % 4);
+            if (row < M)
+                out[(size_t)row * N + col] = acc[b][v];
+        }
+    }
+}
+
+template <int KS, int WS, int QS, int RM>
+static hipError_t launch_gather(const SpmmArgs& a)
+{
+    MfmaParams p;
+    p.A = a.A;
+    p.B = a.B;
+    p.D = a.D;
+    p.cinfo = a.cinfo;
+    p.out = a.split_k > 1 ? a.partial : a.C;
+    p.slice_elems = a.slice_stride;
+    p.M = a.M;
+    p.N = a.N;
+    p.W = a.W;
+    p.nwin = a.W / WS;
+    p.split_k = a.split_k;
+    p.tiles_m = (a.M + RM * 32 - 1) / (RM * 32);
+    p.tiles_n = a.N / (QS * 32);
+    dim3 grid(p.tiles_m * p.tiles_n, a.split_k, 1);
+    spmm_gather_kernel<KS, WS, QS, RM><<<grid, dim3(64 * QS), 0, a.stream>>>(p);
+    return hipGetLastError();
+}
+
 template <int KS, int WS, int QS, int WR, int RM, bool HIGH, int NBUF>
 static hipError_t launch_cfg(const SpmmArgs& a)
 {
@@ -476,6 +709,20 @@ constexpr int kCus = 256;
 template <int KS, int WS, bool HIGH>
 static hipError_t launch_ns(const SpmmArgs& a)
 {
+#if NMSPMM_GATHER
+    if constexpr (HIGH) {
+        const bool tall = (long long)((a.M + 255) / 256) * (a.N / a.Ns) * a.split_k >= 2 * kCus;
+        switch (a.Ns) {
+        case 128: {
+            // 256-row waves only while two workgroups still fit a CU (64 KiB of LDS each)
+            constexpr int tall_rm = 2 * 4 * WS * 256 * (int)sizeof(float) <= 64 * 1024 ? NMSPMM_GATHER_RM_TALL : 4;
+            return tall ? launch_gather<KS, WS, 4, tall_rm>(a) : launch_gather<KS, WS, 4, 4>(a);
+        }
+        case 64: return launch_gather<KS, WS, 2, 4>(a);
+        case 32: return launch_gather<KS, WS, 1, 4>(a);
+        }
+    }
+#endif
     switch (a.Ns) {
     case 128:
         if (NMSPMM_TALL && (long long)((a.M + 255) / 256) * (a.N / 128) * a.split_k >= 2 * kCus) {
