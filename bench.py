@@ -85,7 +85,18 @@ class Case:
         return 2.0 * M * N * self.W
 
 
-def time_launches(torch, fn, steps, warmup):
+PREWARM_S = 1.0
+
+
+def time_launches(torch, fn, steps, warmup, prewarm_s=None):
+    """`warmup` untimed steps, then exactly `steps` timed ones.  Before both, the step is repeated
+    for about prewarm_s seconds: an idle MI355X sits near 1 GHz and takes some hundred milliseconds of
+    load to reach its sustained shader clock, far longer than a few sub-millisecond launches."""
+    t_end = time.perf_counter() + (PREWARM_S if prewarm_s is None else prewarm_s)
+    while time.perf_counter() < t_end:
+        for _ in range(50):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -209,7 +220,7 @@ def main():
         "metric": "useful fp32 TFLOP/s, M=Ncols=K=4096, 2:4 (vector length 32)",
         "value": round(achieved, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "dtype": "f32", "data": "synthetic", "clock_prewarm_s": PREWARM_S,
         "config": {"workload": "square sweep M=Ncols=K=4096 fp32, uniform(-1,1), seeded n:m patterns per 32-column "
                                "vector; value at 2:4, others under sweep", "tile": "Ns=128", "split_k": 1},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",

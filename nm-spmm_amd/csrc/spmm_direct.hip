@@ -1,0 +1,332 @@
+// Matrix-core kernel for C = A . B with an N:M-sparse B whose index pattern is shared by 32
+// adjacent columns (reference kernels: src/kernel_{64x128_8x8,64x64_8x8,32x64_8x4,32x32_4x4}.cu;
+// this file replaces their role, not their design).
+//
+// Design for gfx950 (64-lane waves, v_mfma_f32_32x32x2_f32):
+//  * A 32-column index vector is exactly the N extent of one 32x32x2 MFMA, so one wave owns one
+//    column vector and RM row blocks of 32 rows, and is independent of every other wave: no LDS,
+//    no barrier.
+//  * The A operand of one MFMA is A[row][k] with lane = (row % 32, k half): lanes 0-31 take kept
+//    row 2s of the window, lanes 32-63 kept row 2s+1, and each half reads the dense row of A that
+//    *its* index selects.  A is column-major, so that is M contiguous floats: the gather is a
+//    per-lane row offset of an ordinary load and moves no data.
+//  * The wave's RM row blocks interleave rows (block b holds rows 4*r + b; a 256-row wave has two
+//    such groups 128 rows apart), so one 128-bit load per lane is the A operand of four MFMAs -
+//    two 512-byte row segments per wave and instruction - and the B operand is reused RM times.
+//  * Rolling register pipeline: right after the MFMAs of k-step s have been issued, the operands
+//    of k-step s of the next chunk of kept rows are loaded into the same registers, so every load
+//    has a whole chunk of MFMA work (thousands of cycles) to land, memory instructions are spread
+//    evenly between the MFMAs, and one set of operand registers suffices.  The reuse of A between
+//    the column vectors of a workgroup and between neighbouring workgroups is left to the vector
+//    L1 and the L2: the tile walk keeps the workgroups resident on one XCD in a compact patch of C.
+//  * Index metadata arrives as one wave-wide load per window ([kept][Ns/32] ints, plus the
+//    column_info list of the window on the high-sparsity layout), two windows ahead, and is
+//    handed to the lanes with v_readlane: the row numbers become scalars, the per-lane select
+//    between the two halves is one v_cndmask.
+//  * All loads go through buffer descriptors whose extent ends with the window's last row, so no
+//    lane reads outside A or B without a branch; lanes whose rows lie beyond M read zeros or
+//    other rows' values into accumulators that are never stored.
+#include "internal.h"
+
+namespace nmspmm {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kXcds = 8;
+constexpr int kCus = 256;
+
+struct DirectParams {
+    const float* A;
+    const float* B;
+    const int32_t* D;
+    const int32_t* cinfo;
+    float* out;          // C, or the first partial slice when split_k > 1
+    size_t slice_elems;  // floats between partial slices
+    int M, N, W;
+    int nwin;            // windows in the whole reduction
+    int split_k;
+    int tiles_m, tiles_n;
+};
+
+struct float8 { float4 lo, hi; };
+template <int RM> struct AFrag;
+template <> struct AFrag<8> { typedef float8 type; };
+template <> struct AFrag<4> { typedef float4 type; };
+
+__device__ inline float frag_get(const float4& v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+__device__ inline float frag_get(const float8& v, int i) { return i < 4 ? frag_get(v.lo, i) : frag_get(v.hi, i - 4); }
+
+// Buffer descriptors give branch-free guarded loads: an offset at or beyond num_records reads 0
+// without touching memory.
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+__device__ inline float4 buffer_load_f4(__amdgpu_buffer_rsrc_t r, uint32_t byte_off)
+{
+    auto v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
+    return *reinterpret_cast<float4*>(&v);
+}
+__device__ inline float buffer_load_f1(__amdgpu_buffer_rsrc_t r, uint32_t byte_off, uint32_t s_off)
+{
+    return __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, byte_off, s_off, 0));
+}
+
+// Tuning knobs (compile-time): waves per SIMD the register allocation must allow for 128-row
+// waves (256-row waves get two), and the tile-walk band height.
+#ifndef NMSPMM_OCC
+#define NMSPMM_OCC 3
+#endif
+#ifndef NMSPMM_GROUP
+#define NMSPMM_GROUP 8
+#endif
+#ifndef NMSPMM_RM_TALL
+#define NMSPMM_RM_TALL 8
+#endif
+
+// KS: dense rows per window, WS: kept rows per window, QS: column vectors per preprocessed column
+// block (Ns = 32*QS), WR: waves along M, RM: 32-row blocks per wave (4 or 8), HIGH:
+// high-sparsity layout (D holds ranks into the window's column_info list).
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+__global__ void __launch_bounds__(64 * QS * WR, RM == 8 ? 2 : NMSPMM_OCC)
+spmm_direct_kernel(const DirectParams p)
+{
+    static_assert(RM == 4 || RM == 8, "128- or 256-row waves");
+    static_assert(WS % 2 == 0, "two kept rows per MFMA");
+    typedef typename AFrag<RM>::type afrag_t;
+    constexpr int MW = RM * 32;               // rows per wave
+    constexpr int MS = WR * MW;               // rows per workgroup tile
+    constexpr int NS = QS * 32;
+    constexpr int CH = WS <= 16 ? WS : 16;    // kept rows per pipeline chunk
+    constexpr int NCH = WS / CH;
+    constexpr int CS = CH / 2;                // MFMA k-steps per chunk
+    constexpr int ND = (WS * QS + 63) / 64;   // wave-wide loads per window of indices
+    static_assert(WS % CH == 0, "whole chunks");
+
+    // ---- tile walk: consecutive ids go to different XCDs, so give each XCD a contiguous run of
+    // logical tiles, walked in bands of GROUP row tiles across all column blocks.
+    const int total = p.tiles_m * p.tiles_n;
+    int logical;
+    {
+        const int id = blockIdx.x;
+        const int q = total / kXcds, r = total % kXcds;
+        const int xcd = id % kXcds, loc = id / kXcds;
+        logical = xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc;
+    }
+    constexpr int GROUP = NMSPMM_GROUP;
+    int tile_m, tile_n;
+    {
+        const int band = logical / (GROUP * p.tiles_n);
+        const int first_m = band * GROUP;
+        const int rows = min(GROUP, p.tiles_m - first_m);
+        const int in_band = logical - band * GROUP * p.tiles_n;
+        tile_m = first_m + in_band % rows;
+        tile_n = in_band / rows;
+    }
+    int w_begin, w_count;
+    split_windows(p.nwin, p.split_k, blockIdx.y, &w_begin, &w_count);
+    const int w_last = w_begin + w_count - 1;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int vec = wave % QS;
+    const int wr = wave / QS;
+    const int h = lane >> 5;
+    const int j = lane & 31;
+    const int M = p.M, N = p.N;
+    const int bi = tile_m * MS + wr * MW;     // first row of this wave (may be >= M: loads nothing)
+    const int bj = tile_n * NS + vec * 32;
+
+    const float* const Ablk = p.A + min(bi, M);
+    const float* const Bvec = p.B + bj;
+    const int32_t* const Dblk = p.D + (size_t)tile_n * p.W * QS;
+    const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)tile_n * p.nwin * KS : nullptr;
+    // extents: the last dense row of a window ends with the matrix, the last kept row of B with
+    // this vector's 32 columns
+    const uint32_t a_bytes = bi < M ? (uint32_t)(((size_t)(KS - 1) * M + (size_t)(M - bi)) * sizeof(float)) : 0u;
+    const uint32_t b_bytes = (uint32_t)(((size_t)(WS - 1) * N + 32) * sizeof(float));
+    const uint32_t row_bytes = (uint32_t)((size_t)M * sizeof(float));
+    const uint32_t a_vlane = (uint32_t)(j * 16);  // this lane's run of four rows inside the wave's rows
+    const uint32_t b_chunk = (uint32_t)((size_t)CH * N * sizeof(float));
+    uint32_t b_off[CS];
+#pragma unroll
+    for (int s = 0; s < CS; ++s)
+        b_off[s] = (uint32_t)(((size_t)(2 * s + h) * N + j) * sizeof(float));
+
+    // ---- index metadata: d_vec / ci_vec belong to the window whose operands are being loaded,
+    // d_nxt / ci_nxt to the one after it
+    int d_vec[ND], d_nxt[ND], ci_vec = -1, ci_nxt = -1;
+    auto load_meta = [&](int w) {
+        const __amdgpu_buffer_rsrc_t rd = make_rsrc(Dblk + (size_t)w * WS * QS, WS * QS * sizeof(int32_t));
+#pragma unroll
+        for (int q = 0; q < ND; ++q)
+            d_nxt[q] = __builtin_amdgcn_raw_buffer_load_b32(rd, (lane + 64 * q) * (int)sizeof(int32_t), 0, 0);
+        if constexpr (HIGH) {
+            const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cinfo + (size_t)w * KS, KS * sizeof(int32_t));
+            ci_nxt = __builtin_amdgcn_raw_buffer_load_b32(rc, lane * (int)sizeof(int32_t), 0, 0);
+        }
+    };
+    auto take_meta = [&]() {
+#pragma unroll
+        for (int q = 0; q < ND; ++q)
+            d_vec[q] = d_nxt[q];
+        ci_vec = ci_nxt;
+    };
+    // window-local dense row of kept row pp of this wave's vector (a scalar)
+    auto row_of = [&](int pp) -> int {
+        const int e = pp * QS;
+        const int idx = __builtin_amdgcn_readlane(d_vec[e / 64], e % 64 + vec);
+        if constexpr (!HIGH)
+            return idx;
+        return __builtin_amdgcn_readlane(ci_vec, idx & 63);
+    };
+
+    afrag_t a_op[CS];
+    float b_op[CS];
+    // operands of k-step s of chunk c of the window the descriptors point at
+    auto load_step = [&](int c, int s, __amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb) {
+        const int r0 = row_of(c * CH + 2 * s), r1 = row_of(c * CH + 2 * s + 1);
+        const uint32_t off = (uint32_t)(h ? r1 : r0) * row_bytes + a_vlane;
+        if constexpr (RM == 8) {
+            a_op[s].lo = buffer_load_f4(ra, off);
+            a_op[s].hi = buffer_load_f4(ra, off + 512);
+        } else {
+            a_op[s] = buffer_load_f4(ra, off);
+        }
+        b_op[s] = buffer_load_f1(rb, b_off[s], c * b_chunk);
+    };
+
+    floatx16 acc[RM];
+#pragma unroll
+    for (int b = 0; b < RM; ++b)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            acc[b][v] = 0.0f;
+
+    if (w_count > 0) {
+        load_meta(w_begin);
+        take_meta();
+        const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w_begin * KS * M, a_bytes);
+        const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)w_begin * WS * N, b_bytes);
+#pragma unroll
+        for (int s = 0; s < CS; ++s)
+            load_step(0, s, ra, rb);
+        load_meta(min(w_begin + 1, w_last));
+    }
+    for (int t = 0; t < w_count; ++t) {
+        const int w = w_begin + t;
+        const int wn = min(w + 1, w_last);  // the last window reloads itself; nothing consumes it
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            // while chunk c is multiplied, chunk c+1 (or chunk 0 of the next window) is loaded
+            const bool wrap = c == NCH - 1;
+            if (wrap) {
+                __builtin_amdgcn_sched_barrier(0);
+                take_meta();
+                load_meta(min(w + 2, w_last));
+            }
+            const int wl = wrap ? wn : w;
+            const int cl = wrap ? 0 : c + 1;
+            const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)wl * KS * M, a_bytes);
+            const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)wl * WS * N, b_bytes);
+#pragma unroll
+            for (int s = 0; s < CS; ++s) {
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int b = 0; b < RM; ++b)
+                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_get(a_op[s], b), b_op[s], acc[b], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                load_step(cl, s, ra, rb);
+            }
+        }
+    }
+
+    // ---- epilogue: MFMA result register v of lane (h, j) is row 8*(v/4) + 4*h + v%4 of the block,
+    // column j; block b of the wave holds rows (b/4)*128 + 4*r + b%4
+    float* out = p.out + (size_t)blockIdx.y * p.slice_elems;
+    const int col = bj + j;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int r32 = 8 * (v / 4) + 4 * h + (v % 4);
+#pragma unroll
+        for (int b = 0; b < RM; ++b) {
+            const int row = bi + (b / 4) * 128 + r32 * 4 + (b % 4);
+            if (row < M)
+                out[(size_t)row * N + col] = acc[b][v];
+        }
+    }
+}
+
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+static hipError_t launch_cfg(const SpmmArgs& a)
+{
+    constexpr int MS = WR * RM * 32;
+    DirectParams p;
+    p.A = a.A;
+    p.B = a.B;
+    p.D = a.D;
+    p.cinfo = a.cinfo;
+    p.out = a.split_k > 1 ? a.partial : a.C;
+    p.slice_elems = a.slice_stride;
+    p.M = a.M;
+    p.N = a.N;
+    p.W = a.W;
+    p.nwin = a.W / WS;
+    p.split_k = a.split_k;
+    p.tiles_m = (a.M + MS - 1) / MS;
+    p.tiles_n = a.N / (QS * 32);
+    const dim3 grid(p.tiles_m * p.tiles_n, a.split_k, 1);
+    spmm_direct_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, dim3(64 * QS * WR), 0, a.stream>>>(p);
+    return hipGetLastError();
+}
+
+// Every workgroup has four waves: 1 x 4, 2 x 2 or 4 x 1 (rows x column vectors), chosen by the
+// column-block width the indices were preprocessed for.  A wave is 256 rows tall when that still
+// leaves every SIMD two waves (the taller wave halves the B and index loads per MFMA), 128 rows
+// otherwise.
+template <int KS, int WS, bool HIGH>
+static hipError_t launch_ns(const SpmmArgs& a)
+{
+    const long long waves_tall = (long long)((a.M + 255) / 256) * (a.N / 32) * a.split_k;
+    const bool tall = waves_tall >= 2LL * 4 * kCus;
+    switch (a.Ns) {
+    case 128:
+        return tall ? launch_cfg<KS, WS, 4, 1, NMSPMM_RM_TALL, HIGH>(a) : launch_cfg<KS, WS, 4, 1, 4, HIGH>(a);
+    case 64:
+        return tall ? launch_cfg<KS, WS, 2, 2, NMSPMM_RM_TALL, HIGH>(a) : launch_cfg<KS, WS, 2, 2, 4, HIGH>(a);
+    case 32:
+        return tall ? launch_cfg<KS, WS, 1, 4, NMSPMM_RM_TALL, HIGH>(a) : launch_cfg<KS, WS, 1, 4, 4, HIGH>(a);
+    }
+    return hipErrorInvalidValue;
+}
+
+bool mfma_supported(const SpmmArgs& a)
+{
+    if (a.vec_len != 32 || (a.Ns != 32 && a.Ns != 64 && a.Ns != 128))
+        return false;
+    if (a.M % 4 != 0 || a.M < 32)
+        return false;
+    // 32-bit buffer offsets: one window of A and one window of B must stay below 2 GiB
+    if ((size_t)a.window * a.M * sizeof(float) >= 0x80000000ull || (size_t)a.kept * a.N * sizeof(float) >= 0x80000000ull)
+        return false;
+    const bool high = a.cinfo != nullptr;
+    if (!high)
+        return a.window == 32 && (a.kept == 32 || a.kept == 16 || a.kept == 12);
+    return a.window == 64 && (a.kept == 16 || a.kept == 8);
+}
+
+hipError_t launch_mfma(const SpmmArgs& a)
+{
+    const bool high = a.cinfo != nullptr;
+    if (!high) {
+        if (a.kept == 32) return launch_ns<32, 32, false>(a);
+        if (a.kept == 16) return launch_ns<32, 16, false>(a);
+        if (a.kept == 12) return launch_ns<32, 12, false>(a);
+    } else {
+        if (a.kept == 16) return launch_ns<64, 16, true>(a);
+        if (a.kept == 8) return launch_ns<64, 8, true>(a);
+    }
+    return hipErrorInvalidValue;
+}
+
+} // namespace nmspmm

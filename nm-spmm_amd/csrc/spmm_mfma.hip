@@ -149,6 +149,9 @@ constexpr int kWaitVm0 = 0x0F70;           // s_waitcnt vmcnt(0), other counters
 #ifndef NMSPMM_GATHER
 #define NMSPMM_GATHER 1          // high-sparsity layout: wave-private gather kernel
 #endif
+#ifndef NMSPMM_DIRECT_LOW
+#define NMSPMM_DIRECT_LOW 0
+#endif
 #ifndef NMSPMM_GATHER_RM_TALL
 #define NMSPMM_GATHER_RM_TALL 8  // its wave height (32-row blocks) for large problems
 #endif
@@ -655,6 +658,158 @@ spmm_gather_kernel(const MfmaParams p)
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Direct gather kernel for the high-sparsity layout: the same wave-private idea without LDS.  A
+// lane's MFMA operand for k-step s is 16 contiguous bytes of A row column_info[rank(2s+h)], so it
+// is loaded straight into the operand registers (128-bit loads, two 512-byte row segments per wave
+// and instruction), one window ahead.  No LDS, no barrier, and the only memory instructions left
+// are the operand loads themselves.
+template <int KS, int WS, int QS, int RM, bool HIGH>
+__global__ void __launch_bounds__(64 * QS, RM == 8 ? 2 : NMSPMM_OCC)
+spmm_direct_kernel(const MfmaParams p)
+{
+    static_assert(RM == 4 || RM == 8, "128- or 256-row waves");
+    typedef typename AFrag<RM>::type afrag_t;
+    constexpr int MS = RM * 32;
+    constexpr int NS = QS * 32;
+    constexpr int KSTEPS = WS / 2;
+    constexpr int ND = (WS * QS + 63) / 64;
+
+    const int total = p.tiles_m * p.tiles_n;
+    int logical;
+    {
+        const int id = blockIdx.x;
+        const int q = total / kXcds, r = total % kXcds;
+        const int xcd = id % kXcds, loc = id / kXcds;
+        logical = xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc;
+    }
+    constexpr int GROUP = NMSPMM_GROUP;
+    int tile_m, tile_n;
+    {
+        const int band = logical / (GROUP * p.tiles_n);
+        const int first_m = band * GROUP;
+        const int rows = min(GROUP, p.tiles_m - first_m);
+        const int in_band = logical - band * GROUP * p.tiles_n;
+        tile_m = first_m + in_band % rows;
+        tile_n = in_band / rows;
+    }
+    const int bi = tile_m * MS;
+    const int bj = tile_n * NS;
+    int w_begin, w_count;
+    split_windows(p.nwin, p.split_k, blockIdx.y, &w_begin, &w_count);
+    const int w_last = w_begin + w_count - 1;
+
+    const int lane = threadIdx.x & 63;
+    const int vec = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int h = lane >> 5;
+    const int j = lane & 31;
+    const int M = p.M, N = p.N;
+    const float* const Ablk = p.A + bi;
+    const float* const Bvec = p.B + bj + vec * 32;
+    const int32_t* const Dblk = p.D + (size_t)tile_n * p.W * QS;
+    const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)tile_n * p.nwin * KS : nullptr;
+    const uint32_t a_bytes = (uint32_t)(((size_t)(KS - 1) * M + (M - bi)) * sizeof(float));
+    const uint32_t b_bytes = (uint32_t)(((size_t)(WS - 1) * N + 32) * sizeof(float));
+    const uint32_t b_lane = (uint32_t)(((size_t)h * N + j) * sizeof(float));
+    const uint32_t b_step = (uint32_t)(2 * (size_t)N * sizeof(float));
+    const uint32_t row_bytes = (uint32_t)((size_t)M * sizeof(float));
+    const uint32_t a_vlane = (uint32_t)(j * 16);  // this lane's run of four rows inside the tile
+
+    int d_vec[ND], d_nxt[ND], ci_vec = -1, ci_nxt = -1;
+    auto load_meta = [&](int w) {
+        const __amdgpu_buffer_rsrc_t rd = make_rsrc(Dblk + (size_t)w * WS * QS, WS * QS * sizeof(int32_t));
+#pragma unroll
+        for (int q = 0; q < ND; ++q)
+            d_nxt[q] = __builtin_amdgcn_raw_buffer_load_b32(rd, (lane + 64 * q) * (int)sizeof(int32_t), 0, 0);
+        if constexpr (HIGH) {
+            const __amdgpu_buffer_rsrc_t rc = make_rsrc(Cinfo + (size_t)w * KS, KS * sizeof(int32_t));
+            ci_nxt = __builtin_amdgcn_raw_buffer_load_b32(rc, lane * (int)sizeof(int32_t), 0, 0);
+        }
+    };
+    auto take_meta = [&]() {
+#pragma unroll
+        for (int q = 0; q < ND; ++q)
+            d_vec[q] = d_nxt[q];
+        ci_vec = ci_nxt;
+    };
+    auto row_of = [&](int pp) -> int {
+        const int e = pp * QS;
+        const int rank = __builtin_amdgcn_readlane(d_vec[e / 64], e % 64 + vec);
+        if constexpr (!HIGH)
+            return rank;  // low-sparsity layout: the index is the window-local row itself
+        return __builtin_amdgcn_readlane(ci_vec, rank & 63);
+    };
+    floatx16 acc[RM];
+#pragma unroll
+    for (int b = 0; b < RM; ++b)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            acc[b][v] = 0.0f;
+
+    // Rolling register pipeline: the operands of k-step s are reloaded for the next window right
+    // after the MFMAs of k-step s have been issued, so every load has one whole window of MFMA work
+    // to land and the operands need a single set of registers.
+    afrag_t a_op[KSTEPS];
+    float b_op[KSTEPS];
+    uint32_t b_off[KSTEPS];
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s)
+        b_off[s] = b_lane + s * b_step;
+    auto load_step = [&](int s, __amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb) {
+        const int r0 = row_of(2 * s), r1 = row_of(2 * s + 1);
+        const uint32_t off = (uint32_t)(h ? r1 : r0) * row_bytes + a_vlane;
+        if constexpr (RM == 8) {
+            a_op[s].lo = buffer_load_f4(ra, off);
+            a_op[s].hi = buffer_load_f4(ra, off + 512);
+        } else {
+            a_op[s] = buffer_load_f4(ra, off);
+        }
+        b_op[s] = buffer_load_f1(rb, b_off[s], 0);
+    };
+    if (w_count > 0) {
+        load_meta(w_begin);
+        take_meta();
+        const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w_begin * KS * M, a_bytes);
+        const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)w_begin * WS * N, b_bytes);
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+            load_step(s, ra, rb);
+        load_meta(min(w_begin + 1, w_last));
+        take_meta();
+    }
+    for (int t = 0; t < w_count; ++t) {
+        const int w = w_begin + t;
+        const int wn = min(w + 1, w_last);
+        const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)wn * KS * M, a_bytes);
+        const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)wn * WS * N, b_bytes);
+        load_meta(min(w + 2, w_last));
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int b = 0; b < RM; ++b)
+                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_get(a_op[s], b), b_op[s], acc[b], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            load_step(s, ra, rb);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        take_meta();
+    }
+
+    float* out = p.out + (size_t)blockIdx.y * p.slice_elems;
+    const int col = bj + vec * 32 + j;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int r32 = 8 * (v / 4) + 4 * h + (v % 4);
+#pragma unroll
+        for (int b = 0; b < RM; ++b) {
+            const int row = bi + (b / 4) * 128 + r32 * 4 + (b % 4);
+            if (row < M)
+                out[(size_t)row * N + col] = acc[b][v];
+        }
+    }
+}
+
 template <int KS, int WS, int QS, int RM>
 static hipError_t launch_gather(const SpmmArgs& a)
 {
@@ -673,7 +828,34 @@ static hipError_t launch_gather(const SpmmArgs& a)
     p.tiles_m = (a.M + RM * 32 - 1) / (RM * 32);
     p.tiles_n = a.N / (QS * 32);
     dim3 grid(p.tiles_m * p.tiles_n, a.split_k, 1);
+#if NMSPMM_GATHER == 2
+    spmm_direct_kernel<KS, WS, QS, RM, true><<<grid, dim3(64 * QS), 0, a.stream>>>(p);
+#else
     spmm_gather_kernel<KS, WS, QS, RM><<<grid, dim3(64 * QS), 0, a.stream>>>(p);
+#endif
+    return hipGetLastError();
+}
+
+template <int KS, int WS, int QS, int RM>
+static hipError_t launch_direct_low(const SpmmArgs& a)
+{
+    constexpr int MS = RM * 32;
+    MfmaParams p;
+    p.A = a.A;
+    p.B = a.B;
+    p.D = a.D;
+    p.cinfo = nullptr;
+    p.out = a.split_k > 1 ? a.partial : a.C;
+    p.slice_elems = a.slice_stride;
+    p.M = a.M;
+    p.N = a.N;
+    p.W = a.W;
+    p.nwin = a.W / WS;
+    p.split_k = a.split_k;
+    p.tiles_m = (a.M + MS - 1) / MS;
+    p.tiles_n = a.N / (QS * 32);
+    dim3 grid(p.tiles_m * p.tiles_n, a.split_k, 1);
+    spmm_direct_kernel<KS, WS, QS, RM, false><<<grid, dim3(64 * QS), 0, a.stream>>>(p);
     return hipGetLastError();
 }
 
@@ -715,11 +897,23 @@ static hipError_t launch_ns(const SpmmArgs& a)
         switch (a.Ns) {
         case 128: {
             // 256-row waves only while two workgroups still fit a CU (64 KiB of LDS each)
+#if NMSPMM_GATHER == 2
+            constexpr int tall_rm = NMSPMM_GATHER_RM_TALL;
+#else
             constexpr int tall_rm = 2 * 4 * WS * 256 * (int)sizeof(float) <= 64 * 1024 ? NMSPMM_GATHER_RM_TALL : 4;
+#endif
             return tall ? launch_gather<KS, WS, 4, tall_rm>(a) : launch_gather<KS, WS, 4, 4>(a);
         }
         case 64: return launch_gather<KS, WS, 2, 4>(a);
         case 32: return launch_gather<KS, WS, 1, 4>(a);
+        }
+    }
+#endif
+#if NMSPMM_DIRECT_LOW
+    if constexpr (!HIGH && WS <= 16) {
+        if (a.Ns == 128) {
+            const bool tall = (long long)((a.M + 255) / 256) * (a.N / a.Ns) * a.split_k >= 2 * kCus;
+            return tall ? launch_direct_low<KS, WS, 4, NMSPMM_GATHER_RM_TALL>(a) : launch_direct_low<KS, WS, 4, 4>(a);
         }
     }
 #endif
