@@ -6,7 +6,7 @@ the baseline: M = Ncols = K = 4096, fp32, operands resident in HBM, at 2:4 (the 
 3:8, 2:8 and 1:8 (reported under "sweep").  Prints ONE JSON line:
 
   value            useful TFLOP/s at 2:4 = 2*M*Ncols*W / t   (W = K*n/m)
-  roofline         the dominant kernel (spmm_mfma_kernel at 2:4) against the fp32 MFMA peak
+  roofline         the dominant kernel (spmm_direct_kernel at 2:4) against the fp32 MFMA peak
   cpu_baseline     the reference project's own nmGEMM_on_cpu (oracle/_ref) on a row slice
   sweep            per pattern: ms, useful and dense-equivalent TFLOP/s, speedup over the dense
                    fp32 GEMM of the same shape (rocBLAS/hipBLASLt through torch.mm), and the GPU
@@ -229,7 +229,7 @@ def main():
                      # factors coming from a plain 256 MiB copy in the same runs
                      # (profiles/spmm_mfma_kernel_4096cubed_2of4.md)
                      "traffic": 652.4e6, "traffic_unit": "bytes per launch", "algorithmic_bytes": 168.8e6,
-                     "kernel": "spmm_mfma_kernel<32,16,4,...>", "flops_per_launch": case.useful_flops(),
+                     "kernel": "spmm_direct_kernel<32,16,4,1,8,false>", "flops_per_launch": case.useful_flops(),
                      "launch_ms_events": round(ms, 5), "launch_ms_wall": round(wall_ms, 5)},
         "cpu_baseline": cpu,
         "dense_fp32_gemm": None if dense_ms is None else {

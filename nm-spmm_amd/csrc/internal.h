@@ -33,7 +33,7 @@ __host__ __device__ inline void split_windows(int nwin, int split_k, int z, int*
     *count = z < q ? p + 1 : p;
 }
 
-// Matrix-core path (spmm_mfma.hip).  Returns false when the geometry has no instantiation.
+// Matrix-core path (spmm_direct.hip).  Returns false when the geometry has no instantiation.
 bool mfma_supported(const SpmmArgs& a);
 hipError_t launch_mfma(const SpmmArgs& a);
 
