@@ -21,8 +21,9 @@
 //    L1 and the L2: the tile walk keeps the workgroups resident on one XCD in a compact patch of C.
 //  * Index metadata arrives as one wave-wide load per window ([kept][Ns/32] ints, plus the
 //    column_info list of the window on the high-sparsity layout), two windows ahead, and is
-//    handed to the lanes with v_readlane: the row numbers become scalars, the per-lane select
-//    between the two halves is one v_cndmask.
+//    handed to the lanes that need it with ds_bpermute (the LDS crossbar, no LDS memory): one
+//    permute and one multiply-add per k-step form the per-lane row offset.  Vector ALU work in
+//    the loop is not free next to back-to-back MFMAs, so it is kept to that.
 //  * All loads go through buffer descriptors whose extent ends with the window's last row, so no
 //    lane reads outside A or B without a branch; lanes whose rows lie beyond M read zeros or
 //    other rows' values into accumulators that are never stored.
@@ -172,21 +173,34 @@ spmm_direct_kernel(const DirectParams p)
             d_vec[q] = d_nxt[q];
         ci_vec = ci_nxt;
     };
-    // window-local dense row of kept row pp of this wave's vector (a scalar)
-    auto row_of = [&](int pp) -> int {
-        const int e = pp * QS;
-        const int idx = __builtin_amdgcn_readlane(d_vec[e / 64], e % 64 + vec);
-        if constexpr (!HIGH)
-            return idx;
-        return __builtin_amdgcn_readlane(ci_vec, idx & 63);
+    // Byte offsets of this lane's A operands for the CS k-steps of chunk c of the window whose
+    // metadata is in d_vec / ci_vec: lane half h of k-step s needs the dense row that index entry
+    // (c*CH + 2s + h) * QS + vec selects.  ds_bpermute fetches that entry from the lane holding it
+    // (a crossbar read, no LDS memory involved).  On the high-sparsity layout the entries are
+    // ranks into the window's column_info list; resolve_ranks() turns all of them into rows with
+    // one more permute per window.
+    const int perm_addr = (h * QS + vec) * (int)sizeof(int32_t);
+    uint32_t a_off[CS];
+    auto resolve_ranks = [&]() {
+        if constexpr (HIGH) {
+            static_assert(!HIGH || ND == 1, "one register of ranks per window");
+            d_vec[0] = __builtin_amdgcn_ds_bpermute(d_vec[0] << 2, ci_vec);
+        }
+    };
+    auto form_offsets = [&](int c) {
+#pragma unroll
+        for (int s = 0; s < CS; ++s) {
+            const int e = (c * CH + 2 * s) * QS;
+            const int row = __builtin_amdgcn_ds_bpermute(perm_addr + (e % 64) * (int)sizeof(int32_t), d_vec[e / 64]);
+            a_off[s] = __umul24((uint32_t)row, row_bytes) + a_vlane;
+        }
     };
 
     afrag_t a_op[CS];
     float b_op[CS];
     // operands of k-step s of chunk c of the window the descriptors point at
     auto load_step = [&](int c, int s, __amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb) {
-        const int r0 = row_of(c * CH + 2 * s), r1 = row_of(c * CH + 2 * s + 1);
-        const uint32_t off = (uint32_t)(h ? r1 : r0) * row_bytes + a_vlane;
+        const uint32_t off = a_off[s];
         if constexpr (RM == 8) {
             a_op[s].lo = buffer_load_f4(ra, off);
             a_op[s].hi = buffer_load_f4(ra, off + 512);
@@ -206,6 +220,8 @@ spmm_direct_kernel(const DirectParams p)
     if (w_count > 0) {
         load_meta(w_begin);
         take_meta();
+        resolve_ranks();
+        form_offsets(0);
         const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w_begin * KS * M, a_bytes);
         const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)w_begin * WS * N, b_bytes);
 #pragma unroll
@@ -223,10 +239,12 @@ spmm_direct_kernel(const DirectParams p)
             if (wrap) {
                 __builtin_amdgcn_sched_barrier(0);
                 take_meta();
+                resolve_ranks();
                 load_meta(min(w + 2, w_last));
             }
             const int wl = wrap ? wn : w;
             const int cl = wrap ? 0 : c + 1;
+            form_offsets(cl);
             const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)wl * KS * M, a_bytes);
             const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)wl * WS * N, b_bytes);
 #pragma unroll
@@ -306,8 +324,11 @@ bool mfma_supported(const SpmmArgs& a)
         return false;
     if (a.M % 4 != 0 || a.M < 32)
         return false;
-    // 32-bit buffer offsets: one window of A and one window of B must stay below 2 GiB
+    // 32-bit buffer offsets: one window of A and one window of B must stay below 2 GiB; the row
+    // offset of A is formed with a 24-bit multiply
     if ((size_t)a.window * a.M * sizeof(float) >= 0x80000000ull || (size_t)a.kept * a.N * sizeof(float) >= 0x80000000ull)
+        return false;
+    if ((size_t)a.M * sizeof(float) >= (1u << 24))
         return false;
     const bool high = a.cinfo != nullptr;
     if (!high)
