@@ -260,17 +260,21 @@ spmm_direct_kernel(const DirectParams p)
     }
 
     // ---- epilogue: MFMA result register v of lane (h, j) is row 8*(v/4) + 4*h + v%4 of the block,
-    // column j; block b of the wave holds rows (b/4)*128 + 4*r + b%4
-    float* out = p.out + (size_t)blockIdx.y * p.slice_elems;
-    const int col = bj + j;
+    // column j; block b of the wave holds rows (b/4)*128 + 4*r + b%4.  Stores go through a
+    // descriptor that ends with the last live row of this wave, so rows beyond M are dropped
+    // without a branch; the per-register part of the offset is a scalar.
+    float* const out = p.out + (size_t)blockIdx.y * p.slice_elems;
+    const int rows_here = min(M - bi, MW);
+    const uint32_t c_bytes = rows_here > 0 ? (uint32_t)(((size_t)(rows_here - 1) * N + 32) * sizeof(float)) : 0u;
+    const __amdgpu_buffer_rsrc_t rc = make_rsrc(out + (size_t)min(bi, M) * N + bj, c_bytes);
+    const uint32_t c_lane = (uint32_t)(((size_t)16 * h * N + j) * sizeof(float));
+    const uint32_t n_bytes = (uint32_t)((size_t)N * sizeof(float));
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-        const int r32 = 8 * (v / 4) + 4 * h + (v % 4);
 #pragma unroll
         for (int b = 0; b < RM; ++b) {
-            const int row = bi + (b / 4) * 128 + r32 * 4 + (b % 4);
-            if (row < M)
-                out[(size_t)row * N + col] = acc[b][v];
+            const uint32_t row = (b / 4) * 128 + 32 * (v / 4) + 4 * (v % 4) + (b % 4);  // without the lane's 16*h
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_int(acc[b][v]), rc, c_lane + row * n_bytes, 0, 0);
         }
     }
 }
@@ -329,6 +333,9 @@ bool mfma_supported(const SpmmArgs& a)
     if ((size_t)a.window * a.M * sizeof(float) >= 0x80000000ull || (size_t)a.kept * a.N * sizeof(float) >= 0x80000000ull)
         return false;
     if ((size_t)a.M * sizeof(float) >= (1u << 24))
+        return false;
+    // a wave's 256 rows of C are addressed with 32-bit offsets
+    if ((size_t)256 * a.N * sizeof(float) >= 0x80000000ull)
         return false;
     const bool high = a.cinfo != nullptr;
     if (!high)
