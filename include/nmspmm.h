@@ -94,6 +94,23 @@ int nmspmm_preprocess_high_device(int32_t* d_column_info, int pruning_M, int pru
  * library neither needs nor touches it.)  Returns 0 for invalid arguments. */
 size_t nmspmm_column_info_ints(int W, int pruning_N, int pruning_M, int N, int Ns);
 
+/* ---- dense <-> compressed operand ---------------------------------------------------------- */
+
+/* No counterpart in the reference, which only synthesises operands that are already compressed
+ * (reference include/utils.h:40-64); these produce and expand exactly that format.
+ * nmspmm_compress_device: dB is the dense row-major float[K][N] operand.  In every window of m rows
+ * and every vector of vec_len columns the n rows with the largest sum of |b| (added pairwise in
+ * fp32: neighbours at distance 1, then 2, 4, ...; equal sums prefer the lower row) are kept:
+ * dBT[W][N] receives their values, dDT[W][N/vec_len] their window-local row numbers, ascending,
+ * W = K*n/m.  The output is what the preprocessing entry points above take.
+ * nmspmm_decompress_device is the inverse (dropped rows become zero).
+ * Requirements: m in {4, 8, 16, 32}, 0 < n < m, vec_len in {4, 8, 16, 32}, K % m == 0,
+ * N % vec_len == 0, 16-byte aligned dB and dBT.  Asynchronous on `stream`. */
+int nmspmm_compress_device(const float* dB, int K, int N, int n, int m, int vec_len, float* dBT,
+                           int32_t* dDT, void* stream);
+int nmspmm_decompress_device(const float* dBT, const int32_t* dDT, int K, int N, int n, int m,
+                             int vec_len, float* dB, void* stream);
+
 /* ---- multiplication ----------------------------------------------------------------------- */
 
 /* Bytes of device workspace nmspmm_spmm needs for a given split_k (0 when split_k <= 1):

@@ -50,6 +50,8 @@ def lib():
         L.nmspmm_preprocess_low_device.argtypes = [c_void_p, c_void_p] + [c_int] * 4 + [c_void_p]
         L.nmspmm_preprocess_high_host.argtypes = [c_void_p, c_int, c_int, c_void_p] + [c_int] * 5
         L.nmspmm_preprocess_high_device.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p] + [c_int] * 5 + [c_void_p]
+        L.nmspmm_compress_device.argtypes = [c_void_p] + [c_int] * 5 + [c_void_p, c_void_p, c_void_p]
+        L.nmspmm_decompress_device.argtypes = [c_void_p, c_void_p] + [c_int] * 5 + [c_void_p, c_void_p]
         L.nmspmm_column_info_ints.restype = c_size_t
         L.nmspmm_column_info_ints.argtypes = [c_int] * 5
         L.nmspmm_workspace_bytes.restype = c_size_t
@@ -105,6 +107,17 @@ def preprocess_high_device(d_cinfo, pM, pN, dDT_in, dDT_out, W, Q, N, Ns, vec_le
     _check("nmspmm_preprocess_high_device",
            lib().nmspmm_preprocess_high_device(_ptr(d_cinfo), pM, pN, _ptr(dDT_in), _ptr(dDT_out), W, Q, N, Ns,
                                                vec_len, _stream()))
+
+
+def compress_device(dB, K, N, n, m, dBT, dDT, vec_len=32):
+    """Dense row-major float32[K][N] on the GPU -> BT float32[K*n/m][N], DT int32[K*n/m][N/vec_len]."""
+    _check("nmspmm_compress_device",
+           lib().nmspmm_compress_device(_ptr(dB), K, N, n, m, vec_len, _ptr(dBT), _ptr(dDT), _stream()))
+
+
+def decompress_device(dBT, dDT, K, N, n, m, dB, vec_len=32):
+    _check("nmspmm_decompress_device",
+           lib().nmspmm_decompress_device(_ptr(dBT), _ptr(dDT), K, N, n, m, vec_len, _ptr(dB), _stream()))
 
 
 def column_info_ints(W, pN, pM, N, Ns):

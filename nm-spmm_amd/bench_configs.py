@@ -3,7 +3,7 @@
 square sweep): LLM-layer shapes, decode-sized M, and the fine-grained / short-vector patterns.
 Prints one markdown table row per case.
 
-    python nm-spmm_amd/bench_configs.py [llm] [decode] [fine]
+    python nm-spmm_amd/bench_configs.py [llm] [decode] [fine] [compress]
 
 useful TFLOP/s = 2*M*Ncols*W / t; GB/s = algorithmic bytes
 4*(M*K + W*Ncols + W*Ncols/L + M*Ncols) (+ column_info) / t.
@@ -144,9 +144,27 @@ def fine():
         del op
 
 
+def compress():
+    print("| op | K x Ncols | pattern | us | GB/s (algorithmic) | of 8 TB/s |")
+    print("|---|---|---|---|---|---|")
+    for (K, N) in ((4096, 4096), (11008, 4096), (8192, 8192)):
+        dense = torch.randn((K, N), dtype=torch.float32, device="cuda")
+        for (n, m) in ((2, 4), (2, 8), (1, 8), (8, 32)):
+            W, Q = K // m * n, N // 32
+            BT = torch.empty((W, N), dtype=torch.float32, device="cuda")
+            DT = torch.empty((W, Q), dtype=torch.int32, device="cuda")
+            back = torch.empty_like(dense)
+            nbytes = 4.0 * (K * N + W * N + W * Q)
+            for name, fn in (("compress", lambda: pkg.compress_device(dense, K, N, n, m, BT, DT)),
+                             ("decompress", lambda: pkg.decompress_device(BT, DT, K, N, n, m, back))):
+                ms = timed(fn)
+                print("| %s | %dx%d | %d:%d | %.1f | %.0f | %.3f |" % (name, K, N, n, m, ms * 1e3, nbytes / ms / 1e6,
+                                                                    nbytes / ms / 1e6 / 8000), flush=True)
+
+
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["llm", "decode", "fine"]
+    which = sys.argv[1:] or ["llm", "decode", "fine", "compress"]
     pkg.lib()
     for name in which:
         print("\n### %s" % name)
-        {"llm": llm, "decode": decode, "fine": fine}[name]()
+        {"llm": llm, "decode": decode, "fine": fine, "compress": compress}[name]()

@@ -261,6 +261,39 @@ int nmspmm_preprocess_high_host(int32_t* column_info, int pruning_M, int pruning
 
 /* ---- multiplication ------------------------------------------------------------------------ */
 
+static int check_compress(const void* dense, const void* bt, const void* dt, int K, int N, int n, int m, int vec_len)
+{
+    if (!dense || !bt || !dt)
+        return NMSPMM_ERR_NULL_POINTER;
+    if (((uintptr_t)dense | (uintptr_t)bt) & 15u)
+        return NMSPMM_ERR_ALIGNMENT;
+    if (!compress_supported(m, vec_len) || n <= 0 || n >= m)
+        return NMSPMM_ERR_BAD_PATTERN;
+    if (K <= 0 || N <= 0 || K % m != 0 || N % vec_len != 0 || (N + 1023) / 1024 > 65535)
+        return NMSPMM_ERR_BAD_SHAPE;
+    return NMSPMM_OK;
+}
+
+int nmspmm_compress_device(const float* dB, int K, int N, int n, int m, int vec_len, float* dBT, int32_t* dDT,
+                           void* stream)
+{
+    const int st = check_compress(dB, dBT, dDT, K, N, n, m, vec_len);
+    if (st != NMSPMM_OK)
+        return st;
+    return launch_compress(dB, dBT, dDT, K, N, n, m, vec_len, (hipStream_t)stream) == hipSuccess ? NMSPMM_OK
+                                                                                                   : NMSPMM_ERR_HIP;
+}
+
+int nmspmm_decompress_device(const float* dBT, const int32_t* dDT, int K, int N, int n, int m, int vec_len,
+                             float* dB, void* stream)
+{
+    const int st = check_compress(dB, dBT, dDT, K, N, n, m, vec_len);
+    if (st != NMSPMM_OK)
+        return st;
+    return launch_decompress(dBT, dDT, dB, K, N, n, m, vec_len, (hipStream_t)stream) == hipSuccess ? NMSPMM_OK
+                                                                                                     : NMSPMM_ERR_HIP;
+}
+
 size_t nmspmm_workspace_bytes(int M, int N, int split_k)
 {
     if (M <= 0 || N <= 0 || split_k <= 1)

@@ -1,0 +1,143 @@
+// Compression of a dense operand to the N:M vector-sparse format and back.  The reference only
+// synthesises operands that are already compressed (include/utils.h:40-64); these kernels produce
+// and expand exactly that format: BT row-major float[W][N] (W = K*n/m kept rows), DT row-major
+// int32[W][Q] of window-local row numbers, one per kept row and L-column vector.
+//
+// Selection rule: in every window of m rows and every vector of L columns, the score of a row is
+// the sum of |b| over the vector's L columns, added pairwise in fp32 (neighbours at distance 1,
+// then 2, 4, ... L/2); the n rows with the largest scores are kept, equal scores prefer the lower
+// row; scores are ordered by their bit patterns, so NaNs rank above everything instead of
+// breaking the order.  Both kernels are HBM-bound: every global access is a coalesced run of
+// 16-byte segments of one row.
+#include "internal.h"
+
+namespace nmspmm {
+
+// One thread owns four adjacent columns (a 16-byte segment of every row), so a vector of L columns
+// is a group of L/4 lanes: the first two levels of the pairwise sum happen inside the thread, the
+// remaining ones by lane exchange.
+constexpr int kColsPerBlock = 1024;
+
+template <int MW>
+__global__ void __launch_bounds__(256)
+compress_kernel(const float* __restrict__ B, float* __restrict__ BT, int32_t* __restrict__ DT, int N, int Q,
+                int n, int L)
+{
+    const int w = blockIdx.x;
+    const int col = blockIdx.y * kColsPerBlock + threadIdx.x * 4;
+    const bool active = col < N;  // whole vectors are active or not: N and 1024 are multiples of L
+    const int lane = threadIdx.x & 63;
+    const int G = L / 4;                // lanes per vector
+    const int c = lane & (G - 1);       // position inside the group
+    const int group = lane & ~(G - 1);  // first lane of the group
+
+    float4 v[MW];
+    uint32_t key[MW];
+#pragma unroll
+    for (int r = 0; r < MW; ++r)
+        v[r] = active ? *reinterpret_cast<const float4*>(B + ((size_t)w * MW + r) * N + col)
+                      : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+    for (int r = 0; r < MW; ++r) {
+        float s = (fabsf(v[r].x) + fabsf(v[r].y)) + (fabsf(v[r].z) + fabsf(v[r].w));
+        for (int mask = 1; mask < G; mask <<= 1)
+            s += __shfl_xor(s, mask, 64);
+        key[r] = __float_as_uint(s);
+    }
+
+    // Lane c of the group ranks rows c, c + G, ...; a ballot hands the verdicts to the whole group.
+    uint32_t keep = 0;
+    for (int t = 0; t * G < MW; ++t) {
+        const int mine = c + t * G;
+        uint32_t key_mine = 0;
+#pragma unroll
+        for (int r = 0; r < MW; ++r)
+            key_mine = r == mine ? key[r] : key_mine;
+        int rank = 0;
+#pragma unroll
+        for (int r = 0; r < MW; ++r)
+            rank += (key[r] > key_mine || (key[r] == key_mine && r < mine)) ? 1 : 0;
+        const unsigned long long votes = __ballot(mine < MW && rank < n);
+        const uint32_t bits = (uint32_t)(votes >> group) & ((1u << G) - 1u);
+        keep |= bits << (t * G);
+    }
+
+    if (!active)
+        return;
+    const int a = col / L;
+#pragma unroll
+    for (int r = 0; r < MW; ++r) {
+        if ((keep >> r) & 1u) {
+            const int p = __popc(keep & ((1u << r) - 1u));
+            const size_t row = (size_t)w * n + p;
+            *reinterpret_cast<float4*>(BT + row * N + col) = v[r];
+            if (c == (r & (G - 1)))
+                DT[row * Q + a] = r;
+        }
+    }
+}
+
+template <int MW>
+__global__ void __launch_bounds__(256)
+decompress_kernel(const float* __restrict__ BT, const int32_t* __restrict__ DT, float* __restrict__ B, int N,
+                  int Q, int n, int L)
+{
+    const int w = blockIdx.x;
+    const int col = blockIdx.y * kColsPerBlock + threadIdx.x * 4;
+    if (col >= N)
+        return;
+    const int a = col / L;
+    uint32_t keep = 0;
+    for (int p = 0; p < n; ++p) {
+        const uint32_t r = (uint32_t)DT[((size_t)w * n + p) * Q + a];
+        if (r < (uint32_t)MW)  // malformed indices must not leave the window
+            keep |= 1u << r;
+    }
+    // every row of the window is written exactly once: a kept row's values or zeros
+#pragma unroll
+    for (int r = 0; r < MW; ++r) {
+        float4 x = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if ((keep >> r) & 1u) {
+            const int p = __popc(keep & ((1u << r) - 1u));
+            x = *reinterpret_cast<const float4*>(BT + ((size_t)w * n + p) * N + col);
+        }
+        *reinterpret_cast<float4*>(B + ((size_t)w * MW + r) * N + col) = x;
+    }
+}
+
+bool compress_supported(int m, int vec_len)
+{
+    return (m == 4 || m == 8 || m == 16 || m == 32) && (vec_len == 4 || vec_len == 8 || vec_len == 16 || vec_len == 32);
+}
+
+hipError_t launch_compress(const float* B, float* BT, int32_t* DT, int K, int N, int n, int m, int vec_len,
+                           hipStream_t stream)
+{
+    const dim3 grid(K / m, (N + kColsPerBlock - 1) / kColsPerBlock), block(256);
+    const int Q = N / vec_len;
+    switch (m) {
+    case 4: compress_kernel<4><<<grid, block, 0, stream>>>(B, BT, DT, N, Q, n, vec_len); break;
+    case 8: compress_kernel<8><<<grid, block, 0, stream>>>(B, BT, DT, N, Q, n, vec_len); break;
+    case 16: compress_kernel<16><<<grid, block, 0, stream>>>(B, BT, DT, N, Q, n, vec_len); break;
+    case 32: compress_kernel<32><<<grid, block, 0, stream>>>(B, BT, DT, N, Q, n, vec_len); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_decompress(const float* BT, const int32_t* DT, float* B, int K, int N, int n, int m, int vec_len,
+                             hipStream_t stream)
+{
+    const dim3 grid(K / m, (N + kColsPerBlock - 1) / kColsPerBlock), block(256);
+    const int Q = N / vec_len;
+    switch (m) {
+    case 4: decompress_kernel<4><<<grid, block, 0, stream>>>(BT, DT, B, N, Q, n, vec_len); break;
+    case 8: decompress_kernel<8><<<grid, block, 0, stream>>>(BT, DT, B, N, Q, n, vec_len); break;
+    case 16: decompress_kernel<16><<<grid, block, 0, stream>>>(BT, DT, B, N, Q, n, vec_len); break;
+    case 32: decompress_kernel<32><<<grid, block, 0, stream>>>(BT, DT, B, N, Q, n, vec_len); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+} // namespace nmspmm

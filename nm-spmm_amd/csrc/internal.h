@@ -55,5 +55,12 @@ hipError_t launch_reblock(const int32_t* in, int32_t* out, int W, int Q, int Qs,
 hipError_t launch_preprocess_high(int32_t* cinfo, int pM, int pN, const int32_t* in, int32_t* out,
                                   int W, int Q, int Qs, hipStream_t stream);
 
+// Dense <-> N:M vector-sparse conversion (compress.hip): m in {4, 8, 16, 32}, vec_len in {4, 8, 16, 32}.
+bool compress_supported(int m, int vec_len);
+hipError_t launch_compress(const float* B, float* BT, int32_t* DT, int K, int N, int n, int m, int vec_len,
+                           hipStream_t stream);
+hipError_t launch_decompress(const float* BT, const int32_t* DT, float* B, int K, int N, int n, int m, int vec_len,
+                             hipStream_t stream);
+
 } // namespace nmspmm
 #endif

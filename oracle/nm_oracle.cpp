@@ -12,6 +12,8 @@
 //   nm_oracle_preprocess_high  sorted(set()) brute force, gather round trip + oracle/_ref
 //   nm_oracle_gemm_cpu         dense fp64 GEMM of the decompressed operand + oracle/_ref (bit-exact)
 //   nm_oracle_decompress       scatter/gather round trip
+//   nm_oracle_compress         recovers generated (BT, DT) from their dense expansion, fp64 score
+//                              dominance of kept over dropped rows, constructed ties, sign symmetry
 // No function here is "parity unpinned".
 //
 // Vocabulary (reference include/utils.h:10-66, include/NM-SpMM.h:8):
@@ -163,6 +165,46 @@ void nm_oracle_decompress(const float* B, const int32_t* D, float* dense, int K,
         const int a = j / vec_len;
         for (int k = 0; k < W; ++k)
             dense[(size_t)D[(size_t)k + (size_t)a * W] * N + j] = B[(size_t)k + (size_t)j * W];
+    }
+}
+
+// Compresses a dense row-major float[K][N] operand to the format of include/utils.h:40-64 (BT
+// row-major float[W][N], DT row-major int32[W][Q] window-local, ascending inside a window).  The
+// reference has no such function; the rule restated here is the library's: per window of m rows
+// and vector of vec_len columns, score(row) = sum of |b| over the vector, added pairwise in fp32
+// (distance 1, 2, 4, ...), keep the n largest, ties to the lower row, scores ordered by bit
+// pattern.
+void nm_oracle_compress(const float* dense, int K, int N, int n, int m, int vec_len, float* BT, int32_t* DT)
+{
+    const int Q = N / vec_len;
+    const int nwin = K / m;
+#pragma omp parallel for schedule(static)
+    for (int w = 0; w < nwin; ++w) {
+        std::vector<float> part(vec_len);
+        std::vector<uint32_t> key(m);
+        std::vector<int> order(m);
+        for (int a = 0; a < Q; ++a) {
+            for (int r = 0; r < m; ++r) {
+                const float* src = dense + ((size_t)w * m + r) * N + (size_t)a * vec_len;
+                for (int c = 0; c < vec_len; ++c)
+                    part[c] = src[c] < 0 ? -src[c] : src[c];
+                for (int width = vec_len; width > 1; width /= 2)  // pairwise: (0,1) (2,3) ... then pairs of pairs
+                    for (int c = 0; c < width / 2; ++c) {
+                        volatile float t = part[2 * c] + part[2 * c + 1];
+                        part[c] = t;
+                    }
+                std::memcpy(&key[r], &part[0], sizeof(uint32_t));
+                order[r] = r;
+            }
+            std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return key[x] > key[y]; });
+            std::sort(order.begin(), order.begin() + n);
+            for (int p = 0; p < n; ++p) {
+                const size_t row = (size_t)w * n + p;
+                DT[row * Q + a] = order[p];
+                const float* src = dense + ((size_t)w * m + order[p]) * N + (size_t)a * vec_len;
+                std::memcpy(BT + row * N + (size_t)a * vec_len, src, sizeof(float) * vec_len);
+            }
+        }
     }
 }
 

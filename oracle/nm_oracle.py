@@ -44,7 +44,8 @@ class Oracle:
         lib.nm_oracle_preprocess_high.argtypes = [_i32p, _int, _int, _i32p, _int, _int, _int, _int]
         lib.nm_oracle_gemm_cpu.argtypes = [_f32p, _f32p, _i32p, _f32p] + [_int] * 6
         lib.nm_oracle_decompress.argtypes = [_f32p, _i32p, _f32p] + [_int] * 4
-        for f in ("trans_index", "preprocess_low", "preprocess_high", "gemm_cpu", "decompress"):
+        lib.nm_oracle_compress.argtypes = [_f32p] + [_int] * 5 + [_f32p, _i32p]
+        for f in ("trans_index", "preprocess_low", "preprocess_high", "gemm_cpu", "decompress", "compress"):
             getattr(lib, "nm_oracle_" + f).restype = None
         self.lib = lib
 
@@ -79,6 +80,17 @@ class Oracle:
         dense = np.empty(K * N, np.float32)
         self.lib.nm_oracle_decompress(B, D, dense, K, N, W, vec_len)
         return dense.reshape(K, N)
+
+
+    def compress(self, dense, n, m, vec_len=32):
+        """dense row-major float32[K][N] -> (BT float32[W][N], DT int32[W][N/vec_len])."""
+        K, N = dense.shape
+        W = K // m * n
+        BT = np.empty((W, N), np.float32)
+        DT = np.empty((W, N // vec_len), np.int32)
+        self.lib.nm_oracle_compress(np.ascontiguousarray(dense, np.float32).reshape(-1), K, N, n, m, vec_len,
+                                    BT.reshape(-1), DT.reshape(-1))
+        return BT, DT
 
 
 class Reference:

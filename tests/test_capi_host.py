@@ -111,6 +111,16 @@ def test_preprocess_rejects_bad_arguments_without_a_gpu():
     assert L.nmspmm_status_string(4).decode().startswith("sparsity belongs")
 
 
+def test_compress_rejects_bad_arguments_without_a_gpu():
+    L = nmspmm.lib()
+    assert L.nmspmm_compress_device(None, 64, 64, 2, 4, 32, FAKE, FAKE, None) == 1
+    assert L.nmspmm_compress_device(FAKE, 64, 64, 4, 4, 32, FAKE, FAKE, None) == 3   # n == m
+    assert L.nmspmm_compress_device(FAKE, 64, 64, 2, 64, 32, FAKE, FAKE, None) == 3  # window not instantiated
+    assert L.nmspmm_compress_device(FAKE, 66, 64, 2, 4, 32, FAKE, FAKE, None) == 2   # K % m
+    assert L.nmspmm_decompress_device(FAKE, None, 64, 64, 2, 4, 32, FAKE, None) == 1
+    assert L.nmspmm_decompress_device(FAKE, FAKE, 64, 40, 2, 4, 32, FAKE, None) == 2  # N % vec_len
+
+
 def test_split_rule_matches_reference_partition():
     """The reference kernels give the first (windows % SPLIT_K) slices one extra window
     (src/kernel_64x128_8x8.cu:20-37, '20 tasks over 8 slices: 3 3 3 3 2 2 2 2')."""
