@@ -1,7 +1,7 @@
 // Decode-sized multiplication (M <= 32): the product is bound by streaming B from HBM once, so
 // the design goal is bytes in flight, not arithmetic.
 //
-//  * One workgroup per 32-column index vector; its NWV waves split the reduction (the windows of
+//  * One workgroup per 32-column index vector; its waves split the reduction (the windows of
 //    the compressed K dimension) between them and sum their partial 32 x 32 results through LDS
 //    in wave order, so the result is deterministic and needs no workspace or second launch.
 //  * No LDS staging and no barrier in the streaming loop: each lane loads its own MFMA operands,
@@ -10,7 +10,7 @@
 //    windows ahead of the v_mfma_f32_32x32x2_f32 that consumes them; rows i >= M are
 //    out-of-range loads that return zero.
 //  * Index metadata comes as one wave-wide load per window ([kept][Ns/32] ints, plus the 64-entry
-//    column_info list on the high-sparsity layout) and is handed to the lanes with readlane.
+//    column_info list on the high-sparsity layout) and is handed to the lanes with ds_bpermute.
 #include "internal.h"
 
 namespace nmspmm {
@@ -37,7 +37,7 @@ __device__ inline float sk_load(__amdgpu_buffer_rsrc_t r, uint32_t off)
 }
 
 #ifndef NMSPMM_SK_WAVES
-#define NMSPMM_SK_WAVES 16
+#define NMSPMM_SK_WAVES 8
 #endif
 #ifndef NMSPMM_SK_UMUL
 #define NMSPMM_SK_UMUL 1
@@ -121,23 +121,27 @@ spmm_skinny_kernel(const SkinnyParams p)
                 b_nxt[u * KSTEPS + s] = sk_load(rb, boff);
         }
     };
-    // A operands of the same windows, from the metadata currently in dvec / civec
+    // A operands of the same windows, from the metadata currently in dvec / civec.  Lane half h of
+    // k-step s needs the dense row that index entry (2s + h) * QS + vec selects: ds_bpermute
+    // fetches it from the lane that holds it (no LDS memory involved); on the high-sparsity layout
+    // one more permute per window first turns all ranks into rows.
+    const int perm_addr = (h * QS + vec) * (int)sizeof(int32_t);
+    const uint32_t row_bytes = (uint32_t)((size_t)M * sizeof(float));
     auto load_a = [&](int w) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int wu = w + u;
             const __amdgpu_buffer_rsrc_t ra_u = sk_rsrc(p.A, wu < w_end ? a_bytes : 0u);
+            const uint32_t win_row = (uint32_t)(min(wu, p.nwin - 1) * KS);
+            if (HIGH) {
+                static_assert(!HIGH || ND == 1, "one register of ranks per window");
+                dvec[u][0] = __builtin_amdgcn_ds_bpermute(dvec[u][0] << 2, civec[u]);
+            }
 #pragma unroll
             for (int s = 0; s < KSTEPS; ++s) {
-                const int e0 = 2 * s * QS, e1 = (2 * s + 1) * QS;
-                int lo = __builtin_amdgcn_readlane(dvec[u][e0 / 64], e0 % 64 + vec);
-                int hi = __builtin_amdgcn_readlane(dvec[u][e1 / 64], e1 % 64 + vec);
-                if (HIGH) {
-                    lo = __builtin_amdgcn_readlane(civec[u], lo & 63);
-                    hi = __builtin_amdgcn_readlane(civec[u], hi & 63);
-                }
-                const int k = min(wu, p.nwin - 1) * KS + (h ? hi : lo);
-                a_nxt[u * KSTEPS + s] = sk_load(ra_u, a_lane + (uint32_t)((size_t)k * M * sizeof(float)));
+                const int e = 2 * s * QS;
+                const int row = __builtin_amdgcn_ds_bpermute(perm_addr + (e % 64) * (int)sizeof(int32_t), dvec[u][e / 64]);
+                a_nxt[u * KSTEPS + s] = sk_load(ra_u, a_lane + (win_row + (uint32_t)row) * row_bytes);
             }
         }
     };
