@@ -61,4 +61,12 @@ void nmGEMM_small_matrices_low_sparsity(float* A, float* B, int* D, float* C,
 void nmGEMM_small_matrices_high_sparsity(float* A, float* B, int* D, int* column_info, float* C,
                                          int M, int N, int K, int W, float sparsity, int SPLIT_K);
 
+// ---- one launcher that chooses for the caller ----------------------------------------------------
+// No counterpart in the reference, whose callers pick the tile and SPLIT_K by timing all of them
+// (benchmark/kernel_performance/run_test/nmspmm/run_nmspmm.sh:19-36).  Indices must have been
+// preprocessed for Ns = 128; the sparsity selects the low- or high-sparsity layout (column_info
+// may be null for the former); the split of the reduction is chosen from the shape.
+void nmGEMM(float* A, float* B, int* D, int* column_info, float* C,
+            int M, int N, int K, int W, float sparsity);
+
 #endif // NM_SPMM_DROP_IN_H

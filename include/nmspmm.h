@@ -141,6 +141,19 @@ int nmspmm_gemm_high_sparsity(int tile, const float* A, const float* B, const in
                               const int32_t* column_info, float* C, int M, int N, int K, int W,
                               float sparsity, int split_k, void* stream);
 
+/* No counterpart in the reference, which leaves tile and SPLIT_K to the caller and finds them by
+ * exhaustive timing (benchmark/kernel_performance/run_test/nmspmm/run_nmspmm.sh:19-36,
+ * benchmark/different_kernel/search_shape/search_shape.sh:16-43).  On this hardware the
+ * column-block width does not change the speed (waves are independent), so only the split is
+ * chosen: nmspmm_suggest_split_k returns the split_k the library would use for a shape (1..16;
+ * 0 for invalid arguments); nmspmm_gemm_auto multiplies with that choice and the per-device
+ * workspace, for indices preprocessed with Ns = 128 (NMSPMM_TILE_HUGE); `sparsity` selects the
+ * geometry and the layout as nmspmm_pattern_from_sparsity does, column_info is required for the
+ * high-sparsity layout and ignored otherwise. */
+int nmspmm_suggest_split_k(int M, int N, int W, int kept);
+int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int32_t* column_info,
+                     float* C, int M, int N, int K, int W, float sparsity, void* stream);
+
 /* Frees the cached split-K workspaces of every device. */
 int nmspmm_release(void);
 

@@ -59,6 +59,8 @@ def lib():
         L.nmspmm_spmm.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, c_void_p]
         L.nmspmm_gemm_low_sparsity.argtypes = [c_int] + [c_void_p] * 4 + [c_int] * 4 + [c_float, c_int, c_void_p]
         L.nmspmm_gemm_high_sparsity.argtypes = [c_int] + [c_void_p] * 5 + [c_int] * 4 + [c_float, c_int, c_void_p]
+        L.nmspmm_suggest_split_k.argtypes = [c_int] * 4
+        L.nmspmm_gemm_auto.argtypes = [c_void_p] * 5 + [c_int] * 4 + [c_float, c_void_p]
         L.nmspmm_release.restype = c_int
         _lib = L
     return _lib
@@ -148,6 +150,16 @@ def gemm_high_sparsity(tile, A, B, D, cinfo, C, M, N, K, W, sparsity, split_k=1)
 
 
 # ---- host-pointer forms: arguments are C-contiguous numpy int32 arrays, updated in place ----------
+
+def suggest_split_k(M, N, W, kept):
+    return lib().nmspmm_suggest_split_k(M, N, W, kept)
+
+
+def gemm_auto(A, B, D, cinfo, C, M, N, K, W, sparsity):
+    """Multiply with the library's own choice of split_k (indices preprocessed for Ns = 128)."""
+    _check("nmspmm_gemm_auto",
+           lib().nmspmm_gemm_auto(_ptr(A), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(C), M, N, K, W, sparsity, _stream()))
+
 
 def _np_ptr(a):
     return ctypes.c_void_p(a.ctypes.data)

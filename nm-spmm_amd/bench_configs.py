@@ -99,23 +99,25 @@ def dense_ms(M, N, K):
 
 
 def llm():
-    print("| M | K x Ncols | pattern | kernel | ms | useful TFLOP/s | dense fp32 GEMM ms | speedup | of ideal 4x | preprocess ms |")
-    print("|---|---|---|---|---|---|---|---|---|---|")
+    print("| M | K x Ncols | pattern | kernel | best split of 1/2/4/8 | ms | useful TFLOP/s | library's split | ms | dense fp32 GEMM ms | speedup | of ideal 4x | preprocess ms |")
+    print("|---|---|---|---|---|---|---|---|---|---|---|---|---|")
     for (K, N) in ((4096, 4096), (4096, 11008), (11008, 4096)):
         for M in (512, 2048, 8192):
             op = Operands(M, N, K, 2, 8, dist="normal", b_scale=0.02, seed=M + K)
             best = (1e9, 1)
-            for split in (1, 2, 4):
+            for split in (1, 2, 4, 8):
                 if split > 1 and (M // 128) * (N // 128) * split > 4096:
                     continue
                 ws = None if split == 1 else torch.empty(pkg.workspace_bytes(M, N, split) // 4, dtype=torch.float32,
                                                          device="cuda")
                 best = min(best, (timed(lambda: op.launch(split, ws)), split))
             ms, split = best
+            auto_split = pkg.suggest_split_k(M, N, op.W, op.kept)
+            auto_ms = timed(lambda: pkg.gemm_auto(op.A, op.B, op.D, op.cinfo, op.C, M, N, K, op.W, 0.75))
             dms = dense_ms(M, N, K)
-            print("| %d | %dx%d | 2:8 | %s sk%d | %.4f | %.1f | %.4f | %.2f | %.2f | %.3f |" % (
-                M, K, N, pkg.last_kernel(), split, ms, op.flops() / ms / 1e9, dms, dms / ms, dms / ms / 4, op.preprocess_ms),
-                flush=True)
+            print("| %d | %dx%d | 2:8 | %s | %d | %.4f | %.1f | %d | %.4f | %.4f | %.2f | %.2f | %.3f |" % (
+                M, K, N, pkg.last_kernel(), split, ms, op.flops() / ms / 1e9, auto_split, auto_ms, dms, dms / auto_ms,
+                dms / auto_ms / 4, op.preprocess_ms), flush=True)
             del op
 
 

@@ -69,3 +69,10 @@ NMSPMM_DEFINE_PAIR(huge, NMSPMM_TILE_HUGE)
 NMSPMM_DEFINE_PAIR(large, NMSPMM_TILE_LARGE)
 NMSPMM_DEFINE_PAIR(medium, NMSPMM_TILE_MEDIUM)
 NMSPMM_DEFINE_PAIR(small, NMSPMM_TILE_SMALL)
+
+void nmGEMM(float* A, float* B, int* D, int* column_info, float* C, int M, int N, int K, int W, float sparsity)
+{
+    const int st = nmspmm_gemm_auto(A, B, D, column_info, C, M, N, K, W, sparsity, nullptr);
+    if (st != NMSPMM_ERR_BAD_PATTERN)
+        report("nmGEMM", st);
+}

@@ -138,6 +138,17 @@ static bool run_tile(const char* name, LowFn low, HighFn high, int Ns, int M, in
     return ok;
 }
 
+// the launcher that picks the split itself, under the signatures of the named ones
+static void auto_low(float* A, float* B, int* D, float* C, int M, int N, int K, int W, float sparsity, int)
+{
+    nmGEMM(A, B, D, nullptr, C, M, N, K, W, sparsity);
+}
+static void auto_high(float* A, float* B, int* D, int* column_info, float* C, int M, int N, int K, int W,
+                      float sparsity, int)
+{
+    nmGEMM(A, B, D, column_info, C, M, N, K, W, sparsity);
+}
+
 int main(int argc, char** argv)
 {
     int M = 512, N = 512, K = 512, pruning_M = 32, split_k = 1;
@@ -162,6 +173,7 @@ int main(int argc, char** argv)
         {"medium", &nmGEMM_medium_matrices_low_sparsity, &nmGEMM_medium_matrices_high_sparsity, 64},
         {"large", &nmGEMM_large_matrices_low_sparsity, &nmGEMM_large_matrices_high_sparsity, 64},
         {"huge", &nmGEMM_huge_matrices_low_sparsity, &nmGEMM_huge_matrices_high_sparsity, 128},
+        {"nmGEMM (split chosen by the library)", &auto_low, &auto_high, 128},
     };
     for (const Tile& t : tiles) {
         if (N % t.Ns != 0) continue;

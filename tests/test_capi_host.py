@@ -34,8 +34,22 @@ def test_library_exports_the_cxx_drop_in_functions():
     for size in ("huge", "large", "medium", "small"):
         wanted.append("nmGEMM_%s_matrices_low_sparsity(float*, float*, int*, float*, int, int, int, int, float, int)" % size)
         wanted.append("nmGEMM_%s_matrices_high_sparsity(float*, float*, int*, int*, float*, int, int, int, int, float, int)" % size)
+    wanted.append("nmGEMM(float*, float*, int*, int*, float*, int, int, int, int, float)")
     for w in wanted:
         assert " T " + w in out, w
+
+
+def test_split_suggestion():
+    L = nmspmm.lib()
+    assert L.nmspmm_suggest_split_k(4096, 4096, 2048, 16) == 1      # 4096 waves already
+    assert L.nmspmm_suggest_split_k(128, 4096, 2048, 16) == 8       # 128 waves, 128 windows
+    assert L.nmspmm_suggest_split_k(512, 4096, 1024, 16) == 2
+    assert L.nmspmm_suggest_split_k(128, 512, 128, 16) in (1, 2, 4, 8)  # never more slices than windows
+    assert L.nmspmm_suggest_split_k(4096, 4096, 16, 16) == 1        # one window cannot be split
+    assert L.nmspmm_suggest_split_k(8, 8192, 1024, 8) == 1          # decode kernel reduces in the workgroup
+    assert L.nmspmm_suggest_split_k(0, 8192, 1024, 8) == 0 and L.nmspmm_suggest_split_k(64, 64, 100, 16) == 0
+    assert L.nmspmm_gemm_auto(FAKE, FAKE, FAKE, None, FAKE, 64, 128, 128, 16, 0.75, None) == 1   # column_info missing
+    assert L.nmspmm_gemm_auto(FAKE, FAKE, FAKE, None, FAKE, 64, 128, 128, 64, 0.3, None) == 3
 
 
 def test_pattern_table():

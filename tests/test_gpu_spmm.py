@@ -142,6 +142,25 @@ def test_named_entry_points_with_gpu_preprocessing(oracle, sparsity, n, m, tile)
     check(oracle, d, C.cpu().numpy())
 
 
+@pytest.mark.parametrize("M,N,K,n,m,sparsity", [(128, 1024, 2048, 2, 4, 0.5), (256, 512, 4096, 2, 8, 0.75),
+                                                 (512, 1024, 1024, 1, 8, 0.875), (2048, 2048, 512, 3, 8, 0.625),
+                                                 (16, 512, 2048, 2, 8, 0.75)])
+def test_auto_entry_point_chooses_the_split_itself(oracle, M, N, K, n, m, sparsity):
+    d = datagen.init_data(M, N, K, n, m, seed=M + K)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    nmspmm.gemm_auto(dev(d["A_km"]), dev(d["BT"]), dev(D), None if cinfo is None else dev(cinfo), C, M, N, K, d["W"],
+                     sparsity)
+    torch.cuda.synchronize()
+    split = nmspmm.suggest_split_k(M, N, d["W"], kept)
+    assert 1 <= split <= 16 and (d["W"] // kept) // split >= 1
+    if M == 128 and K == 2048:
+        assert split > 1          # 128 waves for 1024 SIMDs: the reduction must be split
+    if M == 2048 or M <= 32:
+        assert split == 1
+    check(oracle, d, C.cpu().numpy())
+
+
 def test_llm_layer_shape_2of8(oracle):
     """One BASELINE config-3 shape (M = 512, K = 4096, Ncols = 11008, 2:8, N(0,1) x N(0,0.02^2))."""
     d = datagen.init_data(512, 11008, 4096, 2, 8, seed=3001, dist="normal", b_scale=0.02)
