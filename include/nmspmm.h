@@ -128,6 +128,21 @@ int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t*
                 float* C, int M, int N, int K, int W, int window, int kept, int vec_len, int Ns,
                 int split_k, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Row-major A (M x K, K contiguous per row: activations as a model produces them).  No
+ * counterpart: the reference kernels demand column-major A (reference
+ * src/kernel_64x128_8x8.cu:15), i.e. a transpose before every layer.  nmspmm_transpose_device
+ * writes dst[c][r] = src[r][c] for a rows x cols row-major src (so rows = M, cols = K turns a
+ * row-major A into the layout nmspmm_spmm takes; one such copy serves every weight matrix that
+ * multiplies the same activations).  nmspmm_spmm_rowmajor does both steps: the workspace holds the
+ * column-major copy followed by the split-K slices, nmspmm_workspace_bytes_rowmajor() bytes, never
+ * optional.  Other arguments and requirements as nmspmm_spmm. */
+int nmspmm_transpose_device(const float* src, int rows, int cols, float* dst, void* stream);
+size_t nmspmm_workspace_bytes_rowmajor(int M, int N, int K, int split_k);
+int nmspmm_spmm_rowmajor(const float* A_rowmajor, const float* B, const int32_t* D,
+                         const int32_t* column_info, float* C, int M, int N, int K, int W, int window,
+                         int kept, int vec_len, int Ns, int split_k, void* workspace,
+                         size_t workspace_bytes, void* stream);
+
 /* Replace the reference launchers nmGEMM_{small,medium,large,huge}_matrices_low_sparsity
  * (reference include/NM-SpMM.h:14,17,20,23) and ..._high_sparsity (:15,18,21,24): `tile` is the
  * nmspmm_tile of the named entry point, `sparsity` selects the geometry as

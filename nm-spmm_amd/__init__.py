@@ -59,6 +59,10 @@ def lib():
         L.nmspmm_spmm.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, c_void_p]
         L.nmspmm_gemm_low_sparsity.argtypes = [c_int] + [c_void_p] * 4 + [c_int] * 4 + [c_float, c_int, c_void_p]
         L.nmspmm_gemm_high_sparsity.argtypes = [c_int] + [c_void_p] * 5 + [c_int] * 4 + [c_float, c_int, c_void_p]
+        L.nmspmm_transpose_device.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p]
+        L.nmspmm_workspace_bytes_rowmajor.restype = c_size_t
+        L.nmspmm_workspace_bytes_rowmajor.argtypes = [c_int] * 4
+        L.nmspmm_spmm_rowmajor.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, c_void_p]
         L.nmspmm_suggest_split_k.argtypes = [c_int] * 4
         L.nmspmm_gemm_auto.argtypes = [c_void_p] * 5 + [c_int] * 4 + [c_float, c_void_p]
         L.nmspmm_release.restype = c_int
@@ -150,6 +154,22 @@ def gemm_high_sparsity(tile, A, B, D, cinfo, C, M, N, K, W, sparsity, split_k=1)
 
 
 # ---- host-pointer forms: arguments are C-contiguous numpy int32 arrays, updated in place ----------
+
+def transpose_device(src, rows, cols, dst):
+    _check("nmspmm_transpose_device", lib().nmspmm_transpose_device(_ptr(src), rows, cols, _ptr(dst), _stream()))
+
+
+def workspace_bytes_rowmajor(M, N, K, split_k):
+    return lib().nmspmm_workspace_bytes_rowmajor(M, N, K, split_k)
+
+
+def spmm_rowmajor(A_rm, B, D, cinfo, C, M, N, K, W, window, kept, workspace, vec_len=32, Ns=128, split_k=1):
+    """A_rm is row-major M x K; `workspace` (float32 tensor) holds workspace_bytes_rowmajor() bytes."""
+    _check("nmspmm_spmm_rowmajor",
+           lib().nmspmm_spmm_rowmajor(_ptr(A_rm), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(C), M, N, K, W, window, kept,
+                                      vec_len, Ns, split_k, _ptr(workspace), workspace.numel() * workspace.element_size(),
+                                      _stream()))
+
 
 def suggest_split_k(M, N, W, kept):
     return lib().nmspmm_suggest_split_k(M, N, W, kept)

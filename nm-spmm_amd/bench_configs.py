@@ -3,7 +3,7 @@
 square sweep): LLM-layer shapes, decode-sized M, and the fine-grained / short-vector patterns.
 Prints one markdown table row per case.
 
-    python nm-spmm_amd/bench_configs.py [llm] [decode] [fine] [compress]
+    python nm-spmm_amd/bench_configs.py [llm] [decode] [fine] [compress] [rowmajor]
 
 useful TFLOP/s = 2*M*Ncols*W / t; GB/s = algorithmic bytes
 4*(M*K + W*Ncols + W*Ncols/L + M*Ncols) (+ column_info) / t.
@@ -164,9 +164,28 @@ def compress():
                                                                     nbytes / ms / 1e6 / 8000), flush=True)
 
 
+def rowmajor():
+    print("| M | K x Ncols | pattern | transpose us | GB/s of 2*M*K*4 | multiply ms | both ms | overhead |")
+    print("|---|---|---|---|---|---|---|---|")
+    for (K, N) in ((4096, 4096), (4096, 11008), (11008, 4096)):
+        for M in (512, 2048, 8192):
+            op = Operands(M, N, K, 2, 8, dist="normal", b_scale=0.02, seed=M + K)
+            A_rm = op.A.t().contiguous()
+            split = pkg.suggest_split_k(M, N, op.W, op.kept)
+            ws = torch.empty(pkg.workspace_bytes_rowmajor(M, N, K, split) // 4, dtype=torch.float32, device="cuda")
+            ws_cm = torch.empty(max(pkg.workspace_bytes(M, N, split) // 4, 1), dtype=torch.float32, device="cuda")
+            t_tr = timed(lambda: pkg.transpose_device(A_rm, M, K, ws))
+            t_mm = timed(lambda: op.launch(split, ws_cm if split > 1 else None))
+            t_both = timed(lambda: pkg.spmm_rowmajor(A_rm, op.B, op.D, op.cinfo, op.C, M, N, K, op.W, op.window, op.kept, ws,
+                                                     32, op.Ns, split))
+            print("| %d | %dx%d | 2:8 | %.1f | %.0f | %.4f | %.4f | %.1f %% |" % (
+                M, K, N, t_tr * 1e3, 8.0 * M * K / t_tr / 1e6, t_mm, t_both, 100.0 * (t_both / t_mm - 1.0)), flush=True)
+            del op
+
+
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["llm", "decode", "fine", "compress"]
+    which = sys.argv[1:] or ["llm", "decode", "fine", "compress", "rowmajor"]
     pkg.lib()
     for name in which:
         print("\n### %s" % name)
-        {"llm": llm, "decode": decode, "fine": fine, "compress": compress}[name]()
+        {"llm": llm, "decode": decode, "fine": fine, "compress": compress, "rowmajor": rowmajor}[name]()

@@ -369,6 +369,47 @@ int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t*
     return NMSPMM_OK;
 }
 
+int nmspmm_transpose_device(const float* src, int rows, int cols, float* dst, void* stream)
+{
+    if (!src || !dst)
+        return NMSPMM_ERR_NULL_POINTER;
+    if (rows <= 0 || cols <= 0 || src == dst || (rows + 63) / 64 > 65535)
+        return NMSPMM_ERR_BAD_SHAPE;
+    return launch_transpose(src, dst, rows, cols, (hipStream_t)stream) == hipSuccess ? NMSPMM_OK : NMSPMM_ERR_HIP;
+}
+
+// floats the column-major copy of a row-major A occupies at the head of the workspace
+static size_t rowmajor_copy_floats(int M, int K) { return ((size_t)M * K + 3) / 4 * 4; }
+
+size_t nmspmm_workspace_bytes_rowmajor(int M, int N, int K, int split_k)
+{
+    if (M <= 0 || N <= 0 || K <= 0 || split_k < 1)
+        return 0;
+    return sizeof(float) * rowmajor_copy_floats(M, K) + nmspmm_workspace_bytes(M, N, split_k);
+}
+
+int nmspmm_spmm_rowmajor(const float* A_rowmajor, const float* B, const int32_t* D, const int32_t* column_info,
+                         float* C, int M, int N, int K, int W, int window, int kept, int vec_len, int Ns,
+                         int split_k, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!A_rowmajor)
+        return NMSPMM_ERR_NULL_POINTER;
+    if (M <= 0 || N <= 0 || K <= 0)
+        return NMSPMM_ERR_BAD_SHAPE;
+    if (split_k < 1)
+        return NMSPMM_ERR_BAD_SPLIT;
+    if (!workspace || !aligned16(workspace) || workspace_bytes < nmspmm_workspace_bytes_rowmajor(M, N, K, split_k))
+        return NMSPMM_ERR_WORKSPACE;
+    float* const At = (float*)workspace;
+    float* const slices = At + rowmajor_copy_floats(M, K);
+    const size_t slice_bytes = workspace_bytes - sizeof(float) * rowmajor_copy_floats(M, K);
+    const int st = nmspmm_transpose_device(A_rowmajor, M, K, At, stream);
+    if (st != NMSPMM_OK)
+        return st;
+    return nmspmm_spmm(At, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k,
+                       split_k > 1 ? slices : nullptr, split_k > 1 ? slice_bytes : 0, stream);
+}
+
 static int named_gemm(int want_high, int tile, const float* A, const float* B, const int32_t* D,
                       const int32_t* column_info, float* C, int M, int N, int K, int W, float sparsity,
                       int split_k, void* stream)

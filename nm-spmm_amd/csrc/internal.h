@@ -62,5 +62,8 @@ hipError_t launch_compress(const float* B, float* BT, int32_t* DT, int K, int N,
 hipError_t launch_decompress(const float* BT, const int32_t* DT, float* B, int K, int N, int n, int m, int vec_len,
                              hipStream_t stream);
 
+// dst[c][r] = src[r][c] for a rows x cols row-major src (transpose.hip).
+hipError_t launch_transpose(const float* src, float* dst, int rows, int cols, hipStream_t stream);
+
 } // namespace nmspmm
 #endif

@@ -135,6 +135,20 @@ def test_compress_rejects_bad_arguments_without_a_gpu():
     assert L.nmspmm_decompress_device(FAKE, FAKE, 64, 40, 2, 4, 32, FAKE, None) == 2  # N % vec_len
 
 
+def test_rowmajor_entry_rejects_bad_arguments_without_a_gpu():
+    L = nmspmm.lib()
+    L.nmspmm_workspace_bytes_rowmajor.restype = ctypes.c_size_t
+    assert L.nmspmm_workspace_bytes_rowmajor(64, 128, 256, 1) == 4 * 64 * 256
+    assert L.nmspmm_workspace_bytes_rowmajor(64, 128, 256, 2) == 4 * 64 * 256 + L.nmspmm_workspace_bytes(64, 128, 2)
+    assert L.nmspmm_workspace_bytes_rowmajor(0, 128, 256, 1) == 0
+    assert L.nmspmm_transpose_device(None, 4, 4, FAKE, None) == 1
+    assert L.nmspmm_transpose_device(FAKE, 4, 0, FAKE + 64, None) == 2
+    assert L.nmspmm_transpose_device(FAKE, 4, 4, FAKE, None) == 2                     # in place
+    args = [FAKE, FAKE, FAKE, None, FAKE, 64, 128, 256, 128, 32, 16, 32, 128, 1]
+    assert L.nmspmm_spmm_rowmajor(*args, None, 0, None) == 6                           # workspace is never optional
+    assert L.nmspmm_spmm_rowmajor(*args, FAKE, 4 * 64 * 256 - 16, None) == 6
+
+
 def test_split_rule_matches_reference_partition():
     """The reference kernels give the first (windows % SPLIT_K) slices one extra window
     (src/kernel_64x128_8x8.cu:20-37, '20 tasks over 8 slices: 3 3 3 3 2 2 2 2')."""
