@@ -3,7 +3,7 @@
 square sweep): LLM-layer shapes, decode-sized M, and the fine-grained / short-vector patterns.
 Prints one markdown table row per case.
 
-    python nm-spmm_amd/bench_configs.py [llm] [decode] [fine] [compress] [rowmajor]
+    python nm-spmm_amd/bench_configs.py [llm] [decode] [fine] [compress] [rowmajor] [sweep100]
 
 useful TFLOP/s = 2*M*Ncols*W / t; GB/s = algorithmic bytes
 4*(M*K + W*Ncols + W*Ncols/L + M*Ncols) (+ column_info) / t.
@@ -164,6 +164,59 @@ def compress():
                                                                     nbytes / ms / 1e6 / 8000), flush=True)
 
 
+def sweep100():
+    """The reference's 100-shape comparison against the dense GEMM
+    (benchmark/kernel_performance/run_test/nmspmm/run_nmspmm.sh:16-36): 5 row counts x 20 LLM layer
+    shapes, patterns n:32 at 50 / 62.5 / 75 / 87.5 %, here with the split the library picks instead
+    of the best of four timed ones.  Patterns and values are drawn on the GPU."""
+    Ms = (256, 512, 1024, 2048, 4096)
+    Ns = (2048, 6144, 2048, 5632, 4096, 12288, 4096, 11008, 5120, 15360, 5120, 13824, 6656, 19968, 6656, 17920, 8192,
+          24576, 8192, 22016)
+    Ks = (2048, 2048, 5632, 2048, 4096, 4096, 11008, 4096, 5120, 5120, 13824, 5120, 6656, 6656, 17920, 6656, 8192, 8192,
+          22016, 8192)
+    kinds = ((0.5, 16, 32, 16), (0.625, 12, 32, 12), (0.75, 8, 64, 16), (0.875, 4, 64, 8))  # sparsity, n of 32, window, kept
+    dense = {}
+    speed = {k[0]: [] for k in kinds}
+    print("| sparsity | M | Ncols | K | split | ms | useful TFLOP/s | dense ms | speedup |")
+    print("|---|---|---|---|---|---|---|---|---|")
+    for (N, K) in zip(Ns, Ks):
+        Q = N // 32
+        for (sparsity, n, window, kept) in kinds:
+            W = K // 32 * n
+            B = torch.randn((W, N), dtype=torch.float32, device="cuda") * 0.02
+            pick = torch.rand((K // 32, Q, 32), device="cuda").argsort(dim=2)[:, :, :n].sort(dim=2).values
+            DT = pick.permute(0, 2, 1).reshape(W, Q).to(torch.int32).contiguous()
+            D = torch.empty_like(DT)
+            cinfo = None
+            if window == 64:
+                pn, pm = pkg.trans_index_device(DT, W, N, Q, n, 32)
+                cinfo = torch.empty(pkg.column_info_ints(W, pn, pm, N, 128), dtype=torch.int32, device="cuda")
+                pkg.preprocess_high_device(cinfo, pm, pn, DT, D, W, Q, N, 128)
+            else:
+                pkg.preprocess_low_device(DT, D, W, Q, 128)
+            for M in Ms:
+                A = torch.randn((K, M), dtype=torch.float32, device="cuda")
+                C = torch.empty((M, N), dtype=torch.float32, device="cuda")
+                ms = timed(lambda: pkg.gemm_auto(A, B, D, cinfo, C, M, N, K, W, sparsity), 20, 3, 0.05)
+                if (M, N, K) not in dense:
+                    Bd = torch.randn((K, N), dtype=torch.float32, device="cuda")
+                    Am = A.t().contiguous()
+                    dense[(M, N, K)] = timed(lambda: torch.mm(Am, Bd, out=C), 20, 3, 0.05)
+                    del Bd, Am
+                dms = dense[(M, N, K)]
+                speed[sparsity].append(dms / ms)
+                print("| %.3f | %d | %d | %d | %d | %.4f | %.1f | %.4f | %.2f |" % (
+                    sparsity, M, N, K, pkg.suggest_split_k(M, N, W, kept), ms, 2.0 * M * N * W / ms / 1e9, dms, dms / ms),
+                    flush=True)
+            del B, DT, D, cinfo
+    print()
+    print("| sparsity | shapes | mean speedup over the dense fp32 GEMM | min | max | ideal |")
+    print("|---|---|---|---|---|---|")
+    for (sparsity, n, window, kept) in kinds:
+        v = speed[sparsity]
+        print("| %.3f | %d | %.2f | %.2f | %.2f | %.2f |" % (sparsity, len(v), sum(v) / len(v), min(v), max(v), 32.0 / n))
+
+
 def rowmajor():
     print("| M | K x Ncols | pattern | transpose us | GB/s of 2*M*K*4 | multiply ms | both ms | overhead |")
     print("|---|---|---|---|---|---|---|---|")
@@ -188,4 +241,4 @@ if __name__ == "__main__":
     pkg.lib()
     for name in which:
         print("\n### %s" % name)
-        {"llm": llm, "decode": decode, "fine": fine, "compress": compress, "rowmajor": rowmajor}[name]()
+        {"llm": llm, "decode": decode, "fine": fine, "compress": compress, "rowmajor": rowmajor, "sweep100": sweep100}[name]()

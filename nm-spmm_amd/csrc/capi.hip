@@ -461,22 +461,18 @@ int nmspmm_suggest_split_k(int M, int N, int W, int kept)
         return 0;
     if (M <= 32)
         return 1;  // the decode kernel reduces inside its workgroups
-    // A small cost model, fitted to a sweep of M in 128..4096, N = K in 512..4096 at 2:4, 3:8, 2:8
-    // and 1:8 on one MI355X (its choice is within 1 % of the best split on average, where never
-    // splitting loses 32 %).  A workgroup covers 128 rows x 128 columns and needs kept * 53.5 ns of
-    // a CU's matrix pipes per window (kept/2 k-steps x 4 MFMAs x 64 cycles at 2.39 GHz); the
-    // workgroups of all slices are dealt round-robin to 256 CUs; a CU with a single workgroup (one
-    // wave per SIMD) runs at about 0.8 of its rate.  Splitting adds a second pass that moves
-    // (2 * split + 1) * M * N floats at about 5 TB/s plus a launch; every launch has about 12 us of
-    // fixed cost (gap between launches, first loads, store of C).
+    // The modelled time of the kernel (model_kernel_seconds, at the wave height the kernel would
+    // pick) plus, for a split, the second pass that moves (2 * split + 1) * M * N floats at about
+    // 5 TB/s and its launch; every launch has about 12 us of fixed cost (gap between launches,
+    // first loads, store of C).  Fitted to a sweep of M in 128..4096, N = K in 512..4096 at 2:4,
+    // 3:8, 2:8 and 1:8 on one MI355X: the choice is within 1 % of the best split on average,
+    // where never splitting loses 32 %.
     const int nwin = W / kept;
-    const long long groups = (long long)((M + 127) / 128) * ((N + 127) / 128);
     int best = 1;
     double best_t = 0.0;
     for (int split = 1; split <= 16 && split <= nwin; split *= 2) {
-        const long long per_cu = (groups * split + 255) / 256;
-        const double rate = groups * split <= 256 ? 0.8 : 1.0;
-        double t = 12e-6 + (double)per_cu * ((nwin + split - 1) / split) * kept * 53.5e-9 / rate;
+        const int blocks = choose_wave_blocks(M, N, nwin, kept, split);
+        double t = 12e-6 + model_kernel_seconds(M, N, nwin, kept, blocks, split);
         if (split > 1)
             t += (2.0 * split + 1.0) * M * N * sizeof(float) / 5e12 + 3e-6;
         if (split == 1 || t < 0.97 * best_t) {  // a finer split has to win by 3 %

@@ -33,6 +33,35 @@ __host__ __device__ inline void split_windows(int nwin, int split_k, int z, int*
     *count = z < q ? p + 1 : p;
 }
 
+// Modelled run time in seconds of the matrix-core kernel for waves of `blocks` 32-row blocks (4 or
+// 8) and `split` reduction slices, without the second pass of a split.  A workgroup covers
+// 32*blocks rows x 128 columns; per window it needs kept/2 k-steps x blocks MFMAs x 64 cycles of
+// each of its CU's four matrix pipes (2.39 GHz; 256-row waves spend about 4 % less on loads).  A
+// CU holds four workgroups of 128-row waves or two of 256-row waves at once and they share its
+// pipes, so the 256 CUs retire the workgroups in rounds of 1024 or 512; the last, partial round
+// costs as much as its busiest CU, and a CU left with one workgroup (one wave per SIMD) runs at
+// about 0.8 of its rate.  Constants fitted to sweeps on one MI355X.
+inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks, int split)
+{
+    const double per_window = kept * 53.5e-9 * (blocks == 8 ? 2.0 / 1.04 : 1.0);
+    const double unit = per_window * ((nwin + split - 1) / split);
+    const long long groups = (long long)((M + 32 * blocks - 1) / (32 * blocks)) * ((N + 127) / 128) * split;
+    const int slots = blocks == 8 ? 2 : 4;
+    const long long full = groups / (256 * slots), rest = groups % (256 * slots);
+    const long long busiest = (rest + 255) / 256;
+    double t = (double)full * slots * unit;
+    if (busiest > 0)
+        t += busiest * unit / (busiest == 1 && full == 0 ? 0.8 : 1.0);
+    return t;
+}
+// Wave height (32-row blocks) the matrix-core kernel uses for a shape: the faster one by the model.
+inline int choose_wave_blocks(int M, int N, int nwin, int kept, int split)
+{
+    if (M <= 128)
+        return 4;
+    return model_kernel_seconds(M, N, nwin, kept, 8, split) < model_kernel_seconds(M, N, nwin, kept, 4, split) ? 8 : 4;
+}
+
 // Matrix-core path (spmm_direct.hip).  Returns false when the geometry has no instantiation.
 bool mfma_supported(const SpmmArgs& a);
 hipError_t launch_mfma(const SpmmArgs& a);

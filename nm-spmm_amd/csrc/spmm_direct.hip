@@ -34,7 +34,6 @@ namespace nmspmm {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kXcds = 8;
-constexpr int kCus = 256;
 
 struct DirectParams {
     const float* A;
@@ -303,14 +302,13 @@ static hipError_t launch_cfg(const SpmmArgs& a)
 }
 
 // Every workgroup has four waves: 1 x 4, 2 x 2 or 4 x 1 (rows x column vectors), chosen by the
-// column-block width the indices were preprocessed for.  A wave is 256 rows tall when that still
-// leaves every SIMD two waves (the taller wave halves the B and index loads per MFMA), 128 rows
-// otherwise.
+// column-block width the indices were preprocessed for.  A wave is 256 or 128 rows tall, whichever
+// the run-time model expects to finish first: the taller wave halves the B and index loads per
+// MFMA, but only two such workgroups fit a CU, which quantises badly on mid-sized problems.
 template <int KS, int WS, bool HIGH>
 static hipError_t launch_ns(const SpmmArgs& a)
 {
-    const long long waves_tall = (long long)((a.M + 255) / 256) * (a.N / 32) * a.split_k;
-    const bool tall = waves_tall >= 2LL * 4 * kCus;
+    const bool tall = NMSPMM_RM_TALL == 8 && choose_wave_blocks(a.M, a.N, a.W / WS, WS, a.split_k) == 8;
     switch (a.Ns) {
     case 128:
         return tall ? launch_cfg<KS, WS, 4, 1, NMSPMM_RM_TALL, HIGH>(a) : launch_cfg<KS, WS, 4, 1, 4, HIGH>(a);

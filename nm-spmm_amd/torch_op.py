@@ -1,0 +1,99 @@
+"""A drop-in for torch.nn.Linear (inference) whose weight is N:M vector-sparse and whose forward
+runs the library's kernels: dense weight -> compress -> widen / preprocess once at construction,
+then one row-major multiplication per call.  PyTorch only supplies device memory and the stream.
+
+The reference has no framework binding; its driver multiplies synthetic operands
+(tests/test_nmspmm.cu:72-97).  The sequence of calls here is that driver's, on real weights.
+"""
+import importlib
+
+import torch
+
+_nm = importlib.import_module(__name__.rsplit(".", 1)[0])
+
+# (n, m) reduced to lowest terms -> (window, kept) the kernels run the pattern at
+# (reference launchers, src/kernel_64x128_8x8.cu:264-289,584-602)
+_GEOMETRY = {(1, 2): (32, 16), (3, 8): (32, 12), (1, 4): (64, 16), (1, 8): (64, 8)}
+
+
+def _geometry(n, m):
+    from math import gcd
+    g = gcd(n, m)
+    if (n // g, m // g) not in _GEOMETRY:
+        raise ValueError("pattern %d:%d is not one of 1:2, 3:8, 1:4, 1:8 (or a multiple of them)" % (n, m))
+    window, kept = _GEOMETRY[(n // g, m // g)]
+    if window % m != 0:
+        raise ValueError("pattern window %d does not divide the kernel window %d" % (m, window))
+    return window, kept
+
+
+class NMSparseLinear(torch.nn.Module):
+    """y = x @ prune(weight).T + bias with an n:m pattern shared by 32 adjacent output features.
+
+    weight: float32 CUDA tensor [out_features, in_features]; in_features % window == 0 and
+    out_features % 32 == 0.  Rows of x beyond the first dimension are flattened; the matrix-core
+    kernel needs their count to be a multiple of 4 (or at most 32 for the decode kernel), other
+    counts take the generic kernel.
+    """
+
+    def __init__(self, weight, n, m, bias=None):
+        super().__init__()
+        if weight.dtype != torch.float32 or not weight.is_cuda or weight.dim() != 2:
+            raise ValueError("weight must be a 2-D float32 CUDA tensor")
+        self.out_features, self.in_features = weight.shape
+        self.n, self.m = n, m
+        self.window, self.kept = _geometry(n, m)
+        N, K = self.out_features, self.in_features
+        if K % self.window != 0 or N % 32 != 0:
+            raise ValueError("in_features must be a multiple of %d and out_features of 32" % self.window)
+        self.Ns = 128 if N % 128 == 0 else 64 if N % 64 == 0 else 32
+        self.W, self.Q = K // m * n, N // 32
+        dense = weight.t().contiguous()                                   # K x N, row-major
+        BT = torch.empty((self.W, N), dtype=torch.float32, device=weight.device)
+        DT = torch.empty((self.W, self.Q), dtype=torch.int32, device=weight.device)
+        _nm.compress_device(dense, K, N, n, m, BT, DT)
+        pn, pm = n, m
+        while pm < self.window:
+            pn, pm = _nm.trans_index_device(DT, self.W, N, self.Q, pn, pm)
+        D = torch.empty_like(DT)
+        cinfo = None
+        if self.window == 64:
+            cinfo = torch.empty(_nm.column_info_ints(self.W, pn, pm, N, self.Ns), dtype=torch.int32, device=weight.device)
+            _nm.preprocess_high_device(cinfo, pm, pn, DT, D, self.W, self.Q, N, self.Ns)
+        else:
+            _nm.preprocess_low_device(DT, D, self.W, self.Q, self.Ns)
+        self.register_buffer("values", BT)
+        self.register_buffer("indices", D.reshape(-1))
+        self.register_buffer("column_info", cinfo)
+        self.register_buffer("bias", None if bias is None else bias.detach().to(torch.float32))
+        self._workspace = None
+
+    def dense_weight(self):
+        """The pruned weight as a dense [out_features, in_features] tensor (for checking)."""
+        # undo the preprocessing by compressing the expansion instead of storing DT twice: the kept
+        # values are in `values`, their rows are recovered from a multiplication with the identity
+        eye = torch.eye(self.in_features, dtype=torch.float32, device=self.values.device)
+        return self.forward(eye, add_bias=False).t().contiguous()
+
+    def forward(self, x, add_bias=True):
+        if x.dtype != torch.float32 or not x.is_cuda or x.shape[-1] != self.in_features:
+            raise ValueError("x must be a float32 CUDA tensor whose last dimension is in_features")
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, self.in_features).contiguous()
+        M, N, K = x2.shape[0], self.out_features, self.in_features
+        y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+        if M == 0:
+            return y.reshape(*lead, N)
+        split = _nm.suggest_split_k(M, N, self.W, self.kept)
+        need = _nm.workspace_bytes_rowmajor(M, N, K, split) // 4
+        if self._workspace is None or self._workspace.numel() < need or self._workspace.device != x.device:
+            self._workspace = torch.empty(need, dtype=torch.float32, device=x.device)
+        _nm.spmm_rowmajor(x2, self.values, self.indices, self.column_info, y, M, N, K, self.W, self.window, self.kept,
+                          self._workspace, 32, self.Ns, split)
+        if add_bias and self.bias is not None:
+            y += self.bias
+        return y.reshape(*lead, N)
+
+    def extra_repr(self):
+        return "in_features=%d, out_features=%d, pattern=%d:%d, bias=%s" % (
+            self.in_features, self.out_features, self.n, self.m, self.bias is not None)
