@@ -301,9 +301,11 @@ size_t nmspmm_workspace_bytes(int M, int N, int split_k)
     return sizeof(float) * slice_stride(M, N) * (size_t)split_k;
 }
 
-int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C, int M,
-                int N, int K, int W, int window, int kept, int vec_len, int Ns, int split_k, void* workspace,
-                size_t workspace_bytes, void* stream)
+// lda: floats between consecutive dense rows of A; 0 lets the function choose (M, or M rounded up
+// to 4 when `may_pad` allows it and that puts the shape on the matrix-core path) and reports it.
+static int spmm_impl(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C, int M,
+                     int N, int K, int W, int window, int kept, int vec_len, int Ns, int split_k, void* workspace,
+                     size_t workspace_bytes, void* stream, int lda, bool dry_run, int* lda_out)
 {
     if (!A || !B || !D || !C)
         return NMSPMM_ERR_NULL_POINTER;
@@ -333,6 +335,7 @@ int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t*
     a.partial = split_k > 1 ? (float*)workspace : nullptr;
     a.slice_stride = slice_stride(M, N);
     a.M = M;
+    a.lda = lda > 0 ? lda : M;
     a.N = N;
     a.K = K;
     a.W = W;
@@ -342,6 +345,17 @@ int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t*
     a.Ns = Ns;
     a.split_k = split_k;
     a.stream = (hipStream_t)stream;
+
+    if (lda == 0 && M > 32 && M % 4 != 0) {
+        // a padded copy of A is only worth making if it reaches the matrix-core kernel
+        a.lda = (M + 3) / 4 * 4;
+        if (!mfma_supported(a))
+            a.lda = M;
+    }
+    if (lda_out)
+        *lda_out = a.lda;
+    if (dry_run)
+        return NMSPMM_OK;
 
     hipError_t e;
     if (skinny_supported(a)) {
@@ -375,11 +389,13 @@ int nmspmm_transpose_device(const float* src, int rows, int cols, float* dst, vo
         return NMSPMM_ERR_NULL_POINTER;
     if (rows <= 0 || cols <= 0 || src == dst || (rows + 63) / 64 > 65535)
         return NMSPMM_ERR_BAD_SHAPE;
-    return launch_transpose(src, dst, rows, cols, (hipStream_t)stream) == hipSuccess ? NMSPMM_OK : NMSPMM_ERR_HIP;
+    return launch_transpose(src, dst, rows, cols, rows, (hipStream_t)stream) == hipSuccess ? NMSPMM_OK
+                                                                                            : NMSPMM_ERR_HIP;
 }
 
-// floats the column-major copy of a row-major A occupies at the head of the workspace
-static size_t rowmajor_copy_floats(int M, int K) { return ((size_t)M * K + 3) / 4 * 4; }
+// floats reserved at the head of the workspace for the column-major copy of a row-major A: K rows
+// of M rounded up to 4
+static size_t rowmajor_copy_floats(int M, int K) { return (size_t)K * ((size_t)(M + 3) / 4 * 4); }
 
 size_t nmspmm_workspace_bytes_rowmajor(int M, int N, int K, int split_k)
 {
@@ -394,7 +410,7 @@ int nmspmm_spmm_rowmajor(const float* A_rowmajor, const float* B, const int32_t*
 {
     if (!A_rowmajor)
         return NMSPMM_ERR_NULL_POINTER;
-    if (M <= 0 || N <= 0 || K <= 0)
+    if (M <= 0 || N <= 0 || K <= 0 || (M + 63) / 64 > 65535)
         return NMSPMM_ERR_BAD_SHAPE;
     if (split_k < 1)
         return NMSPMM_ERR_BAD_SPLIT;
@@ -403,11 +419,24 @@ int nmspmm_spmm_rowmajor(const float* A_rowmajor, const float* B, const int32_t*
     float* const At = (float*)workspace;
     float* const slices = At + rowmajor_copy_floats(M, K);
     const size_t slice_bytes = workspace_bytes - sizeof(float) * rowmajor_copy_floats(M, K);
-    const int st = nmspmm_transpose_device(A_rowmajor, M, K, At, stream);
+    // check every argument and settle the row pitch of the copy before anything is launched
+    int lda = M;
+    const int st = spmm_impl(At, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k,
+                             split_k > 1 ? slices : nullptr, split_k > 1 ? slice_bytes : 0, stream, 0, true, &lda);
     if (st != NMSPMM_OK)
         return st;
-    return nmspmm_spmm(At, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k,
-                       split_k > 1 ? slices : nullptr, split_k > 1 ? slice_bytes : 0, stream);
+    if (launch_transpose(A_rowmajor, At, M, K, lda, (hipStream_t)stream) != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    return spmm_impl(At, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k,
+                     split_k > 1 ? slices : nullptr, split_k > 1 ? slice_bytes : 0, stream, lda, false, nullptr);
+}
+
+int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C, int M,
+                int N, int K, int W, int window, int kept, int vec_len, int Ns, int split_k, void* workspace,
+                size_t workspace_bytes, void* stream)
+{
+    return spmm_impl(A, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k, workspace,
+                     workspace_bytes, stream, M, false, nullptr);
 }
 
 static int named_gemm(int want_high, int tile, const float* A, const float* B, const int32_t* D,

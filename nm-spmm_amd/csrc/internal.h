@@ -10,7 +10,7 @@ namespace nmspmm {
 
 // One multiplication, already validated by the C-ABI layer.
 struct SpmmArgs {
-    const float* A;        // column-major M x K
+    const float* A;        // column-major M x K: element (i,k) at A[i + k*lda]
     const float* B;        // row-major W x N
     const int32_t* D;      // [N/Ns][W][Ns/vec_len]
     const int32_t* cinfo;  // [N/Ns][W/kept][window] or nullptr (low-sparsity layout)
@@ -18,6 +18,8 @@ struct SpmmArgs {
     float* partial;        // split_k slices of slice_stride floats when split_k > 1, else nullptr
     size_t slice_stride;   // M * N rounded up to a multiple of 4
     int M, N, K, W;
+    int lda;               // floats between consecutive dense rows of A; M unless the copy of a
+                           // row-major A was padded (matrix-core path only)
     int window, kept, vec_len, Ns;
     int split_k;
     hipStream_t stream;
@@ -91,8 +93,8 @@ hipError_t launch_compress(const float* B, float* BT, int32_t* DT, int K, int N,
 hipError_t launch_decompress(const float* BT, const int32_t* DT, float* B, int K, int N, int n, int m, int vec_len,
                              hipStream_t stream);
 
-// dst[c][r] = src[r][c] for a rows x cols row-major src (transpose.hip).
-hipError_t launch_transpose(const float* src, float* dst, int rows, int cols, hipStream_t stream);
+// dst[c * dst_ld + r] = src[r * cols + c] for a rows x cols row-major src (transpose.hip).
+hipError_t launch_transpose(const float* src, float* dst, int rows, int cols, int dst_ld, hipStream_t stream);
 
 } // namespace nmspmm
 #endif

@@ -43,6 +43,7 @@ struct DirectParams {
     float* out;          // C, or the first partial slice when split_k > 1
     size_t slice_elems;  // floats between partial slices
     int M, N, W;
+    int lda;             // floats between consecutive dense rows of A (>= M, a multiple of 4)
     int nwin;            // windows in the whole reduction
     int split_k;
     int tiles_m, tiles_n;
@@ -133,19 +134,20 @@ spmm_direct_kernel(const DirectParams p)
     const int wr = wave / QS;
     const int h = lane >> 5;
     const int j = lane & 31;
-    const int M = p.M, N = p.N;
+    const int M = p.M, N = p.N, lda = p.lda;
     const int bi = tile_m * MS + wr * MW;     // first row of this wave (may be >= M: loads nothing)
     const int bj = tile_n * NS + vec * 32;
 
-    const float* const Ablk = p.A + min(bi, M);
+    const float* const Ablk = p.A + min(bi, lda);
     const float* const Bvec = p.B + bj;
     const int32_t* const Dblk = p.D + (size_t)tile_n * p.W * QS;
     const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)tile_n * p.nwin * KS : nullptr;
-    // extents: the last dense row of a window ends with the matrix, the last kept row of B with
-    // this vector's 32 columns
-    const uint32_t a_bytes = bi < M ? (uint32_t)(((size_t)(KS - 1) * M + (size_t)(M - bi)) * sizeof(float)) : 0u;
+    // extents: the last dense row of a window ends with its lda floats (rows between M and lda are
+    // padding that may be read and is never stored), the last kept row of B with this vector's 32
+    // columns
+    const uint32_t a_bytes = bi < M ? (uint32_t)(((size_t)(KS - 1) * lda + (size_t)(lda - bi)) * sizeof(float)) : 0u;
     const uint32_t b_bytes = (uint32_t)(((size_t)(WS - 1) * N + 32) * sizeof(float));
-    const uint32_t row_bytes = (uint32_t)((size_t)M * sizeof(float));
+    const uint32_t row_bytes = (uint32_t)((size_t)lda * sizeof(float));
     const uint32_t a_vlane = (uint32_t)(j * 16);  // this lane's run of four rows inside the wave's rows
     const uint32_t b_chunk = (uint32_t)((size_t)CH * N * sizeof(float));
     uint32_t b_off[CS];
@@ -221,7 +223,7 @@ spmm_direct_kernel(const DirectParams p)
         take_meta();
         resolve_ranks();
         form_offsets(0);
-        const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w_begin * KS * M, a_bytes);
+        const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w_begin * KS * lda, a_bytes);
         const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)w_begin * WS * N, b_bytes);
 #pragma unroll
         for (int s = 0; s < CS; ++s)
@@ -244,7 +246,7 @@ spmm_direct_kernel(const DirectParams p)
             const int wl = wrap ? wn : w;
             const int cl = wrap ? 0 : c + 1;
             form_offsets(cl);
-            const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)wl * KS * M, a_bytes);
+            const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)wl * KS * lda, a_bytes);
             const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)wl * WS * N, b_bytes);
 #pragma unroll
             for (int s = 0; s < CS; ++s) {
@@ -290,6 +292,7 @@ static hipError_t launch_cfg(const SpmmArgs& a)
     p.out = a.split_k > 1 ? a.partial : a.C;
     p.slice_elems = a.slice_stride;
     p.M = a.M;
+    p.lda = a.lda;
     p.N = a.N;
     p.W = a.W;
     p.nwin = a.W / WS;
@@ -324,13 +327,13 @@ bool mfma_supported(const SpmmArgs& a)
 {
     if (a.vec_len != 32 || (a.Ns != 32 && a.Ns != 64 && a.Ns != 128))
         return false;
-    if (a.M % 4 != 0 || a.M < 32)
+    if (a.lda % 4 != 0 || a.lda < a.M || a.M < 32)
         return false;
     // 32-bit buffer offsets: one window of A and one window of B must stay below 2 GiB; the row
     // offset of A is formed with a 24-bit multiply
-    if ((size_t)a.window * a.M * sizeof(float) >= 0x80000000ull || (size_t)a.kept * a.N * sizeof(float) >= 0x80000000ull)
+    if ((size_t)a.window * a.lda * sizeof(float) >= 0x80000000ull || (size_t)a.kept * a.N * sizeof(float) >= 0x80000000ull)
         return false;
-    if ((size_t)a.M * sizeof(float) >= (1u << 24))
+    if ((size_t)a.lda * sizeof(float) >= (1u << 24))
         return false;
     // a wave's 256 rows of C are addressed with 32-bit offsets
     if ((size_t)256 * a.N * sizeof(float) >= 0x80000000ull)

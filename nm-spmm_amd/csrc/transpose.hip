@@ -8,11 +8,12 @@ namespace nmspmm {
 
 constexpr int kTile = 64;
 
-// dst[c][r] = src[r][c]; src is rows x cols, dst is cols x rows.  VEC: rows and cols are multiples
-// of 4 and both pointers 16-byte aligned.
+// dst[c * dst_ld + r] = src[r * cols + c]; src is rows x cols.  VEC: cols and dst_ld are multiples
+// of 4, dst_ld covers rows rounded up to 4 (the excess is written with zeros) and both pointers are
+// 16-byte aligned.
 template <bool VEC>
 __global__ void __launch_bounds__(256)
-transpose_kernel(const float* __restrict__ src, float* __restrict__ dst, int rows, int cols)
+transpose_kernel(const float* __restrict__ src, float* __restrict__ dst, int rows, int cols, int dst_ld)
 {
     __shared__ float tile[kTile][kTile + 1];
     const int r0 = blockIdx.y * kTile, c0 = blockIdx.x * kTile;
@@ -36,7 +37,7 @@ transpose_kernel(const float* __restrict__ src, float* __restrict__ dst, int row
             const int c = pass * 16 + (t >> 4);
             if (c0 + c < cols && r0 + q < rows) {
                 const float4 v = make_float4(tile[q][c], tile[q + 1][c], tile[q + 2][c], tile[q + 3][c]);
-                *reinterpret_cast<float4*>(dst + (size_t)(c0 + c) * rows + r0 + q) = v;
+                *reinterpret_cast<float4*>(dst + (size_t)(c0 + c) * dst_ld + r0 + q) = v;
             }
         }
     } else {
@@ -46,19 +47,20 @@ transpose_kernel(const float* __restrict__ src, float* __restrict__ dst, int row
         __syncthreads();
         for (int c = t >> 6; c < kTile; c += 4)
             if (c0 + c < cols && r0 + x < rows)
-                dst[(size_t)(c0 + c) * rows + r0 + x] = tile[x][c];
+                dst[(size_t)(c0 + c) * dst_ld + r0 + x] = tile[x][c];
     }
 }
 
-hipError_t launch_transpose(const float* src, float* dst, int rows, int cols, hipStream_t stream)
+hipError_t launch_transpose(const float* src, float* dst, int rows, int cols, int dst_ld, hipStream_t stream)
 {
     const dim3 grid((cols + kTile - 1) / kTile, (rows + kTile - 1) / kTile), block(256);
-    const bool vec = rows % 4 == 0 && cols % 4 == 0 &&
+    // a partial run of four rows at the bottom edge is stored whole: it lands in dst's padding
+    const bool vec = cols % 4 == 0 && dst_ld % 4 == 0 && dst_ld >= (rows + 3) / 4 * 4 &&
                      ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0;
     if (vec)
-        transpose_kernel<true><<<grid, block, 0, stream>>>(src, dst, rows, cols);
+        transpose_kernel<true><<<grid, block, 0, stream>>>(src, dst, rows, cols, dst_ld);
     else
-        transpose_kernel<false><<<grid, block, 0, stream>>>(src, dst, rows, cols);
+        transpose_kernel<false><<<grid, block, 0, stream>>>(src, dst, rows, cols, dst_ld);
     return hipGetLastError();
 }
 

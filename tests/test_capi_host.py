@@ -139,6 +139,7 @@ def test_rowmajor_entry_rejects_bad_arguments_without_a_gpu():
     L = nmspmm.lib()
     L.nmspmm_workspace_bytes_rowmajor.restype = ctypes.c_size_t
     assert L.nmspmm_workspace_bytes_rowmajor(64, 128, 256, 1) == 4 * 64 * 256
+    assert L.nmspmm_workspace_bytes_rowmajor(61, 128, 256, 1) == 4 * 64 * 256      # row pitch rounded up to 4
     assert L.nmspmm_workspace_bytes_rowmajor(64, 128, 256, 2) == 4 * 64 * 256 + L.nmspmm_workspace_bytes(64, 128, 2)
     assert L.nmspmm_workspace_bytes_rowmajor(0, 128, 256, 1) == 0
     assert L.nmspmm_transpose_device(None, 4, 4, FAKE, None) == 1
