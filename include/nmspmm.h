@@ -175,7 +175,7 @@ int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int
 int nmspmm_release(void);
 
 /* Name of the kernel family the last successful nmspmm_spmm call on this thread dispatched to
- * ("mfma", "skinny", "simt"), for tests and profiles.  Never NULL. */
+ * ("mfma", "short", "skinny", "simt"), for tests and profiles.  Never NULL. */
 const char* nmspmm_last_kernel(void);
 
 #ifdef __cplusplus

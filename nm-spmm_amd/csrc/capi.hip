@@ -349,7 +349,7 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     if (lda == 0 && M > 32 && M % 4 != 0) {
         // a padded copy of A is only worth making if it reaches the matrix-core kernel
         a.lda = (M + 3) / 4 * 4;
-        if (!mfma_supported(a))
+        if (!mfma_supported(a) && !short_supported(a))
             a.lda = M;
     }
     if (lda_out)
@@ -367,6 +367,9 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     if (mfma_supported(a)) {
         e = launch_mfma(a);
         g_last_kernel = "mfma";
+    } else if (short_supported(a)) {
+        e = launch_short(a);
+        g_last_kernel = "short";
     } else if (simt_supported(a)) {
         e = launch_simt(a);
         g_last_kernel = "simt";

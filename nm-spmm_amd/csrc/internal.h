@@ -68,6 +68,11 @@ inline int choose_wave_blocks(int M, int N, int nwin, int kept, int split)
 bool mfma_supported(const SpmmArgs& a);
 hipError_t launch_mfma(const SpmmArgs& a);
 
+// Matrix-core path for index vectors of 4, 8 or 16 columns (spmm_short.hip): low-sparsity layout,
+// windows of 4, 8 or 16 rows, N a multiple of 128, K a multiple of 16.
+bool short_supported(const SpmmArgs& a);
+hipError_t launch_short(const SpmmArgs& a);
+
 // Decode-sized path (spmm_skinny.hip): M <= 32, the reference geometries, no workspace needed.
 bool skinny_supported(const SpmmArgs& a);
 hipError_t launch_skinny(const SpmmArgs& a);

@@ -105,9 +105,10 @@ def test_decode_shape_8192(oracle, M):
 
 
 @pytest.mark.parametrize("vl,n,m", [(4, 2, 4), (8, 1, 8), (16, 3, 8)])
-def test_short_vectors_take_the_simt_path(oracle, vl, n, m):
-    """Per-vector length below 32: indices are used as generated (no widening), any window."""
-    M, N, K = 64, 128, 256
+def test_short_vectors_on_the_generic_kernel(oracle, vl, n, m):
+    """Per-vector length below 32 on a shape the matrix-core kernels do not take (64 columns):
+    indices are used as generated (no widening), any window."""
+    M, N, K = 64, 64, 256
     d = datagen.init_data(M, N, K, n, m, vec_len=vl, seed=vl)
     W, Q = d["W"], d["Q"]
     D = d["DT"].reshape(-1).copy()
@@ -116,6 +117,25 @@ def test_short_vectors_take_the_simt_path(oracle, vl, n, m):
     nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), None, C, M, N, K, W, m, n, vl, 64)
     torch.cuda.synchronize()
     assert nmspmm.last_kernel() == "simt"
+    check(oracle, d, C.cpu().numpy())
+
+
+@pytest.mark.parametrize("vl,n,m,Ns", [(4, 2, 4, 128), (4, 1, 4, 32), (4, 3, 4, 64), (8, 1, 8, 128), (8, 2, 8, 64), (16, 3, 8, 128),
+                                       (4, 4, 8, 128), (8, 2, 16, 32), (16, 4, 16, 64), (4, 8, 16, 128)])
+@pytest.mark.parametrize("M,split_k", [(64, 1), (256, 1), (300, 2), (132, 3)])
+def test_short_vectors_on_the_matrix_cores(oracle, vl, n, m, Ns, M, split_k):
+    """Vector lengths 4, 8 and 16 with windows of 4, 8 and 16 rows: the expanding MFMA kernel."""
+    N, K = 256, 512
+    d = datagen.init_data(M, N, K, n, m, vec_len=vl, seed=vl + n + M)
+    W, Q = d["W"], d["Q"]
+    D = d["DT"].reshape(-1).copy()
+    oracle.preprocess_low(D, W, Q, Ns, vl)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    ws = torch.empty(max(nmspmm.workspace_bytes(M, N, split_k) // 4, 1), dtype=torch.float32, device="cuda")
+    nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), None, C, M, N, K, W, m, n, vl, Ns, split_k,
+                ws if split_k > 1 else None)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == "short"
     check(oracle, d, C.cpu().numpy())
 
 
