@@ -358,7 +358,11 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
         return NMSPMM_OK;
 
     hipError_t e;
-    if (skinny_supported(a)) {
+    // up to 32 rows the decode kernel always wins; up to 128 it competes with the tile kernel at
+    // the caller's split
+    if (skinny_supported(a) && (M <= 32 || model_decode_seconds(M, N, W / kept, kept) <
+                                               model_tile_seconds(M, N, W / kept, kept, split_k) ||
+                                !mfma_supported(a))) {
         // one launch, reduction inside the workgroup: split_k and the workspace are not needed
         e = launch_skinny(a);
         g_last_kernel = "skinny";
@@ -493,25 +497,23 @@ int nmspmm_suggest_split_k(int M, int N, int W, int kept)
         return 0;
     if (M <= 32)
         return 1;  // the decode kernel reduces inside its workgroups
-    // The modelled time of the kernel (model_kernel_seconds, at the wave height the kernel would
-    // pick) plus, for a split, the second pass that moves (2 * split + 1) * M * N floats at about
-    // 5 TB/s and its launch; every launch has about 12 us of fixed cost (gap between launches,
-    // first loads, store of C).  Fitted to a sweep of M in 128..4096, N = K in 512..4096 at 2:4,
-    // 3:8, 2:8 and 1:8 on one MI355X: the choice is within 1 % of the best split on average,
-    // where never splitting loses 32 %.
+    // The split with the smallest modelled time of the tile kernel (model_tile_seconds); a finer
+    // split has to win by 3 %.  Fitted to sweeps of M in 48..4096, N and K in 512..14336 at 2:4,
+    // 3:8, 2:8 and 1:8 on one MI355X: the choice is within 1 % of the best split on average, where
+    // never splitting loses 32 %.  Up to 128 rows the one-launch decode kernel is the alternative;
+    // where its model is faster no split is needed.
     const int nwin = W / kept;
     int best = 1;
     double best_t = 0.0;
     for (int split = 1; split <= 16 && split <= nwin; split *= 2) {
-        const int blocks = choose_wave_blocks(M, N, nwin, kept, split);
-        double t = 12e-6 + model_kernel_seconds(M, N, nwin, kept, blocks, split);
-        if (split > 1)
-            t += (2.0 * split + 1.0) * M * N * sizeof(float) / 5e12 + 3e-6;
-        if (split == 1 || t < 0.97 * best_t) {  // a finer split has to win by 3 %
+        const double t = model_tile_seconds(M, N, nwin, kept, split);
+        if (split == 1 || t < 0.97 * best_t) {
             best = split;
             best_t = t;
         }
     }
+    if (M <= 128 && model_decode_seconds(M, N, nwin, kept) < best_t)
+        return 1;
     return best;
 }
 

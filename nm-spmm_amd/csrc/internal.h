@@ -42,7 +42,7 @@ __host__ __device__ inline void split_windows(int nwin, int split_k, int z, int*
 // CU holds four workgroups of 128-row waves or two of 256-row waves at once and they share its
 // pipes, so the 256 CUs retire the workgroups in rounds of 1024 or 512; the last, partial round
 // costs as much as its busiest CU, and a CU left with one workgroup (one wave per SIMD) runs at
-// about 0.8 of its rate.  Constants fitted to sweeps on one MI355X.
+// about 0.9 of its rate.  Constants fitted to sweeps on one MI355X (mean error 6 %).
 inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks, int split)
 {
     const double per_window = kept * 53.5e-9 * (blocks == 8 ? 2.0 / 1.04 : 1.0);
@@ -53,7 +53,7 @@ inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks,
     const long long busiest = (rest + 255) / 256;
     double t = (double)full * slots * unit;
     if (busiest > 0)
-        t += busiest * unit / (busiest == 1 && full == 0 ? 0.8 : 1.0);
+        t += busiest * unit / (busiest == 1 && full == 0 ? 0.9 : 1.0);
     return t;
 }
 // Wave height (32-row blocks) the matrix-core kernel uses for a shape: the faster one by the model.
@@ -62,6 +62,28 @@ inline int choose_wave_blocks(int M, int N, int nwin, int kept, int split)
     if (M <= 128)
         return 4;
     return model_kernel_seconds(M, N, nwin, kept, 8, split) < model_kernel_seconds(M, N, nwin, kept, 4, split) ? 8 : 4;
+}
+
+// Whole multiplication on the tile kernel: 6 us per launch, C written at about 8 TB/s, the kernel,
+// and for a split the second pass that moves (2 * split + 1) * M * N floats at about 8 TB/s (the
+// slices are cache resident) plus its launch.
+inline double model_tile_seconds(int M, int N, int nwin, int kept, int split)
+{
+    const double c_bytes = (double)M * N * sizeof(float);
+    double t = 6e-6 + c_bytes / 8e12 +
+               model_kernel_seconds(M, N, nwin, kept, choose_wave_blocks(M, N, nwin, kept, split), split);
+    if (split > 1)
+        t += (2.0 * split + 1.0) * c_bytes / 8e12 + 2e-6;
+    return t;
+}
+// Whole multiplication on the decode kernel (M <= 128): one workgroup per 32-column vector, 256
+// of them at a time, each needing kept/2 k-steps x (1, 2 or 4) MFMAs per window on the four
+// matrix pipes of its CU (4.2 ns per kept row and 32-row block, measured), plus 5 us.
+inline double model_decode_seconds(int M, int N, int nwin, int kept)
+{
+    const int blocks = M <= 32 ? 1 : M <= 64 ? 2 : 4;
+    const long long rounds = ((N + 31) / 32 + 255) / 256;
+    return 5e-6 + (double)rounds * nwin * kept * blocks * 4.2e-9;
 }
 
 // Matrix-core path (spmm_direct.hip).  Returns false when the geometry has no instantiation.

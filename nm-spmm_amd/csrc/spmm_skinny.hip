@@ -1,14 +1,17 @@
-// Decode-sized multiplication (M <= 32): the product is bound by streaming B from HBM once, so
-// the design goal is bytes in flight, not arithmetic.
+// Decode-sized multiplication (M <= 128): the product is bound by streaming B from HBM once (and,
+// towards 128 rows, by the matrix pipes), so the design goal is bytes in flight and a single launch.
 //
-//  * One workgroup per 32-column index vector; its waves split the reduction (the windows of
-//    the compressed K dimension) between them and sum their partial 32 x 32 results through LDS
-//    in wave order, so the result is deterministic and needs no workspace or second launch.
+//  * One workgroup per 32-column index vector; its waves split the reduction (the windows of the
+//    compressed K dimension) between them and sum their partial results through LDS in wave
+//    order, so the result is deterministic and needs no workspace or second launch.
+//  * A wave covers 32 * RB rows (RB = 1, 2 or 4 for M <= 32, 64, 128) with the rows interleaved
+//    (block b holds rows RB*r + b), so the A operands of all RB blocks of a k-step are one load of
+//    RB adjacent floats per lane and the B operand is reused RB times.
 //  * No LDS staging and no barrier in the streaming loop: each lane loads its own MFMA operands,
 //    B[2s+h][j] (two 128-byte row segments per wave and instruction, read exactly once from HBM)
-//    and A[i][k(2s+h)] (M contiguous floats per half wave, L2 resident), a whole chunk of
-//    windows ahead of the v_mfma_f32_32x32x2_f32 that consumes them; rows i >= M are
-//    out-of-range loads that return zero.
+//    and A[i][k(2s+h)] (L2 resident), a whole chunk of windows ahead of the
+//    v_mfma_f32_32x32x2_f32 that consumes them; rows i >= M are out-of-range loads that return
+//    zero, or neighbouring values that land in accumulators that are never stored.
 //  * Index metadata comes as one wave-wide load per window ([kept][Ns/32] ints, plus the 64-entry
 //    column_info list on the high-sparsity layout) and is handed to the lanes with ds_bpermute.
 #include "internal.h"
@@ -23,7 +26,7 @@ struct SkinnyParams {
     const int32_t* D;
     const int32_t* cinfo;
     float* C;
-    int M, N, W, K;
+    int M, N, W, K, lda;
     int nwin;
 };
 
@@ -36,25 +39,54 @@ __device__ inline float sk_load(__amdgpu_buffer_rsrc_t r, uint32_t off)
     return __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
 }
 
+// the A operands of one k-step: RB adjacent floats
+template <int RB> struct SkFrag { float v[RB]; };
+template <int RB> __device__ inline SkFrag<RB> sk_load_frag(__amdgpu_buffer_rsrc_t r, uint32_t off);
+template <> __device__ inline SkFrag<1> sk_load_frag<1>(__amdgpu_buffer_rsrc_t r, uint32_t off)
+{
+    SkFrag<1> f;
+    f.v[0] = sk_load(r, off);
+    return f;
+}
+template <> __device__ inline SkFrag<2> sk_load_frag<2>(__amdgpu_buffer_rsrc_t r, uint32_t off)
+{
+    auto x = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+    SkFrag<2> f;
+    f.v[0] = __int_as_float(x[0]);
+    f.v[1] = __int_as_float(x[1]);
+    return f;
+}
+template <> __device__ inline SkFrag<4> sk_load_frag<4>(__amdgpu_buffer_rsrc_t r, uint32_t off)
+{
+    auto x = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+    SkFrag<4> f;
+    f.v[0] = __int_as_float(x[0]);
+    f.v[1] = __int_as_float(x[1]);
+    f.v[2] = __int_as_float(x[2]);
+    f.v[3] = __int_as_float(x[3]);
+    return f;
+}
+
+#ifndef NMSPMM_SK_MAX_M
+#define NMSPMM_SK_MAX_M 128
+#endif
 #ifndef NMSPMM_SK_WAVES
 #define NMSPMM_SK_WAVES 8
 #endif
-#ifndef NMSPMM_SK_UMUL
-#define NMSPMM_SK_UMUL 1
-#endif
-#define NMSPMM_SK_U(u) ((u) * NMSPMM_SK_UMUL)
 constexpr int kSkinnyWaves = NMSPMM_SK_WAVES;
 constexpr uint32_t kSkNoLoad = 0x80000000u;
 
 // KS: dense rows per window, WS: kept rows per window, QS: column vectors per preprocessed column
-// block, HIGH: high-sparsity layout, U: windows per chunk (all loads of a chunk are in flight at once).
-template <int KS, int WS, int QS, bool HIGH, int U>
+// block, HIGH: high-sparsity layout, RB: 32-row blocks per wave, U: windows per chunk (all loads
+// of a chunk are in flight at once).
+template <int KS, int WS, int QS, bool HIGH, int RB, int U>
 __global__ void __launch_bounds__(64 * kSkinnyWaves)
 spmm_skinny_kernel(const SkinnyParams p)
 {
     constexpr int KSTEPS = WS / 2;
-    constexpr int STEPS = U * KSTEPS;          // MFMAs per chunk
+    constexpr int STEPS = U * KSTEPS;          // k-steps per chunk
     constexpr int ND = (WS * QS + 63) / 64;    // wave-wide loads per window of indices
+    typedef SkFrag<RB> afrag_t;
     __shared__ float red[kSkinnyWaves][16][64];
 
     const int tid = threadIdx.x;
@@ -65,7 +97,7 @@ spmm_skinny_kernel(const SkinnyParams p)
     const int vec_g = blockIdx.x;     // global column vector
     const int jb = vec_g / QS;        // preprocessed column block
     const int vec = vec_g % QS;       // vector inside it
-    const int M = p.M, N = p.N;
+    const int M = p.M, N = p.N, lda = p.lda;
 
     // windows of this wave: the same partition rule the large-tile kernels use for split-K
     int w_begin, w_count;
@@ -75,20 +107,26 @@ spmm_skinny_kernel(const SkinnyParams p)
     const float* const Bvec = p.B + (size_t)vec_g * 32;
     const int32_t* const Dblk = p.D + (size_t)jb * p.W * QS;
     const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)jb * p.nwin * KS : nullptr;
-    const uint32_t a_bytes = (uint32_t)((size_t)p.K * M * sizeof(float));
-    const uint32_t a_lane = j < M ? (uint32_t)(j * sizeof(float)) : kSkNoLoad;
+    const uint32_t a_bytes = (uint32_t)((size_t)p.K * lda * sizeof(float));
+    const uint32_t a_lane = RB * j < M ? (uint32_t)(RB * j * sizeof(float)) : kSkNoLoad;
+    const uint32_t row_bytes = (uint32_t)((size_t)lda * sizeof(float));
     const uint32_t b_lane = (uint32_t)(((size_t)h * N + j) * sizeof(float));
     const uint32_t b_step = (uint32_t)(2 * (size_t)N * sizeof(float));
     const uint32_t b_bytes = (uint32_t)(((size_t)(WS - 1) * N + 32) * sizeof(float));
+    const int perm_addr = (h * QS + vec) * (int)sizeof(int32_t);
 
-    floatx16 acc;
+    floatx16 acc[RB];
 #pragma unroll
-    for (int v = 0; v < 16; ++v)
-        acc[v] = 0.0f;
+    for (int b = 0; b < RB; ++b)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            acc[b][v] = 0.0f;
 
     int dvec[U][ND];
     int civec[U];
-    float a_nxt[STEPS], b_nxt[STEPS];
+    // two operand sets: one is multiplied while the other is in flight
+    afrag_t a0[STEPS], a1[STEPS];
+    float b0[STEPS], b1[STEPS];
 
     // metadata of the U windows starting at w (windows past the end are clamped; their operand
     // loads are suppressed below, so whatever they index contributes nothing)
@@ -109,7 +147,7 @@ spmm_skinny_kernel(const SkinnyParams p)
     // B operands of the U windows starting at w: addresses depend on nothing, so these go out first
     // and the HBM stream starts with the kernel.  A window past this wave's share loads nothing
     // (zero-sized descriptor) and so adds exact zeros.
-    auto load_b = [&](int w) {
+    auto load_b = [&](int w, float (&b_dst)[STEPS]) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int wu = w + u;
@@ -118,16 +156,14 @@ spmm_skinny_kernel(const SkinnyParams p)
             uint32_t boff = b_lane;
 #pragma unroll
             for (int s = 0; s < KSTEPS; ++s, boff += b_step)
-                b_nxt[u * KSTEPS + s] = sk_load(rb, boff);
+                b_dst[u * KSTEPS + s] = sk_load(rb, boff);
         }
     };
     // A operands of the same windows, from the metadata currently in dvec / civec.  Lane half h of
     // k-step s needs the dense row that index entry (2s + h) * QS + vec selects: ds_bpermute
     // fetches it from the lane that holds it (no LDS memory involved); on the high-sparsity layout
     // one more permute per window first turns all ranks into rows.
-    const int perm_addr = (h * QS + vec) * (int)sizeof(int32_t);
-    const uint32_t row_bytes = (uint32_t)((size_t)M * sizeof(float));
-    auto load_a = [&](int w) {
+    auto load_a = [&](int w, afrag_t (&a_dst)[STEPS]) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int wu = w + u;
@@ -141,56 +177,65 @@ spmm_skinny_kernel(const SkinnyParams p)
             for (int s = 0; s < KSTEPS; ++s) {
                 const int e = 2 * s * QS;
                 const int row = __builtin_amdgcn_ds_bpermute(perm_addr + (e % 64) * (int)sizeof(int32_t), dvec[u][e / 64]);
-                a_nxt[u * KSTEPS + s] = sk_load(ra_u, a_lane + (win_row + (uint32_t)row) * row_bytes);
+                a_dst[u * KSTEPS + s] = sk_load_frag<RB>(ra_u, a_lane + (win_row + (uint32_t)row) * row_bytes);
             }
         }
+    };
+    // one chunk: the next chunk's loads go out, then this chunk's operands are multiplied
+    auto chunk = [&](int w, afrag_t (&a_cur)[STEPS], float (&b_cur)[STEPS], afrag_t (&a_nxt)[STEPS],
+                     float (&b_nxt)[STEPS]) {
+        if (w + U < w_end) {
+            load_b(w + U, b_nxt);
+            load_a(w + U, a_nxt);
+            if (w + 2 * U < w_end)
+                load_meta(w + 2 * U);
+        }
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+            for (int b = 0; b < RB; ++b)
+                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_cur[s].v[b], b_cur[s], acc[b], 0, 0, 0);
     };
 
     // Load order per chunk: metadata, B, then (once the metadata has landed) A.  Loads return in
     // order, so waiting for the metadata never waits for the B stream issued after it.
     if (w_count > 0) {
         load_meta(w_begin);
-        load_b(w_begin);
-        load_a(w_begin);
+        load_b(w_begin, b0);
+        load_a(w_begin, a0);
         if (U < w_count)
             load_meta(w_begin + U);
     }
-    for (int w = w_begin; w < w_end; w += U) {
-        float a_cur[STEPS], b_cur[STEPS];
-#pragma unroll
-        for (int s = 0; s < STEPS; ++s) {
-            a_cur[s] = a_nxt[s];
-            b_cur[s] = b_nxt[s];
-        }
-        if (w + U < w_end) {
-            load_b(w + U);
-            load_a(w + U);
-            if (w + 2 * U < w_end)
-                load_meta(w + 2 * U);
-        }
-#pragma unroll
-        for (int s = 0; s < STEPS; ++s)
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_cur[s], b_cur[s], acc, 0, 0, 0);
+    for (int w = w_begin; w < w_end; w += 2 * U) {
+        chunk(w, a0, b0, a1, b1);
+        if (w + U < w_end)
+            chunk(w + U, a1, b1, a0, b0);
     }
 
-    // ---- sum the waves' partial tiles in wave order and store the M live rows ---------------------
+    // ---- sum the waves' partial tiles in wave order, one 32-row block at a time, and store the
+    // live rows.  Result register v of lane (h, j) is row 8*(v/4) + 4*h + v%4 of its block, column
+    // j; block b holds rows RB*r + b.
 #pragma unroll
-    for (int v = 0; v < 16; ++v)
-        red[wave][v][lane] = acc[v];
-    __syncthreads();
-    // wave v finishes result register v: rows 8*(v/4) + 4*h + v%4 (h = lane half), column j
-    for (int v = wave; v < 16; v += kSkinnyWaves) {
-        float s = red[0][v][lane];
+    for (int b = 0; b < RB; ++b) {
+        if (b > 0)
+            __syncthreads();
 #pragma unroll
-        for (int x = 1; x < kSkinnyWaves; ++x)
-            s += red[x][v][lane];
-        const int row = 8 * (v / 4) + 4 * h + (v % 4);
-        if (row < M)
-            p.C[(size_t)row * N + (size_t)vec_g * 32 + j] = s;
+        for (int v = 0; v < 16; ++v)
+            red[wave][v][lane] = acc[b][v];
+        __syncthreads();
+        for (int v = wave; v < 16; v += kSkinnyWaves) {
+            float s = red[0][v][lane];
+#pragma unroll
+            for (int x = 1; x < kSkinnyWaves; ++x)
+                s += red[x][v][lane];
+            const int row = RB * (8 * (v / 4) + 4 * h + (v % 4)) + b;
+            if (row < M)
+                p.C[(size_t)row * N + (size_t)vec_g * 32 + j] = s;
+        }
     }
 }
 
-template <int KS, int WS, bool HIGH, int U>
+template <int KS, int WS, bool HIGH, int RB, int U>
 static hipError_t launch_qs(const SpmmArgs& a)
 {
     SkinnyParams p;
@@ -203,39 +248,57 @@ static hipError_t launch_qs(const SpmmArgs& a)
     p.N = a.N;
     p.W = a.W;
     p.K = a.K;
+    p.lda = a.lda;
     p.nwin = a.W / WS;
     const dim3 grid(a.N / 32), block(64 * kSkinnyWaves);
     switch (a.Ns) {
-    case 128: spmm_skinny_kernel<KS, WS, 4, HIGH, U><<<grid, block, 0, a.stream>>>(p); break;
-    case 64: spmm_skinny_kernel<KS, WS, 2, HIGH, U><<<grid, block, 0, a.stream>>>(p); break;
-    case 32: spmm_skinny_kernel<KS, WS, 1, HIGH, U><<<grid, block, 0, a.stream>>>(p); break;
+    case 128: spmm_skinny_kernel<KS, WS, 4, HIGH, RB, U><<<grid, block, 0, a.stream>>>(p); break;
+    case 64: spmm_skinny_kernel<KS, WS, 2, HIGH, RB, U><<<grid, block, 0, a.stream>>>(p); break;
+    case 32: spmm_skinny_kernel<KS, WS, 1, HIGH, RB, U><<<grid, block, 0, a.stream>>>(p); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }
 
+// 32-row blocks per wave for a row count
+static int skinny_blocks(int M) { return M <= 32 ? 1 : M <= 64 ? 2 : 4; }
+
 bool skinny_supported(const SpmmArgs& a)
 {
-    if (a.M > 32 || a.vec_len != 32 || (a.Ns != 32 && a.Ns != 64 && a.Ns != 128))
+    if (a.M > NMSPMM_SK_MAX_M || a.vec_len != 32 || (a.Ns != 32 && a.Ns != 64 && a.Ns != 128))
         return false;
-    if ((size_t)a.K * a.M * sizeof(float) >= 0x80000000ull)
+    if (a.lda < a.M || a.lda % skinny_blocks(a.M) != 0)  // a lane's run of rows must not straddle the pitch
+        return false;
+    if ((size_t)a.K * a.lda * sizeof(float) >= 0x80000000ull)
         return false;
     const bool high = a.cinfo != nullptr;
     if (!high)
-        return a.window == 32 && (a.kept == 32 || a.kept == 16 || a.kept == 12);
+        return a.window == 32 && ((a.kept == 32 && a.M <= 32) || a.kept == 16 || a.kept == 12);
     return a.window == 64 && (a.kept == 16 || a.kept == 8);
+}
+
+// Windows per chunk: about forty operand registers in flight per set.
+template <int KS, int WS, bool HIGH, int U1>
+static hipError_t launch_rb(const SpmmArgs& a)
+{
+    constexpr int UN = U1 >= 4 ? U1 / 2 : 1;  // for 64 and 128 rows
+    switch (skinny_blocks(a.M)) {
+    case 1: return launch_qs<KS, WS, HIGH, 1, U1>(a);
+    case 2: return launch_qs<KS, WS, HIGH, 2, UN>(a);
+    default: return launch_qs<KS, WS, HIGH, 4, UN>(a);
+    }
 }
 
 hipError_t launch_skinny(const SpmmArgs& a)
 {
     const bool high = a.cinfo != nullptr;
     if (!high) {
-        if (a.kept == 32) return launch_qs<32, 32, false, NMSPMM_SK_U(1)>(a);
-        if (a.kept == 16) return launch_qs<32, 16, false, NMSPMM_SK_U(2)>(a);
-        if (a.kept == 12) return launch_qs<32, 12, false, NMSPMM_SK_U(2)>(a);
+        if (a.kept == 32) return launch_qs<32, 32, false, 1, 1>(a);
+        if (a.kept == 16) return launch_rb<32, 16, false, 2>(a);
+        if (a.kept == 12) return launch_rb<32, 12, false, 2>(a);
     } else {
-        if (a.kept == 16) return launch_qs<64, 16, true, NMSPMM_SK_U(2)>(a);
-        if (a.kept == 8) return launch_qs<64, 8, true, NMSPMM_SK_U(4)>(a);
+        if (a.kept == 16) return launch_rb<64, 16, true, 2>(a);
+        if (a.kept == 8) return launch_rb<64, 8, true, 4>(a);
     }
     return hipErrorInvalidValue;
 }

@@ -67,6 +67,25 @@ def test_config1_512_cubed_2of4(oracle):
 def test_ragged_row_counts(oracle, M, n, m, Ns):
     d = datagen.init_data(M, 256, 256, n, m, seed=M + n)
     got, fam = run_gpu(oracle, d, Ns)
+    assert fam == "mfma" if M > 128 else fam in ("mfma", "skinny")   # up to 128 rows the two kernels compete
+    check(oracle, d, got)
+
+
+@pytest.mark.parametrize("M", [34, 48, 64, 68, 96, 100, 128])
+@pytest.mark.parametrize("n,m,Ns", [(1, 8, 128), (2, 8, 64), (2, 4, 32), (3, 8, 128)])
+def test_decode_kernel_up_to_128_rows(oracle, M, n, m, Ns):
+    """Two and four 32-row blocks per wave; K gives the waves of a workgroup unequal shares.  The
+    shape (many columns, short reduction) is one where the run-time model prefers this kernel."""
+    K = 512 if m == 8 else 576
+    d = datagen.init_data(M, 8192, K, n, m, seed=M + Ns, dist="normal", b_scale=0.02)
+    got, fam = run_gpu(oracle, d, Ns)
+    assert fam == "skinny"
+    check(oracle, d, got)
+
+
+def test_dense_pattern_above_32_rows_stays_on_the_tile_kernel(oracle):
+    d = datagen.init_data(64, 128, 256, 32, 32, seed=5)
+    got, fam = run_gpu(oracle, d, 128)
     assert fam == "mfma"
     check(oracle, d, got)
 
@@ -74,7 +93,7 @@ def test_ragged_row_counts(oracle, M, n, m, Ns):
 @pytest.mark.parametrize("split_k", [2, 3, 4, 8, 16])
 @pytest.mark.parametrize("n,m,Ns", [(2, 4, 128), (1, 8, 128), (2, 8, 32)])
 def test_split_k_through_workspace(oracle, split_k, n, m, Ns):
-    d = datagen.init_data(128, 256, 1280, n, m, seed=split_k)  # 40 or 20 windows: uneven splits included
+    d = datagen.init_data(160, 256, 1280, n, m, seed=split_k)  # 40 or 20 windows: uneven splits included
     got, _ = run_gpu(oracle, d, Ns, split_k)
     check(oracle, d, got)
     one, _ = run_gpu(oracle, d, Ns, 1)
@@ -162,7 +181,7 @@ def test_named_entry_points_with_gpu_preprocessing(oracle, sparsity, n, m, tile)
     check(oracle, d, C.cpu().numpy())
 
 
-@pytest.mark.parametrize("M,N,K,n,m,sparsity", [(128, 1024, 2048, 2, 4, 0.5), (256, 512, 4096, 2, 8, 0.75),
+@pytest.mark.parametrize("M,N,K,n,m,sparsity", [(160, 1024, 2048, 2, 4, 0.5), (256, 512, 4096, 2, 8, 0.75),
                                                  (512, 1024, 1024, 1, 8, 0.875), (2048, 2048, 512, 3, 8, 0.625),
                                                  (16, 512, 2048, 2, 8, 0.75)])
 def test_auto_entry_point_chooses_the_split_itself(oracle, M, N, K, n, m, sparsity):
@@ -174,8 +193,8 @@ def test_auto_entry_point_chooses_the_split_itself(oracle, M, N, K, n, m, sparsi
     torch.cuda.synchronize()
     split = nmspmm.suggest_split_k(M, N, d["W"], kept)
     assert 1 <= split <= 16 and (d["W"] // kept) // split >= 1
-    if M == 128 and K == 2048:
-        assert split > 1          # 128 waves for 1024 SIMDs: the reduction must be split
+    if M == 160 and K == 2048:
+        assert split > 1          # 64 workgroups for 256 CUs: the reduction must be split
     if M == 2048 or M <= 32:
         assert split == 1
     check(oracle, d, C.cpu().numpy())
