@@ -117,11 +117,19 @@ int nmspmm_decompress_device(const float* dBT, const int32_t* dDT, int K, int N,
  * split_k partial M x N fp32 results that a second pass sums in a fixed order. */
 size_t nmspmm_workspace_bytes(int M, int N, int split_k);
 
+/* Bytes of optional scratch with which nmspmm_spmm, called with split_k == 1 and Ns == 128, cuts
+ * the tiles of a ragged last round along K so that they fill the GPU once more (0 when there is
+ * nothing to gain: a 2752-tile problem on 512 tile slots leaves 192 tiles for a sixth round that a
+ * quarter of the CUs would run alone).  No counterpart in the reference. */
+size_t nmspmm_tail_workspace_bytes(int M, int N, int W, int kept);
+
 /* General entry point: C = A . B for one (window, kept, vec_len, Ns) geometry.
  * column_info == NULL selects the low-sparsity layout (all window rows staged), non-NULL the
  * high-sparsity layout (only the rows column_info lists are staged, D holds ranks).
  * split_k > 1 requires `workspace` of at least nmspmm_workspace_bytes(); unlike the reference's
- * atomicAdd reduction (include/ptx.h:34-40) C is overwritten, not accumulated into.
+ * atomicAdd reduction (include/ptx.h:34-40) C is overwritten, not accumulated into.  With
+ * split_k == 1 the workspace is optional: NULL, or nmspmm_tail_workspace_bytes() bytes (16-byte
+ * aligned) that enable the tail split; a smaller one is ignored.
  * Requirements: N % Ns == 0, Ns % vec_len == 0, W % kept == 0, 1 <= split_k <= W / kept,
  * K * kept == W * window, 16-byte aligned A, B and C. */
 int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t* column_info,

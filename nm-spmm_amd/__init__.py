@@ -54,6 +54,8 @@ def lib():
         L.nmspmm_decompress_device.argtypes = [c_void_p, c_void_p] + [c_int] * 5 + [c_void_p, c_void_p]
         L.nmspmm_column_info_ints.restype = c_size_t
         L.nmspmm_column_info_ints.argtypes = [c_int] * 5
+        L.nmspmm_tail_workspace_bytes.restype = c_size_t
+        L.nmspmm_tail_workspace_bytes.argtypes = [c_int] * 4
         L.nmspmm_workspace_bytes.restype = c_size_t
         L.nmspmm_workspace_bytes.argtypes = [c_int] * 3
         L.nmspmm_spmm.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, c_void_p]
@@ -128,6 +130,10 @@ def decompress_device(dBT, dDT, K, N, n, m, dB, vec_len=32):
 
 def column_info_ints(W, pN, pM, N, Ns):
     return lib().nmspmm_column_info_ints(W, pN, pM, N, Ns)
+
+
+def tail_workspace_bytes(M, N, W, kept):
+    return lib().nmspmm_tail_workspace_bytes(M, N, W, kept)
 
 
 def workspace_bytes(M, N, split_k):

@@ -294,6 +294,13 @@ int nmspmm_decompress_device(const float* dBT, const int32_t* dDT, int K, int N,
                                                                                                      : NMSPMM_ERR_HIP;
 }
 
+size_t nmspmm_tail_workspace_bytes(int M, int N, int W, int kept)
+{
+    if (M <= 128 || N <= 0 || W <= 0 || kept <= 0 || W % kept != 0)
+        return 0;
+    return plan_tail(M, N, W / kept, kept).ws_bytes;
+}
+
 size_t nmspmm_workspace_bytes(int M, int N, int split_k)
 {
     if (M <= 0 || N <= 0 || split_k <= 1)
@@ -344,6 +351,10 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     a.vec_len = vec_len;
     a.Ns = Ns;
     a.split_k = split_k;
+    // without a split the workspace, if any, serves the tail split of the tile kernel
+    const bool scratch = split_k == 1 && workspace != nullptr && aligned16(workspace);
+    a.tail_ws = scratch ? (float*)workspace : nullptr;
+    a.tail_ws_bytes = scratch ? workspace_bytes : 0;
     a.stream = (hipStream_t)stream;
 
     if (lda == 0 && M > 32 && M % 4 != 0) {
@@ -428,14 +439,14 @@ int nmspmm_spmm_rowmajor(const float* A_rowmajor, const float* B, const int32_t*
     const size_t slice_bytes = workspace_bytes - sizeof(float) * rowmajor_copy_floats(M, K);
     // check every argument and settle the row pitch of the copy before anything is launched
     int lda = M;
-    const int st = spmm_impl(At, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k,
-                             split_k > 1 ? slices : nullptr, split_k > 1 ? slice_bytes : 0, stream, 0, true, &lda);
+    const int st = spmm_impl(At, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k, slices,
+                             slice_bytes, stream, 0, true, &lda);
     if (st != NMSPMM_OK)
         return st;
     if (launch_transpose(A_rowmajor, At, M, K, lda, (hipStream_t)stream) != hipSuccess)
         return NMSPMM_ERR_HIP;
-    return spmm_impl(At, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k,
-                     split_k > 1 ? slices : nullptr, split_k > 1 ? slice_bytes : 0, stream, lda, false, nullptr);
+    return spmm_impl(At, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k, slices, slice_bytes,
+                     stream, lda, false, nullptr);
 }
 
 int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C, int M,
@@ -467,9 +478,9 @@ static int named_gemm(int want_high, int tile, const float* A, const float* B, c
     if (split_k < 1 || split_k > W / kept)
         return NMSPMM_ERR_BAD_SPLIT;
     void* ws = nullptr;
-    size_t ws_bytes = 0;
-    if (split_k > 1) {
-        ws_bytes = nmspmm_workspace_bytes(M, N, split_k);
+    size_t ws_bytes = split_k > 1 ? nmspmm_workspace_bytes(M, N, split_k)
+                                  : (tile == 128 ? nmspmm_tail_workspace_bytes(M, N, W, kept) : 0);
+    if (ws_bytes > 0) {
         const int rc = cached_workspace(ws_bytes, &ws);
         if (rc != NMSPMM_OK)
             return rc;

@@ -22,6 +22,8 @@ struct SpmmArgs {
                            // row-major A was padded (matrix-core path only)
     int window, kept, vec_len, Ns;
     int split_k;
+    float* tail_ws;        // optional scratch for splitting the tiles of a ragged last round (split_k == 1)
+    size_t tail_ws_bytes;
     hipStream_t stream;
 };
 
@@ -40,9 +42,10 @@ __host__ __device__ inline void split_windows(int nwin, int split_k, int z, int*
 // 32*blocks rows x 128 columns; per window it needs kept/2 k-steps x blocks MFMAs x 64 cycles of
 // each of its CU's four matrix pipes (2.39 GHz; 256-row waves spend about 4 % less on loads).  A
 // CU holds four workgroups of 128-row waves or two of 256-row waves at once and they share its
-// pipes, so the 256 CUs retire the workgroups in rounds of 1024 or 512; the last, partial round
-// costs as much as its busiest CU, and a CU left with one workgroup (one wave per SIMD) runs at
-// about 0.9 of its rate.  Constants fitted to sweeps on one MI355X (mean error 6 %).
+// pipes, so the 256 CUs retire the workgroups in rounds of 1024 or 512.  After one full round the
+// leftovers spread over the CUs and cost as much as the busiest CU (a CU left with one workgroup,
+// one wave per SIMD, runs at about 0.9 of its rate); after two or more the leftovers land packed
+// on the CUs that happen to free up and cost a whole round.  Constants fitted to sweeps on one MI355X (mean error 6 %).
 inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks, int split)
 {
     const double per_window = kept * 53.5e-9 * (blocks == 8 ? 2.0 / 1.04 : 1.0);
@@ -53,7 +56,7 @@ inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks,
     const long long busiest = (rest + 255) / 256;
     double t = (double)full * slots * unit;
     if (busiest > 0)
-        t += busiest * unit / (busiest == 1 && full == 0 ? 0.9 : 1.0);
+        t += full >= 2 ? slots * unit : busiest * unit / (busiest == 1 && full == 0 ? 0.9 : 1.0);
     return t;
 }
 // Wave height (32-row blocks) the matrix-core kernel uses for a shape: the faster one by the model.
@@ -62,6 +65,52 @@ inline int choose_wave_blocks(int M, int N, int nwin, int kept, int split)
     if (M <= 128)
         return 4;
     return model_kernel_seconds(M, N, nwin, kept, 8, split) < model_kernel_seconds(M, N, nwin, kept, 4, split) ? 8 : 4;
+}
+
+// Tail split of the tile kernel (split_k == 1): the 256 CUs retire 128 x 128 tiles 1024 at a time
+// (256 x 128 tiles 512 at a time); when the last round is ragged, its `tail` tiles are cut into
+// `slices` pieces along K so that they fill the machine once more, written to scratch and summed
+// by a small second kernel.  slices == 1 means no split.
+struct TailPlan {
+    int blocks;      // 32-row blocks per wave (4 or 8)
+    long long head;  // tiles computed whole
+    long long tail;  // tiles computed in slices
+    int slices;
+    size_t ws_bytes; // scratch needed
+};
+inline TailPlan plan_tail(int M, int N, int nwin, int kept)
+{
+    TailPlan t;
+    t.blocks = choose_wave_blocks(M, N, nwin, kept, 1);
+    const long long tiles = (long long)((M + 32 * t.blocks - 1) / (32 * t.blocks)) * ((N + 127) / 128);
+    const long long slots = 256LL * (t.blocks == 8 ? 2 : 4);
+    t.head = tiles;
+    t.tail = 0;
+    t.slices = 1;
+    t.ws_bytes = 0;
+    const long long rest = tiles % slots;
+    if (tiles < slots || rest == 0)
+        return t;
+    // In steady state (two or more full rounds) workgroups finish at staggered times and the
+    // dispatcher refills a CU's freed slots together, so the leftover tiles end up packed on few
+    // CUs and the last round lasts as long as a full one (measured: 2752 tiles on 512 slots take six
+    // rounds, not 5.4).  Cutting each leftover tile into floor(slots / rest) pieces keeps them in
+    // one round of proportionally shorter pieces.  After a single full round the leftovers spread
+    // over idle CUs by themselves and the second pass costs more than it saves (measured).
+    if (tiles < 2 * slots)
+        return t;
+    int slices = (int)(slots / rest);
+    if (slices > 4)
+        slices = 4;  // the scratch grows with the number of pieces
+    while (slices > 1 && nwin / slices < 4)
+        --slices;
+    if (slices < 2)
+        return t;
+    t.head = tiles - rest;
+    t.tail = rest;
+    t.slices = slices;
+    t.ws_bytes = (size_t)rest * slices * (32 * t.blocks) * 128 * sizeof(float);
+    return t;
 }
 
 // Whole multiplication on the tile kernel: 6 us per launch, C written at about 8 TB/s, the kernel,
@@ -89,6 +138,8 @@ inline double model_decode_seconds(int M, int N, int nwin, int kept)
 // Matrix-core path (spmm_direct.hip).  Returns false when the geometry has no instantiation.
 bool mfma_supported(const SpmmArgs& a);
 hipError_t launch_mfma(const SpmmArgs& a);
+// Scratch bytes with which launch_mfma splits a ragged last round (0: nothing to gain or unsupported).
+size_t mfma_tail_workspace_bytes(const SpmmArgs& a);
 
 // Matrix-core path for index vectors of 4, 8 or 16 columns (spmm_short.hip): low-sparsity layout,
 // windows of 4, 8 or 16 rows, N a multiple of 128, K a multiple of 16.

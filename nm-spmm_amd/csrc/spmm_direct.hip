@@ -47,6 +47,9 @@ struct DirectParams {
     int nwin;            // windows in the whole reduction
     int split_k;
     int tiles_m, tiles_n;
+    int head_tiles;      // tiles computed whole; the rest are cut into tail_slices pieces along K
+    int tail_slices;     // 1: no tail split
+    float* tail_ws;      // [tail tile][slice][MS][NS] partial tiles
 };
 
 struct float8 { float4 lo, hi; };
@@ -105,14 +108,19 @@ spmm_direct_kernel(const DirectParams p)
     static_assert(WS % CH == 0, "whole chunks");
 
     // ---- tile walk: consecutive ids go to different XCDs, so give each XCD a contiguous run of
-    // logical tiles, walked in bands of GROUP row tiles across all column blocks.
-    const int total = p.tiles_m * p.tiles_n;
+    // logical tiles, walked in bands of GROUP row tiles across all column blocks.  Ids beyond the
+    // head tiles are slices of the tail tiles (a ragged last round cut along K).
+    const bool tail_unit = p.tail_slices > 1 && (int)blockIdx.x >= p.head_tiles;
+    const int unit = (int)blockIdx.x - p.head_tiles;  // slice number among the tail slices
     int logical;
-    {
+    if (!tail_unit) {
+        const int total = p.tail_slices > 1 ? p.head_tiles : p.tiles_m * p.tiles_n;
         const int id = blockIdx.x;
         const int q = total / kXcds, r = total % kXcds;
         const int xcd = id % kXcds, loc = id / kXcds;
         logical = xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc;
+    } else {
+        logical = p.head_tiles + unit / p.tail_slices;
     }
     constexpr int GROUP = NMSPMM_GROUP;
     int tile_m, tile_n;
@@ -125,7 +133,10 @@ spmm_direct_kernel(const DirectParams p)
         tile_n = in_band / rows;
     }
     int w_begin, w_count;
-    split_windows(p.nwin, p.split_k, blockIdx.y, &w_begin, &w_count);
+    if (!tail_unit)
+        split_windows(p.nwin, p.split_k, blockIdx.y, &w_begin, &w_count);
+    else
+        split_windows(p.nwin, p.tail_slices, unit % p.tail_slices, &w_begin, &w_count);
     const int w_last = w_begin + w_count - 1;
 
     const int lane = threadIdx.x & 63;
@@ -264,12 +275,16 @@ spmm_direct_kernel(const DirectParams p)
     // column j; block b of the wave holds rows (b/4)*128 + 4*r + b%4.  Stores go through a
     // descriptor that ends with the last live row of this wave, so rows beyond M are dropped
     // without a branch; the per-register part of the offset is a scalar.
+    // A slice of a tail tile goes to its own MS x NS block of the scratch instead, all rows.
     float* const out = p.out + (size_t)blockIdx.y * p.slice_elems;
-    const int rows_here = min(M - bi, MW);
-    const uint32_t c_bytes = rows_here > 0 ? (uint32_t)(((size_t)(rows_here - 1) * N + 32) * sizeof(float)) : 0u;
-    const __amdgpu_buffer_rsrc_t rc = make_rsrc(out + (size_t)min(bi, M) * N + bj, c_bytes);
-    const uint32_t c_lane = (uint32_t)(((size_t)16 * h * N + j) * sizeof(float));
-    const uint32_t n_bytes = (uint32_t)((size_t)N * sizeof(float));
+    const int pitch = tail_unit ? NS : N;
+    const int rows_here = tail_unit ? MW : min(M - bi, MW);
+    float* const c_base = tail_unit ? p.tail_ws + ((size_t)unit * MS + wr * MW) * NS + vec * 32
+                                    : out + (size_t)min(bi, M) * N + bj;
+    const uint32_t c_bytes = rows_here > 0 ? (uint32_t)(((size_t)(rows_here - 1) * pitch + 32) * sizeof(float)) : 0u;
+    const __amdgpu_buffer_rsrc_t rc = make_rsrc(c_base, c_bytes);
+    const uint32_t c_lane = (uint32_t)(((size_t)16 * h * pitch + j) * sizeof(float));
+    const uint32_t n_bytes = (uint32_t)((size_t)pitch * sizeof(float));
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
 #pragma unroll
@@ -280,10 +295,45 @@ spmm_direct_kernel(const DirectParams p)
     }
 }
 
+// Sums the slices of the tail tiles in slice order into C (second pass of the tail split).  One
+// workgroup per tail tile; the tile is found by the same walk as in the main kernel.
+template <int MS, int NS>
+__global__ void __launch_bounds__(256)
+tail_reduce_kernel(const float* __restrict__ ws, float* __restrict__ C, int M, int N, int tiles_m, int tiles_n,
+                   int head_tiles, int slices)
+{
+    constexpr int GROUP = NMSPMM_GROUP;
+    const int logical = head_tiles + blockIdx.x;
+    const int band = logical / (GROUP * tiles_n);
+    const int first_m = band * GROUP;
+    const int rows = min(GROUP, tiles_m - first_m);
+    const int in_band = logical - band * GROUP * tiles_n;
+    const int tile_m = first_m + in_band % rows;
+    const int tile_n = in_band / rows;
+    const float* const src = ws + (size_t)blockIdx.x * slices * MS * NS;
+    constexpr int F4_ROW = NS / 4;
+    for (int e = threadIdx.x; e < MS * F4_ROW; e += 256) {
+        const int r = e / F4_ROW, c4 = e % F4_ROW;
+        const int row = tile_m * MS + r;
+        if (row >= M)
+            break;  // rows grow with e
+        float4 sum = reinterpret_cast<const float4*>(src)[e];
+        for (int z = 1; z < slices; ++z) {
+            const float4 v = reinterpret_cast<const float4*>(src + (size_t)z * MS * NS)[e];
+            sum.x += v.x;
+            sum.y += v.y;
+            sum.z += v.z;
+            sum.w += v.w;
+        }
+        *reinterpret_cast<float4*>(C + (size_t)row * N + (size_t)tile_n * NS + c4 * 4) = sum;
+    }
+}
+
 template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
-static hipError_t launch_cfg(const SpmmArgs& a)
+static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
 {
     constexpr int MS = WR * RM * 32;
+    constexpr int NS = QS * 32;
     DirectParams p;
     p.A = a.A;
     p.B = a.B;
@@ -298,29 +348,71 @@ static hipError_t launch_cfg(const SpmmArgs& a)
     p.nwin = a.W / WS;
     p.split_k = a.split_k;
     p.tiles_m = (a.M + MS - 1) / MS;
-    p.tiles_n = a.N / (QS * 32);
-    const dim3 grid(p.tiles_m * p.tiles_n, a.split_k, 1);
+    p.tiles_n = a.N / NS;
+    p.head_tiles = p.tiles_m * p.tiles_n;
+    p.tail_slices = 1;
+    p.tail_ws = nullptr;
+    // the plan counts 128-column tiles of RM blocks; it applies when that is this tile shape
+    const bool split_tail = plan.slices > 1 && WR == 1 && QS == 4 && RM == plan.blocks;
+    dim3 grid(p.tiles_m * p.tiles_n, a.split_k, 1);
+    if (split_tail) {
+        p.head_tiles = (int)plan.head;
+        p.tail_slices = plan.slices;
+        p.tail_ws = a.tail_ws;
+        grid.x = (unsigned)(plan.head + plan.tail * plan.slices);
+    }
     spmm_direct_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, dim3(64 * QS * WR), 0, a.stream>>>(p);
-    return hipGetLastError();
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess && split_tail) {
+        tail_reduce_kernel<MS, NS><<<dim3((unsigned)plan.tail), dim3(256), 0, a.stream>>>(
+            a.tail_ws, a.C, a.M, a.N, p.tiles_m, p.tiles_n, p.head_tiles, plan.slices);
+        e = hipGetLastError();
+    }
+    return e;
 }
 
 // Every workgroup has four waves: 1 x 4, 2 x 2 or 4 x 1 (rows x column vectors), chosen by the
 // column-block width the indices were preprocessed for.  A wave is 256 or 128 rows tall, whichever
 // the run-time model expects to finish first: the taller wave halves the B and index loads per
 // MFMA, but only two such workgroups fit a CU, which quantises badly on mid-sized problems.
+// The tail split is planned for 128-wide column blocks and a single reduction slice, and used
+// when the caller's scratch holds it.
+static TailPlan tail_plan_for(const SpmmArgs& a, bool have_scratch)
+{
+    TailPlan none;
+    none.blocks = choose_wave_blocks(a.M, a.N, a.W / a.kept, a.kept, a.split_k);
+    none.head = none.tail = 0;
+    none.slices = 1;
+    none.ws_bytes = 0;
+    if (a.split_k != 1 || a.Ns != 128 || NMSPMM_RM_TALL != 8)
+        return none;
+    const TailPlan t = plan_tail(a.M, a.N, a.W / a.kept, a.kept);
+    if (t.slices < 2 || t.head + t.tail * t.slices > 0x7fffffffLL)
+        return none;
+    if (have_scratch && (a.tail_ws == nullptr || a.tail_ws_bytes < t.ws_bytes))
+        return none;
+    return t;
+}
+
 template <int KS, int WS, bool HIGH>
 static hipError_t launch_ns(const SpmmArgs& a)
 {
-    const bool tall = NMSPMM_RM_TALL == 8 && choose_wave_blocks(a.M, a.N, a.W / WS, WS, a.split_k) == 8;
+    const TailPlan plan = tail_plan_for(a, true);
+    const bool tall = NMSPMM_RM_TALL == 8 && plan.blocks == 8;
     switch (a.Ns) {
     case 128:
-        return tall ? launch_cfg<KS, WS, 4, 1, NMSPMM_RM_TALL, HIGH>(a) : launch_cfg<KS, WS, 4, 1, 4, HIGH>(a);
+        return tall ? launch_cfg<KS, WS, 4, 1, NMSPMM_RM_TALL, HIGH>(a, plan) : launch_cfg<KS, WS, 4, 1, 4, HIGH>(a, plan);
     case 64:
-        return tall ? launch_cfg<KS, WS, 2, 2, NMSPMM_RM_TALL, HIGH>(a) : launch_cfg<KS, WS, 2, 2, 4, HIGH>(a);
+        return tall ? launch_cfg<KS, WS, 2, 2, NMSPMM_RM_TALL, HIGH>(a, plan) : launch_cfg<KS, WS, 2, 2, 4, HIGH>(a, plan);
     case 32:
-        return tall ? launch_cfg<KS, WS, 1, 4, NMSPMM_RM_TALL, HIGH>(a) : launch_cfg<KS, WS, 1, 4, 4, HIGH>(a);
+        return tall ? launch_cfg<KS, WS, 1, 4, NMSPMM_RM_TALL, HIGH>(a, plan) : launch_cfg<KS, WS, 1, 4, 4, HIGH>(a, plan);
     }
     return hipErrorInvalidValue;
+}
+
+size_t mfma_tail_workspace_bytes(const SpmmArgs& a)
+{
+    return mfma_supported(a) ? tail_plan_for(a, false).ws_bytes : 0;
 }
 
 bool mfma_supported(const SpmmArgs& a)

@@ -200,6 +200,33 @@ def test_auto_entry_point_chooses_the_split_itself(oracle, M, N, K, n, m, sparsi
     check(oracle, d, C.cpu().numpy())
 
 
+@pytest.mark.parametrize("M,N,K,n,m", [(4096, 8448, 512, 2, 8), (8192, 4224, 1024, 2, 4), (4096, 8448, 512, 1, 8)])
+def test_ragged_last_round_is_split_along_k_through_scratch(oracle, M, N, K, n, m):
+    """More tiles than the GPU holds at once and a ragged last round: with scratch the tiles of that
+    round are cut along K and summed by a second kernel; the result matches the checker either way."""
+    d = datagen.init_data(M, N, K, n, m, seed=M + N)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    need = nmspmm.tail_workspace_bytes(M, N, d["W"], kept)
+    assert need > 0
+    A, B, Dd = dev(d["A_km"]), dev(d["BT"]), dev(D)
+    ci = None if cinfo is None else dev(cinfo)
+    ws = torch.full((need // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    outs = []
+    for scratch in (ws, None, ws[: need // 4 - 64]):       # enough, none, too little (ignored)
+        C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        nmspmm.spmm(A, B, Dd, ci, C, M, N, K, d["W"], window, kept, 32, 128, 1, scratch)
+        torch.cuda.synchronize()
+        assert nmspmm.last_kernel() == "mfma" and bool(torch.isfinite(C).all())
+        outs.append(C)
+    assert torch.equal(outs[1], outs[2])                    # both ran without the split
+    assert not torch.equal(outs[0], outs[1])                # the split sums in a different order
+    for (r0, r1) in ((0, 24), (M // 2 - 8, M // 2 + 8), (M - 16, M)):
+        want = oracle.gemm_cpu(d["A_km"].reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), M, N, d["W"],
+                               rows=(r0, r1)).reshape(M, N)[r0:r1]
+        for C in outs[:2]:
+            assert scaled_max_error(C[r0:r1].cpu().numpy(), want) <= REL_TOL
+
+
 def test_llm_layer_shape_2of8(oracle):
     """One BASELINE config-3 shape (M = 512, K = 4096, Ncols = 11008, 2:8, N(0,1) x N(0,0.02^2))."""
     d = datagen.init_data(512, 11008, 4096, 2, 8, seed=3001, dist="normal", b_scale=0.02)
