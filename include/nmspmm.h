@@ -118,9 +118,8 @@ int nmspmm_decompress_device(const float* dBT, const int32_t* dDT, int K, int N,
 size_t nmspmm_workspace_bytes(int M, int N, int split_k);
 
 /* Bytes of optional scratch with which nmspmm_spmm, called with split_k == 1 and Ns == 128, cuts
- * the tiles of a ragged last round along K so that they fill the GPU once more (0 when there is
- * nothing to gain: a 2752-tile problem on 512 tile slots leaves 192 tiles for a sixth round that a
- * quarter of the CUs would run alone).  No counterpart in the reference. */
+ * the few leftover tiles of a ragged last round into four pieces along K so that they occupy four
+ * times as many CUs (0 when there is nothing to gain).  No counterpart in the reference. */
 size_t nmspmm_tail_workspace_bytes(int M, int N, int W, int kept);
 
 /* General entry point: C = A . B for one (window, kept, vec_len, Ns) geometry.

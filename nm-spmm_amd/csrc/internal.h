@@ -45,7 +45,8 @@ __host__ __device__ inline void split_windows(int nwin, int split_k, int z, int*
 // pipes, so the 256 CUs retire the workgroups in rounds of 1024 or 512.  After one full round the
 // leftovers spread over the CUs and cost as much as the busiest CU (a CU left with one workgroup,
 // one wave per SIMD, runs at about 0.9 of its rate); after two or more the leftovers land packed
-// on the CUs that happen to free up and cost a whole round.  Constants fitted to sweeps on one MI355X (mean error 6 %).
+// on the CUs that happen to free up and cost a whole round, unless they are few enough to get a
+// launch of their own (plan_tail, unsplit reductions only).  Constants fitted to sweeps on one MI355X (mean error 6 %).
 inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks, int split)
 {
     const double per_window = kept * 53.5e-9 * (blocks == 8 ? 2.0 / 1.04 : 1.0);
@@ -55,8 +56,15 @@ inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks,
     const long long full = groups / (256 * slots), rest = groups % (256 * slots);
     const long long busiest = (rest + 255) / 256;
     double t = (double)full * slots * unit;
-    if (busiest > 0)
-        t += full >= 2 ? slots * unit : busiest * unit / (busiest == 1 && full == 0 ? 0.9 : 1.0);
+    if (busiest > 0) {
+        const double spread = busiest * unit / (busiest == 1 ? 0.9 : 1.0);
+        if (full < 2)
+            t += spread;
+        else if (split == 1 && rest <= 128 * slots)
+            t += spread + 6e-6;  // the leftovers get a launch of their own (plan_tail)
+        else
+            t += slots * unit;
+    }
     return t;
 }
 // Wave height (32-row blocks) the matrix-core kernel uses for a shape: the faster one by the model.
@@ -67,16 +75,18 @@ inline int choose_wave_blocks(int M, int N, int nwin, int kept, int split)
     return model_kernel_seconds(M, N, nwin, kept, 8, split) < model_kernel_seconds(M, N, nwin, kept, 4, split) ? 8 : 4;
 }
 
-// Tail split of the tile kernel (split_k == 1): the 256 CUs retire 128 x 128 tiles 1024 at a time
-// (256 x 128 tiles 512 at a time); when the last round is ragged, its `tail` tiles are cut into
-// `slices` pieces along K so that they fill the machine once more, written to scratch and summed
-// by a small second kernel.  slices == 1 means no split.
+// Tail handling of the tile kernel (split_k == 1): the 256 CUs retire 128 x 128 tiles 1024 at a
+// time (256 x 128 tiles 512 at a time); when the last round is ragged, its `tail` tiles get a
+// launch of their own, and with scratch they are also cut into `slices` pieces along K so that they
+// fill the machine once more, written to scratch and summed by a small extra kernel.
 struct TailPlan {
     int blocks;      // 32-row blocks per wave (4 or 8)
     long long head;  // tiles computed whole
     long long tail;  // tiles computed in slices
     int slices;
     size_t ws_bytes; // scratch needed
+    bool separate;   // without scratch: give the tail tiles a launch of their own (they then spread
+                     // one or two per CU instead of landing packed on the CUs that free up last)
 };
 inline TailPlan plan_tail(int M, int N, int nwin, int kept)
 {
@@ -88,26 +98,26 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept)
     t.tail = 0;
     t.slices = 1;
     t.ws_bytes = 0;
+    t.separate = false;
     const long long rest = tiles % slots;
     if (tiles < slots || rest == 0)
         return t;
     // In steady state (two or more full rounds) workgroups finish at staggered times and the
     // dispatcher refills a CU's freed slots together, so the leftover tiles end up packed on few
     // CUs and the last round lasts as long as a full one (measured: 2752 tiles on 512 slots take six
-    // rounds, not 5.4).  Cutting each leftover tile into floor(slots / rest) pieces keeps them in
-    // one round of proportionally shorter pieces.  After a single full round the leftovers spread
-    // over idle CUs by themselves and the second pass costs more than it saves (measured).
-    if (tiles < 2 * slots)
+    // rounds, not 5.4).  A launch of their own spreads them one (or two) per CU.  After a single
+    // full round the leftovers spread over idle CUs by themselves (measured).
+    if (tiles < 2 * slots || rest > slots / 2)
         return t;
-    int slices = (int)(slots / rest);
-    if (slices > 4)
-        slices = 4;  // the scratch grows with the number of pieces
-    while (slices > 1 && nwin / slices < 4)
-        --slices;
-    if (slices < 2)
-        return t;
+    t.separate = true;
     t.head = tiles - rest;
     t.tail = rest;
+    // With scratch, a handful of leftover tiles (at most an eighth of the slots) is also cut into
+    // four pieces along K, so that their launch occupies four times as many CUs for a quarter of
+    // the time.  The pieces pay a second pass: measured +2 % to +5 % up to that size, a loss beyond.
+    if (rest > slots / 8 || nwin / 4 < 4)
+        return t;
+    const int slices = 4;
     t.slices = slices;
     t.ws_bytes = (size_t)rest * slices * (32 * t.blocks) * 128 * sizeof(float);
     return t;

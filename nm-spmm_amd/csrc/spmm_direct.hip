@@ -47,9 +47,9 @@ struct DirectParams {
     int nwin;            // windows in the whole reduction
     int split_k;
     int tiles_m, tiles_n;
-    int head_tiles;      // tiles computed whole; the rest are cut into tail_slices pieces along K
-    int tail_slices;     // 1: no tail split
-    float* tail_ws;      // [tail tile][slice][MS][NS] partial tiles
+    int tile_offset;     // first logical tile of this launch (the tail tiles get a launch of their own)
+    int tail_slices;     // > 1: every workgroup of this launch is one of tail_slices pieces of a tile along K
+    float* tail_ws;      // [tile of this launch][slice][MS][NS] partial tiles
 };
 
 struct float8 { float4 lo, hi; };
@@ -108,19 +108,19 @@ spmm_direct_kernel(const DirectParams p)
     static_assert(WS % CH == 0, "whole chunks");
 
     // ---- tile walk: consecutive ids go to different XCDs, so give each XCD a contiguous run of
-    // logical tiles, walked in bands of GROUP row tiles across all column blocks.  Ids beyond the
-    // head tiles are slices of the tail tiles (a ragged last round cut along K).
-    const bool tail_unit = p.tail_slices > 1 && (int)blockIdx.x >= p.head_tiles;
-    const int unit = (int)blockIdx.x - p.head_tiles;  // slice number among the tail slices
+    // logical tiles, walked in bands of GROUP row tiles across all column blocks.  In a launch of
+    // tail slices, consecutive ids are the pieces of one tile.
+    const bool tail_unit = p.tail_slices > 1;
+    const int unit = blockIdx.x;  // slice number among the slices of this launch
     int logical;
     if (!tail_unit) {
-        const int total = p.tail_slices > 1 ? p.head_tiles : p.tiles_m * p.tiles_n;
+        const int total = gridDim.x;
         const int id = blockIdx.x;
         const int q = total / kXcds, r = total % kXcds;
         const int xcd = id % kXcds, loc = id / kXcds;
-        logical = xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc;
+        logical = p.tile_offset + (xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc);
     } else {
-        logical = p.head_tiles + unit / p.tail_slices;
+        logical = p.tile_offset + unit / p.tail_slices;
     }
     constexpr int GROUP = NMSPMM_GROUP;
     int tile_m, tile_n;
@@ -349,23 +349,32 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     p.split_k = a.split_k;
     p.tiles_m = (a.M + MS - 1) / MS;
     p.tiles_n = a.N / NS;
-    p.head_tiles = p.tiles_m * p.tiles_n;
+    p.tile_offset = 0;
     p.tail_slices = 1;
     p.tail_ws = nullptr;
     // the plan counts 128-column tiles of RM blocks; it applies when that is this tile shape
-    const bool split_tail = plan.slices > 1 && WR == 1 && QS == 4 && RM == plan.blocks;
+    const bool own_tail = plan.separate && WR == 1 && QS == 4 && RM == plan.blocks;
+    const dim3 block(64 * QS * WR);
     dim3 grid(p.tiles_m * p.tiles_n, a.split_k, 1);
-    if (split_tail) {
-        p.head_tiles = (int)plan.head;
-        p.tail_slices = plan.slices;
-        p.tail_ws = a.tail_ws;
-        grid.x = (unsigned)(plan.head + plan.tail * plan.slices);
+    if (!own_tail) {
+        spmm_direct_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, a.stream>>>(p);
+        return hipGetLastError();
     }
-    spmm_direct_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, dim3(64 * QS * WR), 0, a.stream>>>(p);
+    // head tiles, then the leftover tiles in a launch of their own, whole or in slices
+    grid.x = (unsigned)plan.head;
+    spmm_direct_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, a.stream>>>(p);
     hipError_t e = hipGetLastError();
-    if (e == hipSuccess && split_tail) {
+    if (e != hipSuccess)
+        return e;
+    p.tile_offset = (int)plan.head;
+    p.tail_slices = plan.slices;
+    p.tail_ws = plan.slices > 1 ? a.tail_ws : nullptr;
+    grid.x = (unsigned)(plan.tail * plan.slices);
+    spmm_direct_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, a.stream>>>(p);
+    e = hipGetLastError();
+    if (e == hipSuccess && plan.slices > 1) {
         tail_reduce_kernel<MS, NS><<<dim3((unsigned)plan.tail), dim3(256), 0, a.stream>>>(
-            a.tail_ws, a.C, a.M, a.N, p.tiles_m, p.tiles_n, p.head_tiles, plan.slices);
+            a.tail_ws, a.C, a.M, a.N, p.tiles_m, p.tiles_n, (int)plan.head, plan.slices);
         e = hipGetLastError();
     }
     return e;
@@ -384,13 +393,16 @@ static TailPlan tail_plan_for(const SpmmArgs& a, bool have_scratch)
     none.head = none.tail = 0;
     none.slices = 1;
     none.ws_bytes = 0;
+    none.separate = false;
     if (a.split_k != 1 || a.Ns != 128 || NMSPMM_RM_TALL != 8)
         return none;
-    const TailPlan t = plan_tail(a.M, a.N, a.W / a.kept, a.kept);
-    if (t.slices < 2 || t.head + t.tail * t.slices > 0x7fffffffLL)
+    TailPlan t = plan_tail(a.M, a.N, a.W / a.kept, a.kept);
+    if (t.head + t.tail * t.slices > 0x7fffffffLL)
         return none;
-    if (have_scratch && (a.tail_ws == nullptr || a.tail_ws_bytes < t.ws_bytes))
-        return none;
+    if (have_scratch && t.slices > 1 && (a.tail_ws == nullptr || a.tail_ws_bytes < t.ws_bytes)) {
+        t.slices = 1;  // no scratch: the tail can still have a launch of its own
+        t.ws_bytes = 0;
+    }
     return t;
 }
 

@@ -200,7 +200,7 @@ def test_auto_entry_point_chooses_the_split_itself(oracle, M, N, K, n, m, sparsi
     check(oracle, d, C.cpu().numpy())
 
 
-@pytest.mark.parametrize("M,N,K,n,m", [(4096, 8448, 512, 2, 8), (8192, 4224, 1024, 2, 4), (4096, 8448, 512, 1, 8)])
+@pytest.mark.parametrize("M,N,K,n,m", [(8192, 4224, 1024, 2, 4), (4096, 8448, 1024, 1, 8), (8192, 4224, 2048, 2, 8)])
 def test_ragged_last_round_is_split_along_k_through_scratch(oracle, M, N, K, n, m):
     """More tiles than the GPU holds at once and a ragged last round: with scratch the tiles of that
     round are cut along K and summed by a second kernel; the result matches the checker either way."""
@@ -225,6 +225,31 @@ def test_ragged_last_round_is_split_along_k_through_scratch(oracle, M, N, K, n, 
                                rows=(r0, r1)).reshape(M, N)[r0:r1]
         for C in outs[:2]:
             assert scaled_max_error(C[r0:r1].cpu().numpy(), want) <= REL_TOL
+
+
+@pytest.mark.parametrize("M,N,K,n,m", [(4096, 8448, 256, 2, 4), (8192, 4224, 512, 1, 8)])
+def test_leftover_tiles_in_a_launch_of_their_own(oracle, M, N, K, n, m):
+    """Two full rounds of tiles and a few leftovers, too few windows to cut them: the leftovers run
+    as a second launch of the same kernel; every tile must still be computed exactly once."""
+    d = datagen.init_data(M, N, K, n, m, seed=M + K)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    assert nmspmm.tail_workspace_bytes(M, N, d["W"], kept) == 0
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), None if cinfo is None else dev(cinfo), C, M, N, K, d["W"], window,
+                kept, 32, 128, 1, None)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == "mfma" and bool(torch.isfinite(C).all())
+    # column sums of C against column sums computed from the operands in fp64: touches every tile
+    dense = torch.zeros((K, N), dtype=torch.float64, device="cuda")
+    rows = (torch.arange(d["W"], device="cuda") // n * m)[:, None] + dev(d["DT"]).long()
+    dense[rows.repeat_interleave(32, dim=1), torch.arange(N, device="cuda")[None, :].expand(d["W"], -1)] = dev(d["BT"]).double()
+    want = dev(d["A_km"]).double().sum(dim=1) @ dense
+    got = C.double().sum(dim=0)
+    assert float(((got - want).abs() / want.abs().clamp_min(want.pow(2).mean().sqrt())).max()) <= REL_TOL
+    for (r0, r1) in ((0, 16), (M - 16, M)):
+        ref = oracle.gemm_cpu(d["A_km"].reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), M, N, d["W"],
+                              rows=(r0, r1)).reshape(M, N)[r0:r1]
+        assert scaled_max_error(C[r0:r1].cpu().numpy(), ref) <= REL_TOL
 
 
 def test_llm_layer_shape_2of8(oracle):
