@@ -56,7 +56,9 @@ struct float8 { float4 lo, hi; };
 template <int RM> struct AFrag;
 template <> struct AFrag<8> { typedef float8 type; };
 template <> struct AFrag<4> { typedef float4 type; };
+template <> struct AFrag<2> { typedef float2 type; };
 
+__device__ inline float frag_get(const float2& v, int i) { return i == 0 ? v.x : v.y; }
 __device__ inline float frag_get(const float4& v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
 __device__ inline float frag_get(const float8& v, int i) { return i < 4 ? frag_get(v.lo, i) : frag_get(v.hi, i - 4); }
 
@@ -70,6 +72,11 @@ __device__ inline float4 buffer_load_f4(__amdgpu_buffer_rsrc_t r, uint32_t byte_
 {
     auto v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
     return *reinterpret_cast<float4*>(&v);
+}
+__device__ inline float2 buffer_load_f2(__amdgpu_buffer_rsrc_t r, uint32_t byte_off)
+{
+    auto v = __builtin_amdgcn_raw_buffer_load_b64(r, byte_off, 0, 0);
+    return *reinterpret_cast<float2*>(&v);
 }
 __device__ inline float buffer_load_f1(__amdgpu_buffer_rsrc_t r, uint32_t byte_off, uint32_t s_off)
 {
@@ -88,6 +95,7 @@ __device__ inline float buffer_load_f1(__amdgpu_buffer_rsrc_t r, uint32_t byte_o
 #define NMSPMM_RM_TALL 8
 #endif
 
+
 // KS: dense rows per window, WS: kept rows per window, QS: column vectors per preprocessed column
 // block (Ns = 32*QS), WR: waves along M, RM: 32-row blocks per wave (4 or 8), HIGH:
 // high-sparsity layout (D holds ranks into the window's column_info list).
@@ -95,7 +103,8 @@ template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
 __global__ void __launch_bounds__(64 * QS * WR, RM == 8 ? 2 : NMSPMM_OCC)
 spmm_direct_kernel(const DirectParams p)
 {
-    static_assert(RM == 4 || RM == 8, "128- or 256-row waves");
+    static_assert(RM == 2 || RM == 4 || RM == 8, "64-, 128- or 256-row waves");
+    constexpr int IL = RM < 4 ? RM : 4;  // rows interleaved per lane: block b holds rows IL*r + b%IL (+128 for b >= 4)
     static_assert(WS % 2 == 0, "two kept rows per MFMA");
     typedef typename AFrag<RM>::type afrag_t;
     constexpr int MW = RM * 32;               // rows per wave
@@ -159,7 +168,7 @@ spmm_direct_kernel(const DirectParams p)
     const uint32_t a_bytes = bi < M ? (uint32_t)(((size_t)(KS - 1) * lda + (size_t)(lda - bi)) * sizeof(float)) : 0u;
     const uint32_t b_bytes = (uint32_t)(((size_t)(WS - 1) * N + 32) * sizeof(float));
     const uint32_t row_bytes = (uint32_t)((size_t)lda * sizeof(float));
-    const uint32_t a_vlane = (uint32_t)(j * 16);  // this lane's run of four rows inside the wave's rows
+    const uint32_t a_vlane = (uint32_t)(j * IL * sizeof(float));  // this lane's run of IL rows inside the wave's rows
     const uint32_t b_chunk = (uint32_t)((size_t)CH * N * sizeof(float));
     uint32_t b_off[CS];
 #pragma unroll
@@ -216,8 +225,10 @@ spmm_direct_kernel(const DirectParams p)
         if constexpr (RM == 8) {
             a_op[s].lo = buffer_load_f4(ra, off);
             a_op[s].hi = buffer_load_f4(ra, off + 512);
-        } else {
+        } else if constexpr (RM == 4) {
             a_op[s] = buffer_load_f4(ra, off);
+        } else {
+            a_op[s] = buffer_load_f2(ra, off);
         }
         b_op[s] = buffer_load_f1(rb, b_off[s], c * b_chunk);
     };
@@ -272,7 +283,7 @@ spmm_direct_kernel(const DirectParams p)
     }
 
     // ---- epilogue: MFMA result register v of lane (h, j) is row 8*(v/4) + 4*h + v%4 of the block,
-    // column j; block b of the wave holds rows (b/4)*128 + 4*r + b%4.  Stores go through a
+    // column j; block b of the wave holds rows (b/4)*128 + IL*r + b%IL.  Stores go through a
     // descriptor that ends with the last live row of this wave, so rows beyond M are dropped
     // without a branch; the per-register part of the offset is a scalar.
     // A slice of a tail tile goes to its own MS x NS block of the scratch instead, all rows.
@@ -283,13 +294,14 @@ spmm_direct_kernel(const DirectParams p)
                                     : out + (size_t)min(bi, M) * N + bj;
     const uint32_t c_bytes = rows_here > 0 ? (uint32_t)(((size_t)(rows_here - 1) * pitch + 32) * sizeof(float)) : 0u;
     const __amdgpu_buffer_rsrc_t rc = make_rsrc(c_base, c_bytes);
-    const uint32_t c_lane = (uint32_t)(((size_t)16 * h * pitch + j) * sizeof(float));
+    const uint32_t c_lane = (uint32_t)(((size_t)4 * IL * h * pitch + j) * sizeof(float));
     const uint32_t n_bytes = (uint32_t)((size_t)pitch * sizeof(float));
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
 #pragma unroll
         for (int b = 0; b < RM; ++b) {
-            const uint32_t row = (b / 4) * 128 + 32 * (v / 4) + 4 * (v % 4) + (b % 4);  // without the lane's 16*h
+            // row inside the wave, without the lane's 4*IL*h: IL * (8*(v/4) + v%4) + b%IL, second group + 128
+            const uint32_t row = (b / 4) * 128 + IL * (8 * (v / 4) + (v % 4)) + (b % IL);
             __builtin_amdgcn_raw_buffer_store_b32(__float_as_int(acc[b][v]), rc, c_lane + row * n_bytes, 0, 0);
         }
     }
@@ -411,6 +423,11 @@ static hipError_t launch_ns(const SpmmArgs& a)
 {
     const TailPlan plan = tail_plan_for(a, true);
     const bool tall = NMSPMM_RM_TALL == 8 && plan.blocks == 8;
+    // 64-row waves cost more loads per MFMA; they pay only where 128-row waves would multiply
+    // mostly padding (192 rows: three 64-row waves instead of two 128-row ones, +24 % measured)
+    const int rows64 = (a.M + 63) / 64 * 64, rows128 = (a.M + 127) / 128 * 128;
+    if (!tall && a.Ns == 128 && rows64 * 8 <= rows128 * 7)
+        return launch_cfg<KS, WS, 4, 1, 2, HIGH>(a, plan);
     switch (a.Ns) {
     case 128:
         return tall ? launch_cfg<KS, WS, 4, 1, NMSPMM_RM_TALL, HIGH>(a, plan) : launch_cfg<KS, WS, 4, 1, 4, HIGH>(a, plan);

@@ -62,7 +62,7 @@ def test_config1_512_cubed_2of4(oracle):
     assert scaled_max_error(got, want) <= REL_TOL
 
 
-@pytest.mark.parametrize("M", [36, 64, 100, 192, 328])
+@pytest.mark.parametrize("M", [36, 64, 100, 132, 192, 328, 448])
 @pytest.mark.parametrize("n,m,Ns", [(2, 4, 128), (1, 8, 128), (2, 8, 64), (3, 8, 32)])
 def test_ragged_row_counts(oracle, M, n, m, Ns):
     d = datagen.init_data(M, 256, 256, n, m, seed=M + n)
