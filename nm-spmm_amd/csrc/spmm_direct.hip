@@ -95,9 +95,8 @@ __device__ inline float buffer_load_f1(__amdgpu_buffer_rsrc_t r, uint32_t byte_o
 #define NMSPMM_RM_TALL 8
 #endif
 
-
 // KS: dense rows per window, WS: kept rows per window, QS: column vectors per preprocessed column
-// block (Ns = 32*QS), WR: waves along M, RM: 32-row blocks per wave (4 or 8), HIGH:
+// block (Ns = 32*QS), WR: waves along M, RM: 32-row blocks per wave (2, 4 or 8), HIGH:
 // high-sparsity layout (D holds ranks into the window's column_info list).
 template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
 __global__ void __launch_bounds__(64 * QS * WR, RM == 8 ? 2 : NMSPMM_OCC)
