@@ -89,6 +89,17 @@ int nmspmm_preprocess_high_device(int32_t* d_column_info, int pruning_M, int pru
                                   const int32_t* dDT_in, int32_t* dDT_out, int W, int Q, int N,
                                   int Ns, int vec_len, void* stream);
 
+/* The whole preprocessing of a 32-column-vector pattern in one kernel: dDT_in holds the indices as
+ * generated (n kept rows in every window of m, row-major int32[W][Q]); the transIndex doublings
+ * that take the pattern to the kernels' window (reference tests/test_nmspmm.cu:72-79 calls them one
+ * after the other) are folded into the re-blocking / ranking pass.  dD_out and, for the
+ * high-sparsity geometries, d_column_info receive exactly what the separate calls produce;
+ * *window and *kept are what nmspmm_spmm then takes.  dDT_in is not modified.  n/m must reduce to
+ * 1/1, 1/2, 3/8, 1/4 or 1/8 with m a power-of-two fraction of the kernel window. */
+int nmspmm_preprocess_device(const int32_t* dDT_in, int n, int m, int W, int Q, int N, int Ns,
+                             int32_t* dD_out, int32_t* d_column_info, int* window, int* kept,
+                             void* stream);
+
 /* Number of int32 the high-sparsity preprocessing writes: (N/Ns) * (W/pruning_N) * pruning_M.
  * (The reference driver allocates one extra window of slack, tests/test_nmspmm.cu:23; this
  * library neither needs nor touches it.)  Returns 0 for invalid arguments. */

@@ -52,6 +52,7 @@ def lib():
         L.nmspmm_preprocess_high_device.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p] + [c_int] * 5 + [c_void_p]
         L.nmspmm_compress_device.argtypes = [c_void_p] + [c_int] * 5 + [c_void_p, c_void_p, c_void_p]
         L.nmspmm_decompress_device.argtypes = [c_void_p, c_void_p] + [c_int] * 5 + [c_void_p, c_void_p]
+        L.nmspmm_preprocess_device.argtypes = [c_void_p] + [c_int] * 6 + [c_void_p, c_void_p, ip, ip, c_void_p]
         L.nmspmm_column_info_ints.restype = c_size_t
         L.nmspmm_column_info_ints.argtypes = [c_int] * 5
         L.nmspmm_tail_workspace_bytes.restype = c_size_t
@@ -126,6 +127,15 @@ def compress_device(dB, K, N, n, m, dBT, dDT, vec_len=32):
 def decompress_device(dBT, dDT, K, N, n, m, dB, vec_len=32):
     _check("nmspmm_decompress_device",
            lib().nmspmm_decompress_device(_ptr(dBT), _ptr(dDT), K, N, n, m, vec_len, _ptr(dB), _stream()))
+
+
+def preprocess_device(dDT_in, n, m, W, Q, N, Ns, dD_out, d_cinfo):
+    """Widening + re-blocking (+ ranking) in one kernel; returns (window, kept)."""
+    window, kept = ctypes.c_int(0), ctypes.c_int(0)
+    _check("nmspmm_preprocess_device",
+           lib().nmspmm_preprocess_device(_ptr(dDT_in), n, m, W, Q, N, Ns, _ptr(dD_out), _ptr(d_cinfo),
+                                          ctypes.byref(window), ctypes.byref(kept), _stream()))
+    return window.value, kept.value
 
 
 def column_info_ints(W, pN, pM, N, Ns):

@@ -176,7 +176,7 @@ int nmspmm_preprocess_low_device(const int32_t* dDT_in, int32_t* dDT_out, int W,
         return st;
     if (dDT_in == dDT_out)
         return NMSPMM_ERR_BAD_SHAPE;
-    if (launch_reblock(dDT_in, dDT_out, W, Q, Ns / vec_len, (hipStream_t)stream) != hipSuccess)
+    if (launch_reblock(dDT_in, dDT_out, W, Q, Ns / vec_len, 1, 0, 0, (hipStream_t)stream) != hipSuccess)
         return NMSPMM_ERR_HIP;
     return NMSPMM_OK;
 }
@@ -230,7 +230,7 @@ int nmspmm_preprocess_high_device(int32_t* d_column_info, int pruning_M, int pru
         return st;
     if (dDT_in == dDT_out)
         return NMSPMM_ERR_BAD_SHAPE;
-    if (launch_preprocess_high(d_column_info, pruning_M, pruning_N, dDT_in, dDT_out, W, Q, Ns / vec_len,
+    if (launch_preprocess_high(d_column_info, pruning_M, pruning_N, dDT_in, dDT_out, W, Q, Ns / vec_len, 1, 0, 0,
                                (hipStream_t)stream) != hipSuccess)
         return NMSPMM_ERR_HIP;
     return NMSPMM_OK;
@@ -256,6 +256,40 @@ int nmspmm_preprocess_high_host(int32_t* column_info, int pruning_M, int pruning
     if (hipMemcpy(DT, out.p, bytes, hipMemcpyDeviceToHost) != hipSuccess ||
         hipMemcpy(column_info, ci.p, ci_bytes, hipMemcpyDeviceToHost) != hipSuccess)
         return NMSPMM_ERR_HIP;
+    return NMSPMM_OK;
+}
+
+int nmspmm_preprocess_device(const int32_t* dDT_in, int n, int m, int W, int Q, int N, int Ns, int32_t* dD_out,
+                             int32_t* d_column_info, int* window, int* kept, void* stream)
+{
+    if (!dDT_in || !dD_out || !window || !kept)
+        return NMSPMM_ERR_NULL_POINTER;
+    if (n <= 0 || m <= 0 || n > m)
+        return NMSPMM_ERR_BAD_PATTERN;
+    // the kernel geometry of the pattern's sparsity, reached by doubling the generated window
+    int win = 0, kp = 0, high = 0;
+    const int st0 = nmspmm_pattern_from_sparsity(1.0f - (float)n / (float)m, &win, &kp, &high);
+    if (st0 != NMSPMM_OK)
+        return st0;
+    int times = 0;
+    while ((m << times) < win)
+        ++times;
+    if ((m << times) != win || (n << times) != kp)
+        return NMSPMM_ERR_BAD_PATTERN;
+    const int st = check_reblock(dDT_in, dD_out, W, Q, Ns, 32);
+    if (st != NMSPMM_OK)
+        return st;
+    if (dDT_in == dD_out || N != Q * 32 || W % kp != 0)
+        return NMSPMM_ERR_BAD_SHAPE;
+    if (high && !d_column_info)
+        return NMSPMM_ERR_NULL_POINTER;
+    const hipError_t e = high ? launch_preprocess_high(d_column_info, win, kp, dDT_in, dD_out, W, Q, Ns / 32, n, m,
+                                                       times, (hipStream_t)stream)
+                              : launch_reblock(dDT_in, dD_out, W, Q, Ns / 32, n, m, times, (hipStream_t)stream);
+    if (e != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    *window = win;
+    *kept = kp;
     return NMSPMM_OK;
 }
 

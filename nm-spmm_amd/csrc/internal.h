@@ -170,9 +170,12 @@ hipError_t launch_splitk_reduce(const float* partial, float* C, size_t elems, si
 
 // Index preprocessing kernels (preprocess.hip).
 hipError_t launch_trans_index(int32_t* dDT, int W, int Q, int pN, int pM, hipStream_t stream);
-hipError_t launch_reblock(const int32_t* in, int32_t* out, int W, int Q, int Qs, hipStream_t stream);
+// n0, m0, times: the pattern the indices were generated with and the transIndex doublings to fold
+// into the read (times == 0: none).
+hipError_t launch_reblock(const int32_t* in, int32_t* out, int W, int Q, int Qs, int n0, int m0, int times,
+                          hipStream_t stream);
 hipError_t launch_preprocess_high(int32_t* cinfo, int pM, int pN, const int32_t* in, int32_t* out,
-                                  int W, int Q, int Qs, hipStream_t stream);
+                                  int W, int Q, int Qs, int n0, int m0, int times, hipStream_t stream);
 
 // Dense <-> N:M vector-sparse conversion (compress.hip): m in {4, 8, 16, 32}, vec_len in {4, 8, 16, 32}.
 bool compress_supported(int m, int vec_len);

@@ -17,10 +17,20 @@ trans_index_kernel(int32_t* __restrict__ DT, size_t total, int Q, int pN, int pM
     }
 }
 
+// The indices may still be the narrow n0:m0 windows they were generated with: `times` doublings of
+// transIndex (reference src/preprocessing.cu:3-15) add m0 * ((r / n0) mod 2^times) to the index in
+// compressed row r, which these kernels fold into their read instead of a pass of its own
+// (times == 0: the indices are used as they are).
+__device__ inline int widened(int v, size_t r, int n0, int m0, int times)
+{
+    return v + m0 * (int)((r / n0) & ((1u << times) - 1u));
+}
+
 // [W][Q] -> [Q/Qs][W][Qs] (reference src/preprocessing.cu:61-77,80-100).  Threads run along the
 // output, which is written fully coalesced; reads come in runs of Qs int32.
 __global__ void __launch_bounds__(256)
-reblock_kernel(const int32_t* __restrict__ in, int32_t* __restrict__ out, int W, int Q, int Qs)
+reblock_kernel(const int32_t* __restrict__ in, int32_t* __restrict__ out, int W, int Q, int Qs, int n0, int m0,
+               int times)
 {
     const size_t total = (size_t)W * Q;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -30,7 +40,7 @@ reblock_kernel(const int32_t* __restrict__ in, int32_t* __restrict__ out, int W,
         const size_t rem = o - jb * per_block;
         const size_t r = rem / Qs;
         const size_t c = rem - r * Qs;
-        out[o] = in[r * Q + jb * Qs + c];
+        out[o] = widened(in[r * Q + jb * Qs + c], r, n0, m0, times);
     }
 }
 
@@ -43,7 +53,8 @@ constexpr int kMaxWindow = 1024;
 
 __global__ void __launch_bounds__(64)
 preprocess_high_kernel(int32_t* __restrict__ cinfo, const int32_t* __restrict__ in,
-                       int32_t* __restrict__ out, int W, int Q, int Qs, int pN, int pM, int nwin)
+                       int32_t* __restrict__ out, int W, int Q, int Qs, int pN, int pM, int nwin, int n0, int m0,
+                       int times)
 {
     __shared__ int present[kMaxWindow];
     __shared__ int rank[kMaxWindow];
@@ -57,7 +68,8 @@ preprocess_high_kernel(int32_t* __restrict__ cinfo, const int32_t* __restrict__ 
     __syncthreads();
     for (int e = lane; e < cells; e += 64) {
         const int p = e / Qs, c = e - p * Qs;
-        const int v = in[((size_t)w * pN + p) * Q + (size_t)jb * Qs + c];
+        const size_t r = (size_t)w * pN + p;
+        const int v = widened(in[r * Q + (size_t)jb * Qs + c], r, n0, m0, times);
         if ((unsigned)v < (unsigned)pM)  // malformed indices must not leave the table
             present[v] = 1;
     }
@@ -82,8 +94,9 @@ preprocess_high_kernel(int32_t* __restrict__ cinfo, const int32_t* __restrict__ 
 
     for (int e = lane; e < cells; e += 64) {
         const int p = e / Qs, c = e - p * Qs;
-        const int v = in[((size_t)w * pN + p) * Q + (size_t)jb * Qs + c];
-        out[((size_t)jb * W + (size_t)w * pN + p) * Qs + c] = (unsigned)v < (unsigned)pM ? rank[v] : -1;
+        const size_t r = (size_t)w * pN + p;
+        const int v = widened(in[r * Q + (size_t)jb * Qs + c], r, n0, m0, times);
+        out[((size_t)jb * W + r) * Qs + c] = (unsigned)v < (unsigned)pM ? rank[v] : -1;
     }
 }
 
@@ -104,18 +117,20 @@ hipError_t launch_trans_index(int32_t* dDT, int W, int Q, int pN, int pM, hipStr
     return hipGetLastError();
 }
 
-hipError_t launch_reblock(const int32_t* in, int32_t* out, int W, int Q, int Qs, hipStream_t stream)
+hipError_t launch_reblock(const int32_t* in, int32_t* out, int W, int Q, int Qs, int n0, int m0, int times,
+                          hipStream_t stream)
 {
-    hipLaunchKernelGGL(reblock_kernel, dim3(grid_for((size_t)W * Q)), dim3(256), 0, stream, in, out, W, Q, Qs);
+    hipLaunchKernelGGL(reblock_kernel, dim3(grid_for((size_t)W * Q)), dim3(256), 0, stream, in, out, W, Q, Qs, n0,
+                       m0, times);
     return hipGetLastError();
 }
 
 hipError_t launch_preprocess_high(int32_t* cinfo, int pM, int pN, const int32_t* in, int32_t* out,
-                                  int W, int Q, int Qs, hipStream_t stream)
+                                  int W, int Q, int Qs, int n0, int m0, int times, hipStream_t stream)
 {
     const int nwin = W / pN;
     hipLaunchKernelGGL(preprocess_high_kernel, dim3(nwin, Q / Qs), dim3(64), 0, stream, cinfo, in, out, W, Q,
-                       Qs, pN, pM, nwin);
+                       Qs, pN, pM, nwin, n0, m0, times);
     return hipGetLastError();
 }
 

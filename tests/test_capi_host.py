@@ -126,6 +126,20 @@ def test_preprocess_rejects_bad_arguments_without_a_gpu():
     assert L.nmspmm_status_string(4).decode().startswith("sparsity belongs")
 
 
+def test_one_kernel_preprocessing_rejects_bad_arguments_without_a_gpu():
+    L = nmspmm.lib()
+    w, k = ctypes.c_int(0), ctypes.c_int(0)
+    args = lambda **kw: [kw.get("src", FAKE), kw.get("n", 2), kw.get("m", 8), kw.get("W", 64), 4, 128, kw.get("Ns", 128),
+                         kw.get("dst", FAKE + 4096), kw.get("ci", FAKE + 8192), ctypes.byref(w), ctypes.byref(k), None]
+    assert L.nmspmm_preprocess_device(*args(src=None)) == 1
+    assert L.nmspmm_preprocess_device(*args(ci=None)) == 1          # 2:8 needs column_info
+    assert L.nmspmm_preprocess_device(*args(n=3, m=4)) == 3         # 3:4 is not a kernel sparsity
+    assert L.nmspmm_preprocess_device(*args(n=3, m=24)) == 3        # 1:8, but 24 does not double to 64
+    assert L.nmspmm_preprocess_device(*args(W=72)) == 2             # not whole 16-row windows
+    assert L.nmspmm_preprocess_device(*args(dst=FAKE)) == 2         # in place
+    assert L.nmspmm_preprocess_device(*args(Ns=96)) == 2
+
+
 def test_compress_rejects_bad_arguments_without_a_gpu():
     L = nmspmm.lib()
     assert L.nmspmm_compress_device(None, 64, 64, 2, 4, 32, FAKE, FAKE, None) == 1

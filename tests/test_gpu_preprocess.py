@@ -6,7 +6,7 @@ import os
 import numpy as np
 import pytest
 
-from conftest import GOLDEN_DIR, datagen, nmspmm
+from conftest import GOLDEN_DIR, datagen, kernel_geometry, nmspmm
 
 pytestmark = pytest.mark.gpu
 torch = pytest.importorskip("torch")
@@ -73,6 +73,36 @@ def test_full_size_index_buffers_bit_exact_vs_checker(oracle, N, K, n, m, vl, ti
         nmspmm.preprocess_high_device(ci, pm, pn, x, dst, W, Q, N, Ns, vl)
         assert np.array_equal(dst.cpu().numpy(), want)
         assert np.array_equal(ci.cpu().numpy(), want_ci)
+
+
+@pytest.mark.parametrize("n,m", [(2, 4), (3, 8), (2, 8), (1, 8), (16, 32), (12, 32), (8, 32), (4, 32), (32, 32), (1, 2), (4, 16)])
+@pytest.mark.parametrize("Ns", [128, 64, 32])
+def test_one_kernel_preprocessing_equals_the_separate_calls(oracle, n, m, Ns):
+    """nmspmm_preprocess_device folds the transIndex doublings into the re-blocking / ranking pass:
+    bit-exact against the checker's sequence and it leaves its input alone."""
+    N, K = 1024, 1024 if m != 8 or n != 3 else 1536
+    d = datagen.init_data(4, N, K, n, m, seed=10 * n + m + Ns)
+    W, Q = d["W"], d["Q"]
+    host = d["DT"].reshape(-1).copy()
+    src = dev(host)
+    window, kept, times = kernel_geometry(n, m)
+    want = host.copy()
+    pn, pm = n, m
+    for _ in range(times):
+        pn, pm = oracle.trans_index(want, W, Q, pn, pm)
+    out = torch.full((W * Q,), -9, dtype=torch.int32, device="cuda")
+    if window == 64:
+        want_ci = oracle.preprocess_high(pm, pn, want, W, Q, Ns)
+        ci = torch.full((want_ci.size,), -9, dtype=torch.int32, device="cuda")
+    else:
+        oracle.preprocess_low(want, W, Q, Ns)
+        want_ci, ci = None, None
+    got = nmspmm.preprocess_device(src, n, m, W, Q, N, Ns, out, ci)
+    assert got == (window, kept)
+    assert np.array_equal(out.cpu().numpy(), want)
+    if want_ci is not None:
+        assert np.array_equal(ci.cpu().numpy(), want_ci)
+    assert np.array_equal(src.cpu().numpy(), host)
 
 
 def test_host_pointer_forms_work_in_place(oracle):
