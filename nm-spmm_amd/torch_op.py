@@ -52,16 +52,13 @@ class NMSparseLinear(torch.nn.Module):
         BT = torch.empty((self.W, N), dtype=torch.float32, device=weight.device)
         DT = torch.empty((self.W, self.Q), dtype=torch.int32, device=weight.device)
         _nm.compress_device(dense, K, N, n, m, BT, DT)
-        pn, pm = n, m
-        while pm < self.window:
-            pn, pm = _nm.trans_index_device(DT, self.W, N, self.Q, pn, pm)
         D = torch.empty_like(DT)
         cinfo = None
         if self.window == 64:
-            cinfo = torch.empty(_nm.column_info_ints(self.W, pn, pm, N, self.Ns), dtype=torch.int32, device=weight.device)
-            _nm.preprocess_high_device(cinfo, pm, pn, DT, D, self.W, self.Q, N, self.Ns)
-        else:
-            _nm.preprocess_low_device(DT, D, self.W, self.Q, self.Ns)
+            cinfo = torch.empty(_nm.column_info_ints(self.W, self.kept, self.window, N, self.Ns), dtype=torch.int32,
+                                device=weight.device)
+        got = _nm.preprocess_device(DT, n, m, self.W, self.Q, N, self.Ns, D, cinfo)
+        assert got == (self.window, self.kept)
         self.register_buffer("values", BT)
         self.register_buffer("indices", D.reshape(-1))
         self.register_buffer("column_info", cinfo)
