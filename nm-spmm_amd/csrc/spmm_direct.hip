@@ -89,7 +89,7 @@ __device__ inline float buffer_load_f1(__amdgpu_buffer_rsrc_t r, uint32_t byte_o
 #define NMSPMM_OCC 3
 #endif
 #ifndef NMSPMM_GROUP
-#define NMSPMM_GROUP 8
+#define NMSPMM_GROUP 2
 #endif
 #ifndef NMSPMM_RM_TALL
 #define NMSPMM_RM_TALL 8
