@@ -238,7 +238,7 @@ def main():
                      # bytes behind L2 per launch: rocprofv3 FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the
                      # factors coming from a plain 256 MiB copy in the same runs
                      # (profiles/spmm_direct_kernel_4096cubed_2of4.md)
-                     "traffic": 404.9e6, "traffic_unit": "bytes per launch", "algorithmic_bytes": 168.8e6,
+                     "traffic": 411.2e6, "traffic_unit": "bytes per launch", "algorithmic_bytes": 168.8e6,
                      "kernel": "spmm_direct_kernel<32,16,4,1,8,false>", "flops_per_launch": case.useful_flops(),
                      "launch_ms_events": round(ms, 5), "launch_ms_wall": round(wall_ms, 5)},
         "cpu_baseline": cpu,
