@@ -172,7 +172,9 @@ def main():
     import torch
     pkg = importlib.import_module("nm-spmm_amd")
     datagen = importlib.import_module("nm-spmm_amd.datagen")
-    pkg.lib()  # fails loudly if the HIP library has not been built
+    if not os.path.exists(pkg.LIB_PATH):  # load what is built; build only when nothing is
+        importlib.import_module("__graft_entry__").build()
+    pkg.lib()  # fails loudly if the HIP library is still missing: there is no fallback
     torch.cuda.set_device(0)
     torch.backends.cuda.matmul.allow_tf32 = False
 
