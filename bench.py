@@ -159,7 +159,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the CPU baseline sample (0 = skip)")
     ap.add_argument("--headline-only", action="store_true", help="time only the 2:4 kernel (for profiling runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy 5 times (known traffic, to scale rocprofv3's "
