@@ -1,0 +1,41 @@
+"""The benchmark's command-line contract: more than one GPU is refused with a message (the library
+is a single-GPU kernel library), and on a GPU the default run prints one JSON line with the agreed
+fields."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+from conftest import ROOT
+
+BENCH = os.path.join(ROOT, "bench.py")
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    out = subprocess.run([sys.executable, BENCH, "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert out.returncode != 0
+    assert "single-GPU" in out.stderr and out.stdout.strip() == ""
+
+
+@pytest.mark.gpu
+def test_one_json_line_with_roofline_and_cpu_baseline():
+    out = subprocess.run([sys.executable, BENCH, "--steps", "10", "--warmup", "2", "--cpu-rows", "256"],
+                         capture_output=True, text=True, timeout=600)
+    assert out.returncode == 0, out.stderr
+    lines = [l for l in out.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in d, key
+    assert d["n_gpus"] == 1 and d["steps"] == 10 and d["warmup"] == 2 and d["vs_baseline"] is None
+    assert d["dtype"] == "f32" and "workload" in d["config"]
+    r = d["roofline"]
+    assert r["bound"] == "mfma" and r["peak"] == 157.3 and abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-3
+    assert abs(d["value"] - 2.0 * 4096 ** 2 * 2048 / (d["ms_per_step"] * 1e-3) / 1e12) < 0.01 * d["value"]
+    c = d["cpu_baseline"]
+    assert c["kind"] in ("reference", "port") and c["cores"] >= 1 and c["value"] > 0
+    assert c["gpu_vs_cpu_scaled_max_error"] <= 1e-4
+    assert set(d["sweep"]) == {"2:4", "3:8", "2:8", "1:8"}
