@@ -235,6 +235,150 @@ spmm_skinny_kernel(const SkinnyParams p)
     }
 }
 
+// Up to 16 rows: the same design on v_mfma_f32_16x16x4_f32.  A k-step is four kept rows, so the
+// streaming loop issues half as many loads and spends half as many matrix-pipe cycles per kept
+// row as the 32-row form.  Lane l = (kq, jl) = (l / 16, l % 16) supplies A[jl][row of kept row
+// 4s + kq] and, with one 64-bit load, B[4s + kq][2 jl] and B[4s + kq][2 jl + 1] (four 128-byte row
+// segments per wave and instruction): the even columns of the vector accumulate in one MFMA
+// tile, the odd ones in a second.  Result register v of lane (kq, jl) is row 4 kq + v.
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+template <int KS, int WS, int QS, bool HIGH, int U>
+__global__ void __launch_bounds__(64 * kSkinnyWaves)
+spmm_skinny16_kernel(const SkinnyParams p)
+{
+    constexpr int KSTEPS = WS / 4;
+    constexpr int STEPS = U * KSTEPS;
+    constexpr int ND = (WS * QS + 63) / 64;
+    static_assert(WS % 4 == 0, "k-steps of four kept rows");
+    __shared__ float red[kSkinnyWaves][8][64];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kq = lane >> 4;
+    const int jl = lane & 15;
+    const int vec_g = blockIdx.x;
+    const int jb = vec_g / QS;
+    const int vec = vec_g % QS;
+    const int M = p.M, N = p.N, lda = p.lda;
+
+    int w_begin, w_count;
+    split_windows(p.nwin, kSkinnyWaves, wave, &w_begin, &w_count);
+    const int w_end = w_begin + w_count;
+
+    const float* const Bvec = p.B + (size_t)vec_g * 32;
+    const int32_t* const Dblk = p.D + (size_t)jb * p.W * QS;
+    const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)jb * p.nwin * KS : nullptr;
+    const uint32_t a_bytes = (uint32_t)((size_t)p.K * lda * sizeof(float));
+    const uint32_t a_lane = jl < M ? (uint32_t)(jl * sizeof(float)) : kSkNoLoad;
+    const uint32_t row_bytes = (uint32_t)((size_t)lda * sizeof(float));
+    const uint32_t b_lane = (uint32_t)(((size_t)kq * N + 2 * jl) * sizeof(float));
+    const uint32_t b_step = (uint32_t)(4 * (size_t)N * sizeof(float));
+    const uint32_t b_bytes = (uint32_t)(((size_t)(WS - 1) * N + 32) * sizeof(float));
+    const int perm_addr = (kq * QS + vec) * (int)sizeof(int32_t);
+
+    floatx4 acc_even = {0.0f, 0.0f, 0.0f, 0.0f}, acc_odd = {0.0f, 0.0f, 0.0f, 0.0f};
+
+    int dvec[U][ND];
+    int civec[U];
+    // two operand sets: one is multiplied while the other is in flight
+    float a0[STEPS], a1[STEPS];
+    float2 b0[STEPS], b1[STEPS];
+
+    auto load_meta = [&](int w) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int wu = min(w + u, p.nwin - 1);
+            const __amdgpu_buffer_rsrc_t rd = sk_rsrc(Dblk + (size_t)wu * WS * QS, WS * QS * sizeof(int32_t));
+#pragma unroll
+            for (int q = 0; q < ND; ++q)
+                dvec[u][q] = __builtin_amdgcn_raw_buffer_load_b32(rd, (lane + 64 * q) * (int)sizeof(int32_t), 0, 0);
+            if (HIGH) {
+                const __amdgpu_buffer_rsrc_t rc = sk_rsrc(Cinfo + (size_t)wu * KS, KS * sizeof(int32_t));
+                civec[u] = __builtin_amdgcn_raw_buffer_load_b32(rc, lane * (int)sizeof(int32_t), 0, 0);
+            }
+        }
+    };
+    auto load_b = [&](int w, float2 (&b_dst)[STEPS]) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int wu = w + u;
+            const __amdgpu_buffer_rsrc_t rb =
+                sk_rsrc(Bvec + (size_t)min(wu, p.nwin - 1) * WS * N, wu < w_end ? b_bytes : 0u);
+            uint32_t boff = b_lane;
+#pragma unroll
+            for (int s = 0; s < KSTEPS; ++s, boff += b_step) {
+                const auto x = __builtin_amdgcn_raw_buffer_load_b64(rb, boff, 0, 0);
+                b_dst[u * KSTEPS + s] = make_float2(__int_as_float(x[0]), __int_as_float(x[1]));
+            }
+        }
+    };
+    // lane quarter kq of k-step s needs the dense row that index entry (4s + kq) * QS + vec selects
+    auto load_a = [&](int w, float (&a_dst)[STEPS]) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int wu = w + u;
+            const __amdgpu_buffer_rsrc_t ra_u = sk_rsrc(p.A, wu < w_end ? a_bytes : 0u);
+            const uint32_t win_row = (uint32_t)(min(wu, p.nwin - 1) * KS);
+            if (HIGH) {
+                static_assert(!HIGH || ND == 1, "one register of ranks per window");
+                dvec[u][0] = __builtin_amdgcn_ds_bpermute(dvec[u][0] << 2, civec[u]);
+            }
+#pragma unroll
+            for (int s = 0; s < KSTEPS; ++s) {
+                const int e = 4 * s * QS;
+                const int row = __builtin_amdgcn_ds_bpermute(perm_addr + (e % 64) * (int)sizeof(int32_t), dvec[u][e / 64]);
+                a_dst[u * KSTEPS + s] = sk_load(ra_u, a_lane + (win_row + (uint32_t)row) * row_bytes);
+            }
+        }
+    };
+    auto chunk = [&](int w, float (&a_cur)[STEPS], float2 (&b_cur)[STEPS], float (&a_nxt)[STEPS], float2 (&b_nxt)[STEPS]) {
+        if (w + U < w_end) {
+            load_b(w + U, b_nxt);
+            load_a(w + U, a_nxt);
+            if (w + 2 * U < w_end)
+                load_meta(w + 2 * U);
+        }
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            acc_even = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur[s], b_cur[s].x, acc_even, 0, 0, 0);
+            acc_odd = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur[s], b_cur[s].y, acc_odd, 0, 0, 0);
+        }
+    };
+
+    if (w_count > 0) {
+        load_meta(w_begin);
+        load_b(w_begin, b0);
+        load_a(w_begin, a0);
+        if (U < w_count)
+            load_meta(w_begin + U);
+    }
+    for (int w = w_begin; w < w_end; w += 2 * U) {
+        chunk(w, a0, b0, a1, b1);
+        if (w + U < w_end)
+            chunk(w + U, a1, b1, a0, b0);
+    }
+
+    // sum the waves' partial tiles in wave order: value x of a lane is register x % 4 (row
+    // 4 kq + x % 4) of the even (x < 4) or odd columns
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        red[wave][v][lane] = acc_even[v];
+        red[wave][4 + v][lane] = acc_odd[v];
+    }
+    __syncthreads();
+    for (int x = wave; x < 8; x += kSkinnyWaves) {
+        float s = red[0][x][lane];
+#pragma unroll
+        for (int y = 1; y < kSkinnyWaves; ++y)
+            s += red[y][x][lane];
+        const int row = 4 * kq + (x % 4);
+        if (row < M)
+            p.C[(size_t)row * N + (size_t)vec_g * 32 + 2 * jl + x / 4] = s;
+    }
+}
+
 template <int KS, int WS, bool HIGH, int RB, int U>
 static hipError_t launch_qs(const SpmmArgs& a)
 {
@@ -260,6 +404,33 @@ static hipError_t launch_qs(const SpmmArgs& a)
     return hipGetLastError();
 }
 
+template <int KS, int WS, bool HIGH, int U>
+static hipError_t launch_qs16(const SpmmArgs& a)
+{
+    SkinnyParams p;
+    p.A = a.A;
+    p.B = a.B;
+    p.D = a.D;
+    p.cinfo = a.cinfo;
+    p.C = a.C;
+    p.M = a.M;
+    p.N = a.N;
+    p.W = a.W;
+    p.K = a.K;
+    p.lda = a.lda;
+    p.nwin = a.W / WS;
+    const dim3 grid(a.N / 32), block(64 * kSkinnyWaves);
+    switch (a.Ns) {
+    case 128: spmm_skinny16_kernel<KS, WS, 4, HIGH, U><<<grid, block, 0, a.stream>>>(p); break;
+    case 64: spmm_skinny16_kernel<KS, WS, 2, HIGH, U><<<grid, block, 0, a.stream>>>(p); break;
+    case 32: spmm_skinny16_kernel<KS, WS, 1, HIGH, U><<<grid, block, 0, a.stream>>>(p); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+// the 16-row form reads B with 64-bit loads
+static bool skinny16_applies(const SpmmArgs& a) { return a.M <= 16 && reinterpret_cast<uintptr_t>(a.B) % 8 == 0; }
+
 // 32-row blocks per wave for a row count
 static int skinny_blocks(int M) { return M <= 32 ? 1 : M <= 64 ? 2 : 4; }
 
@@ -277,13 +448,19 @@ bool skinny_supported(const SpmmArgs& a)
     return a.window == 64 && (a.kept == 16 || a.kept == 8);
 }
 
-// Windows per chunk: about forty operand registers in flight per set.
+// Windows per chunk: sixteen kept rows for the 32-row form, thirty-two for the 16-row form (eight
+// k-steps either way; U1 is the count for sixteen k-steps).  Measured against chunks two and three
+// times as long: shorter chunks win by 5 to 15 %, most where there are more workgroups than CUs
+// and the smaller register footprint lets two of them share a CU.
 template <int KS, int WS, bool HIGH, int U1>
 static hipError_t launch_rb(const SpmmArgs& a)
 {
-    constexpr int UN = U1 >= 4 ? U1 / 2 : 1;  // for 64 and 128 rows
+    constexpr int UN = U1 >= 2 ? U1 / 2 : 1;
+    constexpr int U16 = 32 / WS > 0 ? 32 / WS : 1;
+    if (skinny16_applies(a))
+        return launch_qs16<KS, WS, HIGH, U16>(a);
     switch (skinny_blocks(a.M)) {
-    case 1: return launch_qs<KS, WS, HIGH, 1, U1>(a);
+    case 1: return launch_qs<KS, WS, HIGH, 1, UN>(a);
     case 2: return launch_qs<KS, WS, HIGH, 2, UN>(a);
     default: return launch_qs<KS, WS, HIGH, 4, UN>(a);
     }
@@ -293,7 +470,7 @@ hipError_t launch_skinny(const SpmmArgs& a)
 {
     const bool high = a.cinfo != nullptr;
     if (!high) {
-        if (a.kept == 32) return launch_qs<32, 32, false, 1, 1>(a);
+        if (a.kept == 32) return skinny16_applies(a) ? launch_qs16<32, 32, false, 1>(a) : launch_qs<32, 32, false, 1, 1>(a);
         if (a.kept == 16) return launch_rb<32, 16, false, 2>(a);
         if (a.kept == 12) return launch_rb<32, 12, false, 2>(a);
     } else {
