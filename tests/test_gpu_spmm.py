@@ -114,6 +114,21 @@ def test_decode_sized_rows_take_the_skinny_path(oracle, M, n, m, Ns):
         check(oracle, d, got)
 
 
+@pytest.mark.parametrize("M", [1, 16, 256])
+def test_operands_off_a_sixteen_byte_boundary_are_rejected(oracle, M):
+    """The kernels read A and B with 64- and 128-bit loads: the C-ABI rejects a B that is only
+    4-byte aligned instead of launching anything."""
+    d = datagen.init_data(M, 256, 1024, 1, 8, seed=M, dist="normal", b_scale=0.02)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    W = d["W"]
+    base = torch.empty(W * 256 + 1, dtype=torch.float32, device="cuda")
+    B_off = base[1:].view(W, 256)
+    assert B_off.data_ptr() % 8 == 4
+    C = torch.zeros((M, 256), dtype=torch.float32, device="cuda")
+    with pytest.raises(nmspmm.NmSpmmError, match="ALIGNMENT"):
+        nmspmm.spmm(dev(d["A_km"]), B_off, dev(D), dev(cinfo), C, M, 256, 1024, W, window, kept, 32, 128)
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 32])
 def test_decode_shape_8192(oracle, M):
     """One full-size config-4 shape: K = Ncols = 8192 at 1:8."""
