@@ -51,7 +51,7 @@ def test_matrix_core_tiles_every_pattern(oracle, n, m, Ns):
 
 
 def test_config1_512_cubed_2of4(oracle):
-    """BASELINE config 1: M = Ncols = K = 512, 2:4, uniform(-1,1); also checked against the dense
+    """The reference's own CPU-checkable case: M = Ncols = K = 512, 2:4, uniform(-1,1); also checked against the dense
     product with the decompressed operand in fp64."""
     d = datagen.init_data(512, 512, 512, 2, 4, seed=1001)
     got, fam = run_gpu(oracle, d, 128)
@@ -104,7 +104,7 @@ def test_split_k_through_workspace(oracle, split_k, n, m, Ns):
 @pytest.mark.parametrize("n,m", [(1, 8), (2, 8), (2, 4), (3, 8), (32, 32)])
 @pytest.mark.parametrize("Ns", [128, 64, 32])
 def test_decode_sized_rows_take_the_skinny_path(oracle, M, n, m, Ns):
-    """BASELINE config 4 in miniature: M <= 32, B ~ N(0, 0.02^2); K gives every wave of the
+    """The decode workload in miniature: M <= 32, B ~ N(0, 0.02^2); K gives every wave of the
     workgroup a different number of windows, some none."""
     K = 1024 if m == 8 else 1088 if m == 32 else 1152
     d = datagen.init_data(M, 256, K, n, m, seed=M + Ns, dist="normal", b_scale=0.02)
@@ -268,7 +268,7 @@ def test_leftover_tiles_in_a_launch_of_their_own(oracle, M, N, K, n, m):
 
 
 def test_llm_layer_shape_2of8(oracle):
-    """One BASELINE config-3 shape (M = 512, K = 4096, Ncols = 11008, 2:8, N(0,1) x N(0,0.02^2))."""
+    """One LLM-layer shape (M = 512, K = 4096, Ncols = 11008, 2:8, N(0,1) x N(0,0.02^2))."""
     d = datagen.init_data(512, 11008, 4096, 2, 8, seed=3001, dist="normal", b_scale=0.02)
     got, fam = run_gpu(oracle, d, 128)
     assert fam == "mfma"
@@ -277,7 +277,7 @@ def test_llm_layer_shape_2of8(oracle):
 
 @pytest.mark.parametrize("n,m", [(2, 4), (2, 8), (1, 8)])
 def test_full_size_4096_cubed_checksums_and_row_sample(oracle, n, m):
-    """BASELINE config 2 at full size.  The checker would need minutes for all of C, so: (1) rows
+    """The headline square workload at full size.  The checker would need minutes for all of C, so: (1) rows
     [0,32) and [4064,4096) are compared with the checker; (2) checksums that hold for any size:
     C . 1 = A . (B_dense . 1) and 1^T . C = (1^T . A) . B_dense, evaluated in fp64 from the inputs."""
     M = N = K = 4096
