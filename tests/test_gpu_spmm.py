@@ -296,3 +296,63 @@ def test_full_size_4096_cubed_checksums_and_row_sample(oracle, n, m):
     scale = np.sqrt(d["W"] * N / 9.0)  # std of a row/column sum of C for uniform(-1,1) operands
     assert np.max(np.abs(g64.sum(axis=1) - row_sums)) <= 1e-4 * scale
     assert np.max(np.abs(g64.sum(axis=0) - col_sums)) <= 1e-4 * scale
+
+
+def test_result_larger_than_four_gib(oracle):
+    """C of 32768 x 32768 floats is 4 GiB: every row's byte offset from C needs more than 32 bits
+    beyond row 32767 / 2.  A sample of rows from both halves is compared with the checker (rows are
+    independent, so the checker multiplies just those rows of A)."""
+    M = N = 32768
+    K = 64
+    free, _ = torch.cuda.mem_get_info()
+    if free < 6 * 2**30:
+        pytest.skip("needs 6 GiB of free device memory")
+    d = datagen.init_data(M, N, K, 2, 4, seed=4242)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), None, C, M, N, K, d["W"], window, kept, 32, 128)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == "mfma"
+    rows = np.array([0, 1, 255, 256, 16383, 16384, 16385, 20000, 32511, 32512, 32766, 32767])
+    got = C[torch.from_numpy(rows).cuda()].cpu().numpy()
+    A_rows = np.ascontiguousarray(d["A_km"][:, rows])
+    want = oracle.gemm_cpu(A_rows.reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), len(rows), N,
+                           d["W"]).reshape(len(rows), N)
+    assert np.isfinite(got).all() and scaled_max_error(got, want) <= REL_TOL
+    # nothing was left unwritten anywhere
+    assert not torch.isnan(C).any().item()
+
+
+def test_split_k_workspace_larger_than_four_gib(oracle):
+    """Four reduction slices of a 16384 x 16384 result: the slices sit up to 3 GiB beyond the
+    workspace's start and the second pass walks more than 2^32 bytes."""
+    M = N = 16384
+    K, split_k = 256, 4
+    free, _ = torch.cuda.mem_get_info()
+    if free < 8 * 2**30:
+        pytest.skip("needs 8 GiB of free device memory")
+    d = datagen.init_data(M, N, K, 1, 8, seed=4343)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    need = nmspmm.workspace_bytes(M, N, split_k)
+    assert need >= 4 * 2**30
+    ws = torch.full((need // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), dev(cinfo), C, M, N, K, d["W"], window, kept, 32, 128, split_k, ws)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == "mfma"
+    rows = np.array([0, 127, 128, 8191, 8192, 12345, 16255, 16383])
+    got = C[torch.from_numpy(rows).cuda()].cpu().numpy()
+    A_rows = np.ascontiguousarray(d["A_km"][:, rows])
+    want = oracle.gemm_cpu(A_rows.reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), len(rows), N,
+                           d["W"]).reshape(len(rows), N)
+    assert np.isfinite(got).all() and scaled_max_error(got, want) <= REL_TOL
+    assert not torch.isnan(C).any().item()
+
+
+def test_decode_kernel_with_a_million_column_vectors(oracle):
+    """Ncols = 2^22: 131072 workgroups of the decode kernel, B rows 16 MiB apart."""
+    M, N, K = 4, 1 << 22, 64
+    d = datagen.init_data(M, N, K, 2, 4, seed=4444, dist="normal", b_scale=0.02)
+    got, fam = run_gpu(oracle, d, 128)
+    assert fam == "skinny"
+    check(oracle, d, got)
