@@ -356,3 +356,26 @@ def test_decode_kernel_with_a_million_column_vectors(oracle):
     got, fam = run_gpu(oracle, d, 128)
     assert fam == "skinny"
     check(oracle, d, got)
+
+
+@pytest.mark.parametrize("M,family", [((1 << 22) - 4, "mfma"), ((1 << 22) + 4, "simt")])
+def test_row_counts_either_side_of_the_tile_kernels_limit(oracle, M, family):
+    """The tile kernel forms A offsets with 24-bit multiplies, which holds up to 2^22 - 1 rows;
+    beyond that the generic kernel runs.  Sampled rows against the checker on both sides."""
+    N, K = 128, 32
+    free, _ = torch.cuda.mem_get_info()
+    if free < 6 * 2**30:
+        pytest.skip("needs 6 GiB of free device memory")
+    d = datagen.init_data(M, N, K, 2, 4, seed=M % 1000)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), None, C, M, N, K, d["W"], window, kept, 32, 128)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == family
+    rows = np.array([0, 1, 255, 256, M // 2, M // 2 + 1, M - 257, M - 2, M - 1])
+    got = C[torch.from_numpy(rows).cuda()].cpu().numpy()
+    A_rows = np.ascontiguousarray(d["A_km"][:, rows])
+    want = oracle.gemm_cpu(A_rows.reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), len(rows), N,
+                           d["W"]).reshape(len(rows), N)
+    assert np.isfinite(got).all() and scaled_max_error(got, want) <= REL_TOL
+    assert not torch.isnan(C).any().item()
