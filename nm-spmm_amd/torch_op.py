@@ -31,9 +31,9 @@ class NMSparseLinear(torch.nn.Module):
     """y = x @ prune(weight).T + bias with an n:m pattern shared by 32 adjacent output features.
 
     weight: float32 CUDA tensor [out_features, in_features]; in_features % window == 0 and
-    out_features % 32 == 0.  Rows of x beyond the first dimension are flattened; the matrix-core
-    kernel needs their count to be a multiple of 4 (or at most 32 for the decode kernel), other
-    counts take the generic kernel.
+    out_features % 32 == 0.  Leading dimensions of x are flattened into rows; any row count runs on
+    the matrix-core kernels (the copy of x the row-major entry point makes is padded to a row pitch
+    of a multiple of four floats).
     """
 
     def __init__(self, weight, n, m, bias=None):
