@@ -154,8 +154,9 @@ int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t*
  * multiplies the same activations).  nmspmm_spmm_rowmajor does both steps: the workspace holds the
  * column-major copy followed by the split-K slices, nmspmm_workspace_bytes_rowmajor() bytes, never
  * optional.  The copy's row pitch is M rounded up to 4 floats, so any M above 32 runs on the
- * matrix-core kernel (nmspmm_spmm itself needs M % 4 == 0 for that).  Other arguments and
- * requirements as nmspmm_spmm. */
+ * matrix-core kernel (nmspmm_spmm itself needs M % 4 == 0 for that).  Up to 8 rows (decoding) the
+ * kernel reads the row-major A in place and nothing is copied; the workspace is still required,
+ * so that a caller sizes it once for every M.  Other arguments and requirements as nmspmm_spmm. */
 int nmspmm_transpose_device(const float* src, int rows, int cols, float* dst, void* stream);
 size_t nmspmm_workspace_bytes_rowmajor(int M, int N, int K, int split_k);
 int nmspmm_spmm_rowmajor(const float* A_rowmajor, const float* B, const int32_t* D,

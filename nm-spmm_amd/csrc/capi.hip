@@ -344,9 +344,12 @@ size_t nmspmm_workspace_bytes(int M, int N, int split_k)
 
 // lda: floats between consecutive dense rows of A; 0 lets the function choose (M, or M rounded up
 // to 4 when `may_pad` allows it and that puts the shape on the matrix-core path) and reports it.
+// a_rowmajor: A is row-major M x K with `lda` floats between rows; only the decode kernels take
+// that, and kNotTaken comes back (nothing launched) when they do not take the shape.
+constexpr int kNotTaken = -1000;
 static int spmm_impl(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C, int M,
                      int N, int K, int W, int window, int kept, int vec_len, int Ns, int split_k, void* workspace,
-                     size_t workspace_bytes, void* stream, int lda, bool dry_run, int* lda_out)
+                     size_t workspace_bytes, void* stream, int lda, bool dry_run, int* lda_out, bool a_rowmajor = false)
 {
     if (!A || !B || !D || !C)
         return NMSPMM_ERR_NULL_POINTER;
@@ -377,6 +380,7 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     a.slice_stride = slice_stride(M, N);
     a.M = M;
     a.lda = lda > 0 ? lda : M;
+    a.a_rowmajor = a_rowmajor;
     a.N = N;
     a.K = K;
     a.W = W;
@@ -402,6 +406,8 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     if (dry_run)
         return NMSPMM_OK;
 
+    if (a_rowmajor && !(M <= 32 && skinny_supported(a)))
+        return kNotTaken;
     hipError_t e;
     // up to 32 rows the decode kernel always wins; up to 128 it competes with the tile kernel at
     // the caller's split
@@ -471,6 +477,15 @@ int nmspmm_spmm_rowmajor(const float* A_rowmajor, const float* B, const int32_t*
     float* const At = (float*)workspace;
     float* const slices = At + rowmajor_copy_floats(M, K);
     const size_t slice_bytes = workspace_bytes - sizeof(float) * rowmajor_copy_floats(M, K);
+    // Up to 8 rows the decode kernel reads a row-major A in place: no copy, one launch.  (A lane
+    // then fetches its operand from a cache line of its own row; measured against the copy, which
+    // costs 2.5 to 4 us at these sizes: level up to 8 rows, 0.4 to 2 times slower from 16 on.)
+    if (M <= 8 && aligned16(A_rowmajor)) {
+        const int st = spmm_impl(A_rowmajor, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k,
+                                 slices, slice_bytes, stream, K, false, nullptr, true);
+        if (st != kNotTaken)
+            return st;
+    }
     // check every argument and settle the row pitch of the copy before anything is launched
     int lda = M;
     const int st = spmm_impl(At, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k, slices,

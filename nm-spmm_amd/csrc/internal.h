@@ -20,6 +20,8 @@ struct SpmmArgs {
     int M, N, K, W;
     int lda;               // floats between consecutive dense rows of A; M unless the copy of a
                            // row-major A was padded (matrix-core path only)
+    bool a_rowmajor;       // A is row-major M x K instead, `lda` floats between its rows (taken by
+                           // the one-block decode kernels only)
     int window, kept, vec_len, Ns;
     int split_k;
     float* tail_ws;        // optional scratch for splitting the tiles of a ragged last round (split_k == 1)

@@ -445,6 +445,8 @@ size_t mfma_tail_workspace_bytes(const SpmmArgs& a)
 
 bool mfma_supported(const SpmmArgs& a)
 {
+    if (a.a_rowmajor)
+        return false;
     if (a.vec_len != 32 || (a.Ns != 32 && a.Ns != 64 && a.Ns != 128))
         return false;
     if (a.lda % 4 != 0 || a.lda < a.M || a.M < 32)

@@ -213,6 +213,8 @@ static hipError_t launch_short_cfg(const SpmmArgs& a)
 
 bool short_supported(const SpmmArgs& a)
 {
+    if (a.a_rowmajor)
+        return false;
     if (a.cinfo != nullptr || a.vec_len >= 32 || (a.vec_len != 4 && a.vec_len != 8 && a.vec_len != 16))
         return false;
     if (a.N % 128 != 0 || a.Ns % 32 != 0 || a.K % kChunk != 0 || a.M <= 32 || a.lda % 4 != 0 || a.lda < a.M)

@@ -64,6 +64,8 @@ __global__ void __launch_bounds__(64) spmm_simt_kernel(const SimtParams p)
 
 bool simt_supported(const SpmmArgs& a)
 {
+    if (a.a_rowmajor)
+        return false;
     return a.vec_len == 4 || a.vec_len == 8 || a.vec_len == 16 || a.vec_len == 32;
 }
 

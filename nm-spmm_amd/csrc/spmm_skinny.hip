@@ -28,6 +28,9 @@ struct SkinnyParams {
     float* C;
     int M, N, W, K, lda;
     int nwin;
+    // element (i, k) of A lies i * a_row_stride + k * a_k_stride bytes into its a_bytes bytes:
+    // (4, 4 * lda) for the column-major operand, (4 * lda, 4) for a row-major one (up to 32 rows)
+    uint32_t a_row_stride, a_k_stride, a_bytes;
 };
 
 __device__ inline __amdgpu_buffer_rsrc_t sk_rsrc(const void* base, uint32_t bytes)
@@ -107,9 +110,9 @@ spmm_skinny_kernel(const SkinnyParams p)
     const float* const Bvec = p.B + (size_t)vec_g * 32;
     const int32_t* const Dblk = p.D + (size_t)jb * p.W * QS;
     const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)jb * p.nwin * KS : nullptr;
-    const uint32_t a_bytes = (uint32_t)((size_t)p.K * lda * sizeof(float));
-    const uint32_t a_lane = RB * j < M ? (uint32_t)(RB * j * sizeof(float)) : kSkNoLoad;
-    const uint32_t row_bytes = (uint32_t)((size_t)lda * sizeof(float));
+    const uint32_t a_bytes = p.a_bytes;
+    const uint32_t a_lane = RB * j < M ? (uint32_t)(RB * j) * p.a_row_stride : kSkNoLoad;
+    const uint32_t row_bytes = p.a_k_stride;
     const uint32_t b_lane = (uint32_t)(((size_t)h * N + j) * sizeof(float));
     const uint32_t b_step = (uint32_t)(2 * (size_t)N * sizeof(float));
     const uint32_t b_bytes = (uint32_t)(((size_t)(WS - 1) * N + 32) * sizeof(float));
@@ -270,9 +273,9 @@ spmm_skinny16_kernel(const SkinnyParams p)
     const float* const Bvec = p.B + (size_t)vec_g * 32;
     const int32_t* const Dblk = p.D + (size_t)jb * p.W * QS;
     const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)jb * p.nwin * KS : nullptr;
-    const uint32_t a_bytes = (uint32_t)((size_t)p.K * lda * sizeof(float));
-    const uint32_t a_lane = jl < M ? (uint32_t)(jl * sizeof(float)) : kSkNoLoad;
-    const uint32_t row_bytes = (uint32_t)((size_t)lda * sizeof(float));
+    const uint32_t a_bytes = p.a_bytes;
+    const uint32_t a_lane = jl < M ? (uint32_t)jl * p.a_row_stride : kSkNoLoad;
+    const uint32_t row_bytes = p.a_k_stride;
     const uint32_t b_lane = (uint32_t)(((size_t)kq * N + 2 * jl) * sizeof(float));
     const uint32_t b_step = (uint32_t)(4 * (size_t)N * sizeof(float));
     const uint32_t b_bytes = (uint32_t)(((size_t)(WS - 1) * N + 32) * sizeof(float));
@@ -394,6 +397,9 @@ static hipError_t launch_qs(const SpmmArgs& a)
     p.K = a.K;
     p.lda = a.lda;
     p.nwin = a.W / WS;
+    p.a_row_stride = (uint32_t)(a.a_rowmajor ? a.lda * sizeof(float) : sizeof(float));
+    p.a_k_stride = (uint32_t)(a.a_rowmajor ? sizeof(float) : a.lda * sizeof(float));
+    p.a_bytes = (uint32_t)((size_t)(a.a_rowmajor ? a.M : a.K) * a.lda * sizeof(float));
     const dim3 grid(a.N / 32), block(64 * kSkinnyWaves);
     switch (a.Ns) {
     case 128: spmm_skinny_kernel<KS, WS, 4, HIGH, RB, U><<<grid, block, 0, a.stream>>>(p); break;
@@ -419,6 +425,9 @@ static hipError_t launch_qs16(const SpmmArgs& a)
     p.K = a.K;
     p.lda = a.lda;
     p.nwin = a.W / WS;
+    p.a_row_stride = (uint32_t)(a.a_rowmajor ? a.lda * sizeof(float) : sizeof(float));
+    p.a_k_stride = (uint32_t)(a.a_rowmajor ? sizeof(float) : a.lda * sizeof(float));
+    p.a_bytes = (uint32_t)((size_t)(a.a_rowmajor ? a.M : a.K) * a.lda * sizeof(float));
     const dim3 grid(a.N / 32), block(64 * kSkinnyWaves);
     switch (a.Ns) {
     case 128: spmm_skinny16_kernel<KS, WS, 4, HIGH, U><<<grid, block, 0, a.stream>>>(p); break;
@@ -438,10 +447,16 @@ bool skinny_supported(const SpmmArgs& a)
 {
     if (a.M > NMSPMM_SK_MAX_M || a.vec_len != 32 || (a.Ns != 32 && a.Ns != 64 && a.Ns != 128))
         return false;
-    if (a.lda < a.M || a.lda % skinny_blocks(a.M) != 0)  // a lane's run of rows must not straddle the pitch
-        return false;
-    if ((size_t)a.K * a.lda * sizeof(float) >= 0x80000000ull)
-        return false;
+    if (a.a_rowmajor) {
+        // a lane then loads one float of A per k-step, whatever the pitch: the one-block forms only
+        if (a.M > 32 || a.lda < a.K || (size_t)a.M * a.lda * sizeof(float) >= 0x80000000ull)
+            return false;
+    } else {
+        if (a.lda < a.M || a.lda % skinny_blocks(a.M) != 0)  // a lane's run of rows must not straddle the pitch
+            return false;
+        if ((size_t)a.K * a.lda * sizeof(float) >= 0x80000000ull)
+            return false;
+    }
     const bool high = a.cinfo != nullptr;
     if (!high)
         return a.window == 32 && ((a.kept == 32 && a.M <= 32) || a.kept == 16 || a.kept == 12);

@@ -77,3 +77,29 @@ def test_row_major_activations(oracle, M, N, K, n, m, split_k):
     with pytest.raises(nmspmm.NmSpmmError):
         nmspmm.spmm_rowmajor(A_rm, dev(d["BT"]), dev(D), None if cinfo is None else dev(cinfo), C, M, N, K, d["W"], window,
                              kept, ws[: need // 4 - 4], 32, 128, split_k)
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 5, 8, 9, 16, 32])
+@pytest.mark.parametrize("n,m,Ns", [(1, 8, 128), (2, 8, 64), (2, 4, 32), (3, 8, 128), (32, 32, 128)])
+def test_decode_sized_row_major_activations(oracle, M, n, m, Ns):
+    """Up to 8 rows the decode kernel reads the row-major A in place, above it reads the copy;
+    either way the result is the column-major entry point's, bit for bit, and the checker's within
+    tolerance.  The head of the workspace (where a copy would go) stays untouched in place."""
+    K = 1024 if m == 8 else 1088 if m == 32 else 1152
+    N = 256
+    d = datagen.init_data(M, N, K, n, m, seed=3 * M + n, dist="normal", b_scale=0.02)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, Ns)
+    A_rm = dev(d["A_km"].T)
+    dc = None if cinfo is None else dev(cinfo)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    ws = torch.full((nmspmm.workspace_bytes_rowmajor(M, N, K, 1) // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    nmspmm.spmm_rowmajor(A_rm, dev(d["BT"]), dev(D), dc, C, M, N, K, d["W"], window, kept, ws, 32, Ns, 1)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == "skinny"
+    assert torch.isnan(ws).all().item() == (M <= 8)
+    C2 = torch.empty_like(C)
+    nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), dc, C2, M, N, K, d["W"], window, kept, 32, Ns)
+    assert torch.equal(C, C2)
+    want = oracle.gemm_cpu(d["A_km"].reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), M, N, d["W"]).reshape(M, N)
+    got = C.cpu().numpy()
+    assert np.isfinite(got).all() and scaled_max_error(got, want) <= REL_TOL
