@@ -64,6 +64,7 @@ class NMSparseLinear(torch.nn.Module):
         self.register_buffer("column_info", cinfo)
         self.register_buffer("bias", None if bias is None else bias.detach().to(torch.float32))
         self._workspace = None
+        self._plans = {}
 
     def dense_weight(self):
         """The pruned weight as a dense [out_features, in_features] tensor (for checking)."""
@@ -81,8 +82,10 @@ class NMSparseLinear(torch.nn.Module):
         y = torch.empty((M, N), dtype=torch.float32, device=x.device)
         if M == 0:
             return y.reshape(*lead, N)
-        split = _nm.suggest_split_k(M, N, self.W, self.kept)
-        need = _nm.workspace_bytes_rowmajor(M, N, K, split) // 4
+        if M not in self._plans:  # two library calls per row count, not per forward
+            split = _nm.suggest_split_k(M, N, self.W, self.kept)
+            self._plans[M] = (split, _nm.workspace_bytes_rowmajor(M, N, K, split) // 4)
+        split, need = self._plans[M]
         if self._workspace is None or self._workspace.numel() < need or self._workspace.device != x.device:
             self._workspace = torch.empty(need, dtype=torch.float32, device=x.device)
         _nm.spmm_rowmajor(x2, self.values, self.indices, self.column_info, y, M, N, K, self.W, self.window, self.kept,
