@@ -14,6 +14,9 @@
 //    zero, or neighbouring values that land in accumulators that are never stored.
 //  * Index metadata comes as one wave-wide load per window ([kept][Ns/32] ints, plus the 64-entry
 //    column_info list on the high-sparsity layout) and is handed to the lanes with ds_bpermute.
+//  * Up to 16 rows a second kernel does the same on v_mfma_f32_16x16x4_f32 (further down).
+//  * A itself may be row-major for the one-block forms: a lane loads one float of A per k-step,
+//    so the storage order is two strides.  The C-ABI uses that up to 8 rows.
 #include "internal.h"
 
 namespace nmspmm {
