@@ -86,6 +86,7 @@ struct TailPlan {
     long long head;  // tiles computed whole
     long long tail;  // tiles computed in slices
     int slices;
+    int sub;         // > 1: the tail tiles run as `sub` pieces along M each, on waves of blocks / sub blocks
     size_t ws_bytes; // scratch needed
     bool separate;   // without scratch: give the tail tiles a launch of their own (they then spread
                      // one or two per CU instead of landing packed on the CUs that free up last)
@@ -99,22 +100,51 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept)
     t.head = tiles;
     t.tail = 0;
     t.slices = 1;
+    t.sub = 1;
     t.ws_bytes = 0;
     t.separate = false;
     const long long rest = tiles % slots;
     if (tiles < slots || rest == 0)
         return t;
-    // In steady state (two or more full rounds) workgroups finish at staggered times and the
-    // dispatcher refills a CU's freed slots together, so the leftover tiles end up packed on few
-    // CUs and the last round lasts as long as a full one (measured: 2752 tiles on 512 slots take six
-    // rounds, not 5.4).  A launch of their own spreads them one (or two) per CU.  After a single
-    // full round the leftovers spread over idle CUs by themselves (measured).
-    if (tiles < 2 * slots || rest > slots / 2)
-        return t;
-    t.separate = true;
-    t.head = tiles - rest;
-    t.tail = rest;
-    // With scratch, a handful of leftover tiles (at most an eighth of the slots) is also cut into
+    if (t.blocks == 8) {
+        // 256-row waves, two workgroups per CU.  Left in the launch, the leftover tiles land packed
+        // on the CUs that free up first and the last round lasts as long as a full one (measured:
+        // 2752 tiles on 512 slots take six rounds, not 5.4; 768 tiles take two, not 1.5).  In a
+        // launch of their own they spread over all CUs, and cut into 2 or 4 pieces along M (128- or
+        // 64-row waves, 4 % and 20 % more loads per MFMA) they spread more evenly still: the piece
+        // count per CU, times the piece's share of a tile, decides.  T is the time a CU needs for
+        // one tile when its pipes are busy; a CU left with a single workgroup runs at about 0.9.
+        // Over 96 ragged LLM-layer shapes this choice is 4.1 % faster on average than leaving the
+        // tiles in the launch (best choice per shape: 4.3 %), up to 30 % on single shapes.
+        const double T = kept * 53.5e-9 * (2.0 / 1.04) * nwin / 2.0;
+        static const double piece_cost[3] = {1.0, 1.04, 1.2};
+        double best = 2.0 * T;
+        int best_sub = 0;
+        for (int i = 0, sub = 1; i < 3; ++i, sub *= 2) {
+            const long long busiest = (rest * sub + 255) / 256;
+            const double s = busiest * T / sub * piece_cost[i] / (busiest == 1 ? 0.9 : 1.0) + 6e-6;
+            if (s < best) {
+                best = s;
+                best_sub = sub;
+            }
+        }
+        if (best_sub == 0)
+            return t;
+        t.separate = true;
+        t.head = tiles - rest;
+        t.tail = rest;
+        t.sub = best_sub;
+    } else {
+        // 128-row waves, four workgroups per CU: the finer grain already fills the last round well
+        // after one full round (a launch of their own was measured 0 to 16 % SLOWER there).  In
+        // steady state (two or more full rounds) a launch of their own spreads few leftovers.
+        if (tiles < 2 * slots || rest > slots / 2)
+            return t;
+        t.separate = true;
+        t.head = tiles - rest;
+        t.tail = rest;
+    }
+    // With scratch, a handful of leftover tiles (at most an eighth of the slots) is instead cut into
     // four pieces along K, so that their launch occupies four times as many CUs for a quarter of
     // the time.  The pieces pay a second pass: measured +2 % to +5 % up to that size, a loss beyond.
     if (rest > slots / 8 || nwin / 4 < 4)

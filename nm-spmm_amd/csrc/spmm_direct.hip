@@ -50,6 +50,8 @@ struct DirectParams {
     int tile_offset;     // first logical tile of this launch (the tail tiles get a launch of their own)
     int tail_slices;     // > 1: every workgroup of this launch is one of tail_slices pieces of a tile along K
     float* tail_ws;      // [tile of this launch][slice][MS][NS] partial tiles
+    int sub_tiles;       // > 1: every workgroup of this launch is one of sub_tiles pieces, along M, of a
+                         // tile of sub_tiles * MS rows (the tile walk and tiles_m are those taller tiles')
 };
 
 struct float8 { float4 lo, hi; };
@@ -120,8 +122,11 @@ spmm_direct_kernel(const DirectParams p)
     // tail slices, consecutive ids are the pieces of one tile.
     const bool tail_unit = p.tail_slices > 1;
     const int unit = blockIdx.x;  // slice number among the slices of this launch
-    int logical;
-    if (!tail_unit) {
+    int logical, sub = 0;
+    if (p.sub_tiles > 1) {
+        logical = p.tile_offset + unit / p.sub_tiles;
+        sub = unit % p.sub_tiles;
+    } else if (!tail_unit) {
         const int total = gridDim.x;
         const int id = blockIdx.x;
         const int q = total / kXcds, r = total % kXcds;
@@ -154,7 +159,7 @@ spmm_direct_kernel(const DirectParams p)
     const int h = lane >> 5;
     const int j = lane & 31;
     const int M = p.M, N = p.N, lda = p.lda;
-    const int bi = tile_m * MS + wr * MW;     // first row of this wave (may be >= M: loads nothing)
+    const int bi = (tile_m * p.sub_tiles + sub) * MS + wr * MW;  // first row of this wave (may be >= M: loads nothing)
     const int bj = tile_n * NS + vec * 32;
 
     const float* const Ablk = p.A + min(bi, lda);
@@ -363,6 +368,7 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     p.tile_offset = 0;
     p.tail_slices = 1;
     p.tail_ws = nullptr;
+    p.sub_tiles = 1;
     // the plan counts 128-column tiles of RM blocks; it applies when that is this tile shape
     const bool own_tail = plan.separate && WR == 1 && QS == 4 && RM == plan.blocks;
     const dim3 block(64 * QS * WR);
@@ -378,6 +384,20 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     if (e != hipSuccess)
         return e;
     p.tile_offset = (int)plan.head;
+    if (plan.slices == 1 && plan.sub > 1) {
+        // shorter waves for the leftovers: each tile in plan.sub pieces along M, so that the pieces
+        // fill the CUs more evenly than whole tiles would; same sums in the same order, no scratch
+        p.sub_tiles = plan.sub;
+        grid.x = (unsigned)(plan.tail * plan.sub);
+        if (RM / plan.sub == 4) {
+            if constexpr (RM >= 8)
+                spmm_direct_kernel<KS, WS, QS, WR, 4, HIGH><<<grid, block, 0, a.stream>>>(p);
+        } else {
+            if constexpr (RM >= 4)
+                spmm_direct_kernel<KS, WS, QS, WR, 2, HIGH><<<grid, block, 0, a.stream>>>(p);
+        }
+        return hipGetLastError();
+    }
     p.tail_slices = plan.slices;
     p.tail_ws = plan.slices > 1 ? a.tail_ws : nullptr;
     grid.x = (unsigned)(plan.tail * plan.slices);
@@ -405,10 +425,11 @@ static TailPlan tail_plan_for(const SpmmArgs& a, bool have_scratch)
     none.slices = 1;
     none.ws_bytes = 0;
     none.separate = false;
+    none.sub = 1;
     if (a.split_k != 1 || a.Ns != 128 || NMSPMM_RM_TALL != 8)
         return none;
     TailPlan t = plan_tail(a.M, a.N, a.W / a.kept, a.kept);
-    if (t.head + t.tail * t.slices > 0x7fffffffLL)
+    if (t.head + t.tail * t.slices * t.sub > 0x7fffffffLL)
         return none;
     if (have_scratch && t.slices > 1 && (a.tail_ws == nullptr || a.tail_ws_bytes < t.ws_bytes)) {
         t.slices = 1;  // no scratch: the tail can still have a launch of its own

@@ -242,10 +242,14 @@ def test_ragged_last_round_is_split_along_k_through_scratch(oracle, M, N, K, n, 
             assert scaled_max_error(C[r0:r1].cpu().numpy(), want) <= REL_TOL
 
 
-@pytest.mark.parametrize("M,N,K,n,m", [(4096, 8448, 256, 2, 4), (8192, 4224, 512, 1, 8)])
+@pytest.mark.parametrize("M,N,K,n,m", [(4096, 8448, 256, 2, 4), (8192, 4224, 512, 1, 8), (2048, 11008, 256, 2, 4),
+                                       (4096, 11008, 4096, 1, 8), (1024, 24576, 4096, 2, 8), (2000, 11008, 256, 2, 4)])
 def test_leftover_tiles_in_a_launch_of_their_own(oracle, M, N, K, n, m):
-    """Two full rounds of tiles and a few leftovers, too few windows to cut them: the leftovers run
-    as a second launch of the same kernel; every tile must still be computed exactly once."""
+    """More tiles than the GPU holds at once, a ragged last round and too few windows to cut its
+    tiles along K: the leftovers run as a second launch, whole (the first two shapes) or as two or
+    four shorter pieces along M each (688 tiles of 256 rows on 512 slots: 176 leftovers in four
+    pieces; 1376: 352 in two; 768: 256 in two; the last shape with a ragged row count as well).
+    Every tile must still be computed exactly once."""
     d = datagen.init_data(M, N, K, n, m, seed=M + K)
     window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
     assert nmspmm.tail_workspace_bytes(M, N, d["W"], kept) == 0
