@@ -49,16 +49,52 @@ __host__ __device__ inline void split_windows(int nwin, int split_k, int z, int*
 // one wave per SIMD, runs at about 0.9 of its rate); after two or more the leftovers land packed
 // on the CUs that happen to free up and cost a whole round, unless they are few enough to get a
 // launch of their own (plan_tail, unsplit reductions only).  Constants fitted to sweeps on one MI355X (mean error 6 %).
+// Pipe time of a 256-row wave relative to a 128-row one: twice the rows with half the B and index
+// loads per MFMA (4 % less), except at 8 kept rows per window (1:8), where the four 128-row waves
+// per SIMD hide the gather's cache misses better than two tall ones (measured 1 to 7 % in favour
+// of the shorter waves over eight shapes, 4 % at 4096 cubed).
+inline double tall_wave_cost(int kept) { return kept <= 8 ? 2.0 / 0.98 : 2.0 / 1.04; }
+
+// Leftover tiles of 256-row waves (two workgroups per CU) after at least one full round: `rest`
+// tiles, each `unit` seconds of a CU's pipes.  Left in the launch they land packed on the CUs that
+// free up first and the last round lasts as long as a full one (measured: 2752 tiles on 512 slots
+// take six rounds, not 5.4; 768 tiles take two, not 1.5).  In a launch of their own they spread
+// over all CUs, and cut into 2 or 4 pieces along M (128- or 64-row waves, 4 % and 20 % more loads
+// per MFMA) they spread more evenly still: the piece count of the busiest CU, times the piece's
+// share of a tile, decides.  A CU left with a single workgroup runs at about 0.9; the second
+// launch costs about 12 us (the gap, and the first launch draining).  Returns the modelled time
+// of the cheapest way and its piece count (0: leave the tiles in the launch).  Over 96 ragged
+// LLM-layer shapes this choice is 4.1 % faster on average than leaving the tiles in the launch
+// (best choice per shape: 4.3 %), up to 30 % on single shapes.
+inline double tall_tail_seconds(long long rest, double unit, int* pieces)
+{
+    static const double piece_cost[3] = {1.0, 1.04, 1.2};
+    double best = 2.0 * unit;
+    int best_sub = 0;
+    for (int i = 0, sub = 1; i < 3; ++i, sub *= 2) {
+        const long long busiest = (rest * sub + 255) / 256;
+        const double s = busiest * unit / sub * piece_cost[i] / (busiest == 1 ? 0.9 : 1.0) + 12e-6;
+        if (s < best) {
+            best = s;
+            best_sub = sub;
+        }
+    }
+    if (pieces)
+        *pieces = best_sub;
+    return best;
+}
 inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks, int split)
 {
-    const double per_window = kept * 53.5e-9 * (blocks == 8 ? 2.0 / 1.04 : 1.0);
+    const double per_window = kept * 53.5e-9 * (blocks == 8 ? tall_wave_cost(kept) : 1.0);
     const double unit = per_window * ((nwin + split - 1) / split);
     const long long groups = (long long)((M + 32 * blocks - 1) / (32 * blocks)) * ((N + 127) / 128) * split;
     const int slots = blocks == 8 ? 2 : 4;
     const long long full = groups / (256 * slots), rest = groups % (256 * slots);
     const long long busiest = (rest + 255) / 256;
     double t = (double)full * slots * unit;
-    if (busiest > 0) {
+    if (busiest > 0 && blocks == 8 && split == 1 && full >= 1) {
+        t += tall_tail_seconds(rest, unit, nullptr);  // plan_tail gives these leftovers a launch of shorter pieces
+    } else if (busiest > 0) {
         const double spread = busiest * unit / (busiest == 1 ? 0.9 : 1.0);
         if (full < 2)
             t += spread;
@@ -107,33 +143,14 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept)
     if (tiles < slots || rest == 0)
         return t;
     if (t.blocks == 8) {
-        // 256-row waves, two workgroups per CU.  Left in the launch, the leftover tiles land packed
-        // on the CUs that free up first and the last round lasts as long as a full one (measured:
-        // 2752 tiles on 512 slots take six rounds, not 5.4; 768 tiles take two, not 1.5).  In a
-        // launch of their own they spread over all CUs, and cut into 2 or 4 pieces along M (128- or
-        // 64-row waves, 4 % and 20 % more loads per MFMA) they spread more evenly still: the piece
-        // count per CU, times the piece's share of a tile, decides.  T is the time a CU needs for
-        // one tile when its pipes are busy; a CU left with a single workgroup runs at about 0.9.
-        // Over 96 ragged LLM-layer shapes this choice is 4.1 % faster on average than leaving the
-        // tiles in the launch (best choice per shape: 4.3 %), up to 30 % on single shapes.
-        const double T = kept * 53.5e-9 * (2.0 / 1.04) * nwin / 2.0;
-        static const double piece_cost[3] = {1.0, 1.04, 1.2};
-        double best = 2.0 * T;
-        int best_sub = 0;
-        for (int i = 0, sub = 1; i < 3; ++i, sub *= 2) {
-            const long long busiest = (rest * sub + 255) / 256;
-            const double s = busiest * T / sub * piece_cost[i] / (busiest == 1 ? 0.9 : 1.0) + 6e-6;
-            if (s < best) {
-                best = s;
-                best_sub = sub;
-            }
-        }
-        if (best_sub == 0)
+        int pieces = 0;
+        tall_tail_seconds(rest, kept * 53.5e-9 * tall_wave_cost(kept) * nwin, &pieces);
+        if (pieces == 0)
             return t;
         t.separate = true;
         t.head = tiles - rest;
         t.tail = rest;
-        t.sub = best_sub;
+        t.sub = pieces;
     } else {
         // 128-row waves, four workgroups per CU: the finer grain already fills the last round well
         // after one full round (a launch of their own was measured 0 to 16 % SLOWER there).  In

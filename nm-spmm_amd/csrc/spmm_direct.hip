@@ -86,7 +86,10 @@ __device__ inline float buffer_load_f1(__amdgpu_buffer_rsrc_t r, uint32_t byte_o
 }
 
 // Tuning knobs (compile-time): waves per SIMD the register allocation must allow for 128-row
-// waves (256-row waves get two), and the tile-walk band height.
+// waves (256-row waves get two), and the tile-walk band height.  The 2:8 geometry (64-row windows,
+// 16 kept) would take 134 registers at three waves per SIMD, six too many for the four workgroups
+// per CU the run-time model counts on: it is compiled for four (128 registers, nothing spills;
+// the dense geometry would spill, the others are below 128 anyway).
 #ifndef NMSPMM_OCC
 #define NMSPMM_OCC 3
 #endif
@@ -101,7 +104,7 @@ __device__ inline float buffer_load_f1(__amdgpu_buffer_rsrc_t r, uint32_t byte_o
 // block (Ns = 32*QS), WR: waves along M, RM: 32-row blocks per wave (2, 4 or 8), HIGH:
 // high-sparsity layout (D holds ranks into the window's column_info list).
 template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
-__global__ void __launch_bounds__(64 * QS * WR, RM == 8 ? 2 : NMSPMM_OCC)
+__global__ void __launch_bounds__(64 * QS * WR, RM == 8 ? 2 : (HIGH && WS == 16) ? 4 : NMSPMM_OCC)
 spmm_direct_kernel(const DirectParams p)
 {
     static_assert(RM == 2 || RM == 4 || RM == 8, "64-, 128- or 256-row waves");
