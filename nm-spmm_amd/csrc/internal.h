@@ -52,7 +52,10 @@ __host__ __device__ inline void split_windows(int nwin, int split_k, int z, int*
 // Pipe time of a 256-row wave relative to a 128-row one: twice the rows with half the B and index
 // loads per MFMA (4 % less), except at 8 kept rows per window (1:8), where the four 128-row waves
 // per SIMD hide the gather's cache misses better than two tall ones (measured 1 to 7 % in favour
-// of the shorter waves over eight shapes, 4 % at 4096 cubed).
+// of the shorter waves on shapes of up to three rounds, 4 % at 4096 cubed; from five rounds on the
+// tall waves are 1 % ahead again, which this leaves on the table).  A finer table per layout
+// (2:8 is level at 4096 cubed) was tried and chose worse on large shapes, where the tall waves'
+// smaller traffic counts for more than one exact round shows.
 inline double tall_wave_cost(int kept) { return kept <= 8 ? 2.0 / 0.98 : 2.0 / 1.04; }
 
 // Leftover tiles of 256-row waves (two workgroups per CU) after at least one full round: `rest`
@@ -110,6 +113,9 @@ inline int choose_wave_blocks(int M, int N, int nwin, int kept, int split)
 {
     if (M <= 128)
         return 4;
+#ifdef NMSPMM_FORCE_BLOCKS  // tuning builds: measure one wave height everywhere
+    return NMSPMM_FORCE_BLOCKS;
+#endif
     return model_kernel_seconds(M, N, nwin, kept, 8, split) < model_kernel_seconds(M, N, nwin, kept, 4, split) ? 8 : 4;
 }
 
