@@ -411,9 +411,12 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     hipError_t e;
     // up to 32 rows the decode kernel always wins; up to 128 it competes with the tile kernel at
     // the caller's split
-    if (skinny_supported(a) && (M <= 32 || model_decode_seconds(M, N, W / kept, kept) <
-                                               model_tile_seconds(M, N, W / kept, kept, split_k) ||
-                                !mfma_supported(a))) {
+#ifdef NMSPMM_FORCE_DECODE  // tuning builds: the decode kernel wherever it applies
+    const bool decode_wins = true;
+#else
+    const bool decode_wins = model_decode_seconds(M, N, W / kept, kept) < model_tile_seconds(M, N, W / kept, kept, split_k);
+#endif
+    if (skinny_supported(a) && (M <= 32 || decode_wins || !mfma_supported(a))) {
         // one launch, reduction inside the workgroup: split_k and the workspace are not needed
         e = launch_skinny(a);
         g_last_kernel = "skinny";
