@@ -130,7 +130,11 @@ size_t nmspmm_workspace_bytes(int M, int N, int split_k);
 
 /* Bytes of optional scratch with which nmspmm_spmm, called with split_k == 1 and Ns == 128, cuts
  * the few leftover tiles of a ragged last round into four pieces along K so that they occupy four
- * times as many CUs (0 when there is nothing to gain).  No counterpart in the reference. */
+ * times as many CUs (0 when there is nothing to gain).  The pieces are summed in a fixed order,
+ * but not in the order of an unsplit reduction: with the scratch the affected tiles of C may
+ * differ from a call without it in the last bits (both within the 1e-4 bound).  Without scratch
+ * leftover tiles still get a launch of their own where that pays, whole or in shorter pieces
+ * along M, which changes no bit.  No counterpart in the reference. */
 size_t nmspmm_tail_workspace_bytes(int M, int N, int W, int kept);
 
 /* General entry point: C = A . B for one (window, kept, vec_len, Ns) geometry.
