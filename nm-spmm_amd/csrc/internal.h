@@ -40,7 +40,8 @@ __host__ __device__ inline void split_windows(int nwin, int split_k, int z, int*
 }
 
 // Modelled run time in seconds of the matrix-core kernel for waves of `blocks` 32-row blocks (4 or
-// 8) and `split` reduction slices, without the second pass of a split.  A workgroup covers
+// 8; 2 for the 64-row waves of ragged row counts) and `split` reduction slices, without the second
+// pass of a split.  A workgroup covers
 // 32*blocks rows x 128 columns; per window it needs kept/2 k-steps x blocks MFMAs x 64 cycles of
 // each of its CU's four matrix pipes (2.39 GHz; 256-row waves spend about 4 % less on loads).  A
 // CU holds four workgroups of 128-row waves or two of 256-row waves at once and they share its
@@ -88,10 +89,10 @@ inline double tall_tail_seconds(long long rest, double unit, int* pieces)
 }
 inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks, int split)
 {
-    const double per_window = kept * 53.5e-9 * (blocks == 8 ? tall_wave_cost(kept) : 1.0);
+    const double per_window = kept * 53.5e-9 * (blocks == 8 ? tall_wave_cost(kept) : blocks == 2 ? 0.5 * 1.25 : 1.0);
     const double unit = per_window * ((nwin + split - 1) / split);
     const long long groups = (long long)((M + 32 * blocks - 1) / (32 * blocks)) * ((N + 127) / 128) * split;
-    const int slots = blocks == 8 ? 2 : 4;
+    const int slots = blocks == 8 ? 2 : blocks == 2 ? 6 : 4;
     const long long full = groups / (256 * slots), rest = groups % (256 * slots);
     const long long busiest = (rest + 255) / 256;
     double t = (double)full * slots * unit;
@@ -107,6 +108,14 @@ inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks,
             t += slots * unit;
     }
     return t;
+}
+// 64-row waves (two 32-row blocks) cost about 25 % more loads per MFMA; the kernel uses them, in
+// place of 128-row ones on 128-wide column blocks, only where 128-row waves would multiply mostly
+// padding (192 rows: three 64-row waves instead of two 128-row ones, +24 % measured).
+inline bool short_waves_pay(int M)
+{
+    const int rows64 = (M + 63) / 64 * 64, rows128 = (M + 127) / 128 * 128;
+    return rows64 * 8 <= rows128 * 7;
 }
 // Wave height (32-row blocks) the matrix-core kernel uses for a shape: the faster one by the model.
 inline int choose_wave_blocks(int M, int N, int nwin, int kept, int split)
@@ -184,8 +193,10 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept)
 inline double model_tile_seconds(int M, int N, int nwin, int kept, int split)
 {
     const double c_bytes = (double)M * N * sizeof(float);
-    double t = 6e-6 + c_bytes / 8e12 +
-               model_kernel_seconds(M, N, nwin, kept, choose_wave_blocks(M, N, nwin, kept, split), split);
+    int blocks = choose_wave_blocks(M, N, nwin, kept, split);
+    if (blocks == 4 && short_waves_pay(M))
+        blocks = 2;  // as launch_mfma does (the column-block width is taken to be 128)
+    double t = 6e-6 + c_bytes / 8e12 + model_kernel_seconds(M, N, nwin, kept, blocks, split);
     if (split > 1)
         t += (2.0 * split + 1.0) * c_bytes / 8e12 + 2e-6;
     return t;

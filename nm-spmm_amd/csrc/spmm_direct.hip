@@ -446,10 +446,7 @@ static hipError_t launch_ns(const SpmmArgs& a)
 {
     const TailPlan plan = tail_plan_for(a, true);
     const bool tall = NMSPMM_RM_TALL == 8 && plan.blocks == 8;
-    // 64-row waves cost more loads per MFMA; they pay only where 128-row waves would multiply
-    // mostly padding (192 rows: three 64-row waves instead of two 128-row ones, +24 % measured)
-    const int rows64 = (a.M + 63) / 64 * 64, rows128 = (a.M + 127) / 128 * 128;
-    if (!tall && a.Ns == 128 && rows64 * 8 <= rows128 * 7)
+    if (!tall && a.Ns == 128 && short_waves_pay(a.M))
         return launch_cfg<KS, WS, 4, 1, 2, HIGH>(a, plan);
     switch (a.Ns) {
     case 128:
