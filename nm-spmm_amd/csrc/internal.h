@@ -39,17 +39,6 @@ __host__ __device__ inline void split_windows(int nwin, int split_k, int z, int*
     *count = z < q ? p + 1 : p;
 }
 
-// Modelled run time in seconds of the matrix-core kernel for waves of `blocks` 32-row blocks (4 or
-// 8; 2 for the 64-row waves of ragged row counts) and `split` reduction slices, without the second
-// pass of a split.  A workgroup covers
-// 32*blocks rows x 128 columns; per window it needs kept/2 k-steps x blocks MFMAs x 64 cycles of
-// each of its CU's four matrix pipes (2.39 GHz; 256-row waves spend about 4 % less on loads).  A
-// CU holds four workgroups of 128-row waves or two of 256-row waves at once and they share its
-// pipes, so the 256 CUs retire the workgroups in rounds of 1024 or 512.  After one full round the
-// leftovers spread over the CUs and cost as much as the busiest CU (a CU left with one workgroup,
-// one wave per SIMD, runs at about 0.9 of its rate); after two or more the leftovers land packed
-// on the CUs that happen to free up and cost a whole round, unless they are few enough to get a
-// launch of their own (plan_tail, unsplit reductions only).  Constants fitted to sweeps on one MI355X (mean error 6 %).
 // Pipe time of a 256-row wave relative to a 128-row one: twice the rows with half the B and index
 // loads per MFMA (4 % less), except at 8 kept rows per window (1:8), where the four 128-row waves
 // per SIMD hide the gather's cache misses better than two tall ones (measured 1 to 7 % in favour
@@ -87,6 +76,18 @@ inline double tall_tail_seconds(long long rest, double unit, int* pieces)
         *pieces = best_sub;
     return best;
 }
+// Modelled run time in seconds of the matrix-core kernel for waves of `blocks` 32-row blocks (4 or
+// 8; 2 for the 64-row waves of ragged row counts) and `split` reduction slices, without the second
+// pass of a split.  A workgroup covers 32*blocks rows x 128 columns; per window it needs kept/2
+// k-steps x blocks MFMAs x 64 cycles of each of its CU's four matrix pipes (2.39 GHz; taller and
+// shorter waves differ by a few per cent in the loads they issue, tall_wave_cost).  A CU holds
+// four workgroups of 128-row waves or two of 256-row waves at once and they share its pipes, so
+// the 256 CUs retire the workgroups in rounds of 1024 or 512.  After one full round the leftovers
+// of 128-row waves spread over the CUs and cost as much as the busiest CU (a CU left with one
+// workgroup, one wave per SIMD, runs at about 0.9 of its rate); after two or more they land packed
+// on the CUs that happen to free up and cost a whole round, unless they are few enough to get a
+// launch of their own (plan_tail, unsplit reductions only).  Leftovers of 256-row waves:
+// tall_tail_seconds.  Constants fitted to sweeps on one MI355X (mean error 6 %).
 inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks, int split)
 {
     const double per_window = kept * 53.5e-9 * (blocks == 8 ? tall_wave_cost(kept) : blocks == 2 ? 0.5 * 1.25 : 1.0);
