@@ -143,11 +143,14 @@ struct TailPlan {
     bool separate;   // without scratch: give the tail tiles a launch of their own (they then spread
                      // one or two per CU instead of landing packed on the CUs that free up last)
 };
-inline TailPlan plan_tail(int M, int N, int nwin, int kept)
+// `wr`: waves of a workgroup along M (1, 2 or 4 for column blocks of 128, 64 or 32): a tile is
+// 32 * blocks * wr rows x 128 / wr columns.
+inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1)
 {
     TailPlan t;
     t.blocks = choose_wave_blocks(M, N, nwin, kept, 1);
-    const long long tiles = (long long)((M + 32 * t.blocks - 1) / (32 * t.blocks)) * ((N + 127) / 128);
+    const int tile_rows = 32 * t.blocks * wr, tile_cols = 128 / wr;
+    const long long tiles = (long long)((M + tile_rows - 1) / tile_rows) * ((N + tile_cols - 1) / tile_cols);
     const long long slots = 256LL * (t.blocks == 8 ? 2 : 4);
     t.head = tiles;
     t.tail = 0;

@@ -372,8 +372,8 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     p.tail_slices = 1;
     p.tail_ws = nullptr;
     p.sub_tiles = 1;
-    // the plan counts 128-column tiles of RM blocks; it applies when that is this tile shape
-    const bool own_tail = plan.separate && WR == 1 && QS == 4 && RM == plan.blocks;
+    // the plan counts tiles of RM blocks per wave; it applies when that is this tile shape
+    const bool own_tail = plan.separate && RM == plan.blocks;
     const dim3 block(64 * QS * WR);
     dim3 grid(p.tiles_m * p.tiles_n, a.split_k, 1);
     if (!own_tail) {
@@ -418,8 +418,8 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
 // column-block width the indices were preprocessed for.  A wave is 256 or 128 rows tall, whichever
 // the run-time model expects to finish first: the taller wave halves the B and index loads per
 // MFMA, but only two such workgroups fit a CU, which quantises badly on mid-sized problems.
-// The tail split is planned for 128-wide column blocks and a single reduction slice, and used
-// when the caller's scratch holds it.
+// The tail handling is planned for a single reduction slice; its cut along K is used when the
+// caller's scratch holds it.
 static TailPlan tail_plan_for(const SpmmArgs& a, bool have_scratch)
 {
     TailPlan none;
@@ -429,9 +429,9 @@ static TailPlan tail_plan_for(const SpmmArgs& a, bool have_scratch)
     none.ws_bytes = 0;
     none.separate = false;
     none.sub = 1;
-    if (a.split_k != 1 || a.Ns != 128 || NMSPMM_RM_TALL != 8)
+    if (a.split_k != 1 || NMSPMM_RM_TALL != 8)
         return none;
-    TailPlan t = plan_tail(a.M, a.N, a.W / a.kept, a.kept);
+    TailPlan t = plan_tail(a.M, a.N, a.W / a.kept, a.kept, 128 / a.Ns);
     if (t.head + t.tail * t.slices * t.sub > 0x7fffffffLL)
         return none;
     if (have_scratch && t.slices > 1 && (a.tail_ws == nullptr || a.tail_ws_bytes < t.ws_bytes)) {

@@ -3,7 +3,7 @@ minutes: operands are drawn on the GPU, the reference is the dense product with 
 operand in fp64 (torch on the GPU - an independent formulation, not the checker's loop nest).  The
 shapes cross every launch plan: fewer tiles than the GPU holds, several rounds, ragged last rounds
 (leftover tiles in a launch of their own, whole or in pieces), ragged row counts, reduction splits,
-both storage orders of A.  Same tolerance as everywhere (1e-4, scaled max error)."""
+both storage orders of A, all three widths of the column blocks.  Same tolerance as everywhere (1e-4, scaled max error)."""
 import random
 
 import pytest
@@ -24,15 +24,15 @@ def draw_case(rng):
     while M * N * K > 3.5e10:  # keeps the fp64 reference to a fraction of a second
         N = 128 * max(4, N // 256)
     split_k = min(rng.choice([1, 1, 1, 2, 3, 4]), K // 64)
-    return M, N, K, n, m, split_k, rng.random() < 0.3
+    return M, N, K, n, m, split_k, rng.random() < 0.3, rng.choice([128, 128, 64, 32])
 
 
 CASES = [draw_case(random.Random(9000 + i)) for i in range(60)]
 
 
-@pytest.mark.parametrize("case", CASES, ids=lambda c: "M%d-N%d-K%d-%dof%d-s%d-%s" % (c[:6] + ("rm" if c[6] else "cm",)))
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "M%d-N%d-K%d-%dof%d-s%d-%s-Ns%d" % (c[:6] + ("rm" if c[6] else "cm", c[7])))
 def test_random_large_shape(case):
-    M, N, K, n, m, split_k, row_major = case
+    M, N, K, n, m, split_k, row_major, Ns = case
     window, kept = GEOMETRY[(n, m)]
     g = torch.Generator(device="cuda").manual_seed(M * 7 + N + K)
     W, Q = K // m * n, N // 32
@@ -50,16 +50,16 @@ def test_random_large_shape(case):
     D = torch.empty_like(DT)
     cinfo = None
     if window == 64:
-        cinfo = torch.empty(nmspmm.column_info_ints(W, kept, window, N, 128), dtype=torch.int32, device="cuda")
-    assert nmspmm.preprocess_device(DT, n, m, W, Q, N, 128, D, cinfo) == (window, kept)
+        cinfo = torch.empty(nmspmm.column_info_ints(W, kept, window, N, Ns), dtype=torch.int32, device="cuda")
+    assert nmspmm.preprocess_device(DT, n, m, W, Q, N, Ns, D, cinfo) == (window, kept)
     C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
     if row_major or M % 4 != 0:  # (a column-major A with such a row count would take the generic kernel)
         ws = torch.empty(nmspmm.workspace_bytes_rowmajor(M, N, K, split_k) // 4, dtype=torch.float32, device="cuda")
-        nmspmm.spmm_rowmajor(X, BT, D, cinfo, C, M, N, K, W, window, kept, ws, 32, 128, split_k)
+        nmspmm.spmm_rowmajor(X, BT, D, cinfo, C, M, N, K, W, window, kept, ws, 32, Ns, split_k)
     else:
         A = X.t().contiguous()                                                      # K x M: column-major M x K
         ws = torch.empty(max(nmspmm.workspace_bytes(M, N, split_k) // 4, 4), dtype=torch.float32, device="cuda")
-        nmspmm.spmm(A, BT, D, cinfo, C, M, N, K, W, window, kept, 32, 128, split_k, ws if split_k > 1 else None)
+        nmspmm.spmm(A, BT, D, cinfo, C, M, N, K, W, window, kept, 32, Ns, split_k, ws if split_k > 1 else None)
     torch.cuda.synchronize()
     assert nmspmm.last_kernel() == "mfma"
     assert torch.isfinite(C).all().item()

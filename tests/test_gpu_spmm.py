@@ -244,18 +244,19 @@ def test_ragged_last_round_is_split_along_k_through_scratch(oracle, M, N, K, n, 
 
 @pytest.mark.parametrize("M,N,K,n,m", [(4096, 8448, 256, 2, 4), (8192, 4224, 512, 1, 8), (2048, 11008, 256, 2, 4),
                                        (4096, 11008, 4096, 1, 8), (1024, 24576, 4096, 2, 8), (2000, 11008, 256, 2, 4)])
-def test_leftover_tiles_in_a_launch_of_their_own(oracle, M, N, K, n, m):
+@pytest.mark.parametrize("Ns", [128, 64, 32])
+def test_leftover_tiles_in_a_launch_of_their_own(oracle, M, N, K, n, m, Ns):
     """More tiles than the GPU holds at once, a ragged last round and too few windows to cut its
     tiles along K: the leftovers run as a second launch, whole (the first two shapes) or as two or
     four shorter pieces along M each (688 tiles of 256 rows on 512 slots: 176 leftovers in four
     pieces; 1376: 352 in two; 768: 256 in two; the last shape with a ragged row count as well).
-    Every tile must still be computed exactly once."""
+    Every tile must still be computed exactly once, for every width of the column blocks (the
+    workgroup is then 1 x 4, 2 x 2 or 4 x 1 waves and the tile 128, 64 or 32 columns wide)."""
     d = datagen.init_data(M, N, K, n, m, seed=M + K)
-    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
-    assert nmspmm.tail_workspace_bytes(M, N, d["W"], kept) == 0
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, Ns)
     C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
     nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), None if cinfo is None else dev(cinfo), C, M, N, K, d["W"], window,
-                kept, 32, 128, 1, None)
+                kept, 32, Ns, 1, None)
     torch.cuda.synchronize()
     assert nmspmm.last_kernel() == "mfma" and bool(torch.isfinite(C).all())
     # column sums of C against column sums computed from the operands in fp64: touches every tile
