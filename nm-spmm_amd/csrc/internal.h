@@ -59,12 +59,12 @@ inline double tall_wave_cost(int kept) { return kept <= 8 ? 2.0 / 0.98 : 2.0 / 1
 // of the cheapest way and its piece count (0: leave the tiles in the launch).  Over 96 ragged
 // LLM-layer shapes this choice is 4.1 % faster on average than leaving the tiles in the launch
 // (best choice per shape: 4.3 %), up to 30 % on single shapes.
-inline double tall_tail_seconds(long long rest, double unit, int* pieces)
+inline double tall_tail_seconds(long long rest, double unit, int* pieces, int max_pieces = 4)
 {
     static const double piece_cost[3] = {1.0, 1.04, 1.2};
     double best = 2.0 * unit;
     int best_sub = 0;
-    for (int i = 0, sub = 1; i < 3; ++i, sub *= 2) {
+    for (int i = 0, sub = 1; i < 3 && sub <= max_pieces; ++i, sub *= 2) {
         const long long busiest = (rest * sub + 255) / 256;
         const double s = busiest * unit / sub * piece_cost[i] / (busiest == 1 ? 0.9 : 1.0) + 12e-6;
         if (s < best) {
@@ -144,8 +144,9 @@ struct TailPlan {
                      // one or two per CU instead of landing packed on the CUs that free up last)
 };
 // `wr`: waves of a workgroup along M (1, 2 or 4 for column blocks of 128, 64 or 32): a tile is
-// 32 * blocks * wr rows x 128 / wr columns.
-inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1)
+// 32 * blocks * wr rows x 128 / wr columns.  `max_pieces`: the shortest waves the kernel has,
+// as pieces of a 256-row wave.
+inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_pieces = 4)
 {
     TailPlan t;
     t.blocks = choose_wave_blocks(M, N, nwin, kept, 1);
@@ -163,7 +164,7 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1)
         return t;
     if (t.blocks == 8) {
         int pieces = 0;
-        tall_tail_seconds(rest, kept * 53.5e-9 * tall_wave_cost(kept) * nwin, &pieces);
+        tall_tail_seconds(rest, kept * 53.5e-9 * tall_wave_cost(kept) * nwin, &pieces, max_pieces);
         if (pieces == 0)
             return t;
         t.separate = true;

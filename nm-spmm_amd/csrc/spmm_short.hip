@@ -29,6 +29,9 @@ struct ShortParams {
     int nchunk;          // chunks of 16 dense rows in the whole reduction
     int split_k;
     int tiles_m, tiles_n;
+    int tile_offset;     // first tile of this launch (tiles are numbered column block by column block)
+    int sub_tiles;       // > 1: every workgroup of this launch is one of sub_tiles pieces, along M, of a
+                         // tile of sub_tiles * 32 * RM rows (tiles_m counts those taller tiles)
 };
 
 struct sfloat8 { float4 lo, hi; };
@@ -61,8 +64,9 @@ spmm_short_kernel(const ShortParams p)
     constexpr int KSTEPS = kChunk / 2;
     constexpr int RAW = WPC * NK;       // kept rows per chunk
 
-    const int tile_m = blockIdx.x % p.tiles_m;
-    const int tile_n = blockIdx.x / p.tiles_m;
+    const int tile = p.tile_offset + blockIdx.x / p.sub_tiles;
+    const int tile_m = (tile % p.tiles_m) * p.sub_tiles + blockIdx.x % p.sub_tiles;
+    const int tile_n = tile / p.tiles_m;
     int c_begin, c_count;
     split_windows(p.nchunk, p.split_k, blockIdx.y, &c_begin, &c_count);
     const int c_last = c_begin + c_count - 1;
@@ -198,10 +202,36 @@ static hipError_t launch_short_cfg(const SpmmArgs& a)
     p.nchunk = a.K / kChunk;
     p.split_k = a.split_k;
     p.tiles_n = a.N / 128;
-    const bool tall = choose_wave_blocks(a.M, a.N, p.nchunk, kChunk, a.split_k) == 8;
+    p.tile_offset = 0;
+    p.sub_tiles = 1;
+    // wave height and leftover tiles as in the long-vector kernel: a chunk of 16 dense rows costs
+    // what a window of 16 kept rows costs there
+    TailPlan plan = plan_tail(a.M, a.N, p.nchunk, kChunk, 1, 2);
+    if (a.split_k != 1) {
+        plan.blocks = choose_wave_blocks(a.M, a.N, p.nchunk, kChunk, a.split_k);
+        plan.separate = false;
+    }
+    const bool tall = plan.blocks == 8;
     p.tiles_m = (a.M + (tall ? 255 : 127)) / (tall ? 256 : 128);
-    const dim3 grid(p.tiles_m * p.tiles_n, a.split_k), block(256);
+    const dim3 block(256);
+    dim3 grid(p.tiles_m * p.tiles_n, a.split_k);
+    if (plan.separate && plan.head + plan.tail == (long long)p.tiles_m * p.tiles_n)
+        grid.x = (unsigned)plan.head;
+    else
+        plan.separate = false;
     if (tall)
+        spmm_short_kernel<MWIN, NK, 8><<<grid, block, 0, a.stream>>>(p);
+    else
+        spmm_short_kernel<MWIN, NK, 4><<<grid, block, 0, a.stream>>>(p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || !plan.separate)
+        return e;
+    // the leftover tiles of a ragged last round in a launch of their own, whole or as two
+    // 128-row pieces each (internal.h: plan_tail)
+    p.tile_offset = (int)plan.head;
+    p.sub_tiles = tall ? plan.sub : 1;
+    grid.x = (unsigned)(plan.tail * p.sub_tiles);
+    if (tall && p.sub_tiles == 1)
         spmm_short_kernel<MWIN, NK, 8><<<grid, block, 0, a.stream>>>(p);
     else
         spmm_short_kernel<MWIN, NK, 4><<<grid, block, 0, a.stream>>>(p);

@@ -384,3 +384,29 @@ def test_row_counts_either_side_of_the_tile_kernels_limit(oracle, M, family):
                            d["W"]).reshape(len(rows), N)
     assert np.isfinite(got).all() and scaled_max_error(got, want) <= REL_TOL
     assert not torch.isnan(C).any().item()
+
+
+@pytest.mark.parametrize("M,N,K,vl,n,m", [(2048, 11008, 256, 4, 2, 4), (4096, 5120, 512, 8, 1, 8), (1000, 24576, 256, 16, 3, 8)])
+def test_short_vector_kernel_with_leftover_tiles(oracle, M, N, K, vl, n, m):
+    """The short-vector kernel on more tiles than the GPU holds at once with a ragged last round:
+    the leftovers run as a second launch, whole or as two 128-row pieces each.  Column sums in fp64
+    touch every tile; sampled rows against the checker."""
+    d = datagen.init_data(M, N, K, n, m, vec_len=vl, seed=M + vl)
+    W, Q = d["W"], d["Q"]
+    D = d["DT"].reshape(-1).copy()
+    oracle.preprocess_low(D, W, Q, 128, vl)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), None, C, M, N, K, W, m, n, vl, 128)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == "short" and bool(torch.isfinite(C).all())
+    dense = torch.zeros((K, N), dtype=torch.float64, device="cuda")
+    rows = (torch.arange(W, device="cuda") // n * m)[:, None] + dev(d["DT"]).long()
+    dense[rows.repeat_interleave(vl, dim=1), torch.arange(N, device="cuda")[None, :].expand(W, -1)] = dev(d["BT"]).double()
+    want = dev(d["A_km"]).double().sum(dim=1) @ dense
+    got = C.double().sum(dim=0)
+    assert float(((got - want).abs() / want.abs().clamp_min(want.pow(2).mean().sqrt())).max()) <= REL_TOL
+    rows_s = np.array([0, 1, 127, 128, 255, 256, M // 2, M - 129, M - 2, M - 1])
+    A_rows = np.ascontiguousarray(d["A_km"][:, rows_s])
+    ref = oracle.gemm_cpu(A_rows.reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), len(rows_s), N, W,
+                          vl).reshape(len(rows_s), N)
+    assert scaled_max_error(C[torch.from_numpy(rows_s).cuda()].cpu().numpy(), ref) <= REL_TOL
