@@ -103,7 +103,7 @@ spmm_skinny_kernel(const SkinnyParams p)
     const int vec_g = blockIdx.x;     // global column vector
     const int jb = vec_g / QS;        // preprocessed column block
     const int vec = vec_g % QS;       // vector inside it
-    const int M = p.M, N = p.N, lda = p.lda;
+    const int M = p.M, N = p.N;
 
     // windows of this wave: the same partition rule the large-tile kernels use for split-K
     int w_begin, w_count;
@@ -267,7 +267,7 @@ spmm_skinny16_kernel(const SkinnyParams p)
     const int vec_g = blockIdx.x;
     const int jb = vec_g / QS;
     const int vec = vec_g % QS;
-    const int M = p.M, N = p.N, lda = p.lda;
+    const int M = p.M, N = p.N;
 
     int w_begin, w_count;
     split_windows(p.nwin, kSkinnyWaves, wave, &w_begin, &w_count);
