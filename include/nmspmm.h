@@ -128,7 +128,8 @@ int nmspmm_decompress_device(const float* dBT, const int32_t* dDT, int K, int N,
  * split_k partial M x N fp32 results that a second pass sums in a fixed order. */
 size_t nmspmm_workspace_bytes(int M, int N, int split_k);
 
-/* Bytes of optional scratch with which nmspmm_spmm, called with split_k == 1 and Ns == 128, cuts
+/* Bytes of optional scratch with which nmspmm_spmm, called with split_k == 1 (sized for Ns == 128;
+ * with other widths the scratch is used when it suffices), cuts
  * the few leftover tiles of a ragged last round into four pieces along K so that they occupy four
  * times as many CUs (0 when there is nothing to gain).  The pieces are summed in a fixed order,
  * but not in the order of an unsplit reduction: with the scratch the affected tiles of C may
