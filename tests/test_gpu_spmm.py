@@ -216,11 +216,12 @@ def test_auto_entry_point_chooses_the_split_itself(oracle, M, N, K, n, m, sparsi
 
 
 @pytest.mark.parametrize("M,N,K,n,m", [(8192, 4224, 1024, 2, 4), (4096, 8448, 1024, 1, 8), (8192, 4224, 2048, 2, 8)])
-def test_ragged_last_round_is_split_along_k_through_scratch(oracle, M, N, K, n, m):
+@pytest.mark.parametrize("Ns", [128, 64, 32])
+def test_ragged_last_round_is_split_along_k_through_scratch(oracle, M, N, K, n, m, Ns):
     """More tiles than the GPU holds at once and a ragged last round: with scratch the tiles of that
     round are cut along K and summed by a second kernel; the result matches the checker either way."""
     d = datagen.init_data(M, N, K, n, m, seed=M + N)
-    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, Ns)
     need = nmspmm.tail_workspace_bytes(M, N, d["W"], kept)
     assert need > 0
     A, B, Dd = dev(d["A_km"]), dev(d["BT"]), dev(D)
@@ -229,7 +230,7 @@ def test_ragged_last_round_is_split_along_k_through_scratch(oracle, M, N, K, n, 
     outs = []
     for scratch in (ws, None, ws[: need // 4 - 64]):       # enough, none, too little (ignored)
         C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
-        nmspmm.spmm(A, B, Dd, ci, C, M, N, K, d["W"], window, kept, 32, 128, 1, scratch)
+        nmspmm.spmm(A, B, Dd, ci, C, M, N, K, d["W"], window, kept, 32, Ns, 1, scratch)
         torch.cuda.synchronize()
         assert nmspmm.last_kernel() == "mfma" and bool(torch.isfinite(C).all())
         outs.append(C)
