@@ -47,9 +47,11 @@ struct DirectParams {
     int nwin;            // windows in the whole reduction
     int split_k;
     int tiles_m, tiles_n;
-    int tile_offset;     // first logical tile of this launch (the tail tiles get a launch of their own)
+    int tile_offset;     // first logical tile of this launch (the tail tiles may get a launch of their own)
     int tail_slices;     // > 1: every workgroup of this launch is one of tail_slices pieces of a tile along K
     float* tail_ws;      // [tile of this launch][slice][MS][NS] partial tiles
+    int head_units;      // workgroups of this launch that compute whole tiles (the first ones)
+    int tail_offset;     // first logical tile computed in pieces along M by the workgroups after them
     int sub_tiles;       // > 1: every workgroup of this launch is one of sub_tiles pieces, along M, of a
                          // tile of sub_tiles * MS rows (the tile walk and tiles_m are those taller tiles')
 };
@@ -104,8 +106,8 @@ __device__ inline float buffer_load_f1(__amdgpu_buffer_rsrc_t r, uint32_t byte_o
 // block (Ns = 32*QS), WR: waves along M, RM: 32-row blocks per wave (2, 4 or 8), HIGH:
 // high-sparsity layout (D holds ranks into the window's column_info list).
 template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
-__global__ void __launch_bounds__(64 * QS * WR, RM == 8 ? 2 : (HIGH && WS == 16) ? 4 : NMSPMM_OCC)
-spmm_direct_kernel(const DirectParams p)
+__device__ __forceinline__ void direct_unit(const DirectParams& p, const int logical, const int sub, const int sub_tiles,
+                                            const bool tail_unit, const int unit)
 {
     static_assert(RM == 2 || RM == 4 || RM == 8, "64-, 128- or 256-row waves");
     constexpr int IL = RM < 4 ? RM : 4;  // rows interleaved per lane: block b holds rows IL*r + b%IL (+128 for b >= 4)
@@ -120,24 +122,8 @@ spmm_direct_kernel(const DirectParams p)
     constexpr int ND = (WS * QS + 63) / 64;   // wave-wide loads per window of indices
     static_assert(WS % CH == 0, "whole chunks");
 
-    // ---- tile walk: consecutive ids go to different XCDs, so give each XCD a contiguous run of
-    // logical tiles, walked in bands of GROUP row tiles across all column blocks.  In a launch of
-    // tail slices, consecutive ids are the pieces of one tile.
-    const bool tail_unit = p.tail_slices > 1;
-    const int unit = blockIdx.x;  // slice number among the slices of this launch
-    int logical, sub = 0;
-    if (p.sub_tiles > 1) {
-        logical = p.tile_offset + unit / p.sub_tiles;
-        sub = unit % p.sub_tiles;
-    } else if (!tail_unit) {
-        const int total = gridDim.x;
-        const int id = blockIdx.x;
-        const int q = total / kXcds, r = total % kXcds;
-        const int xcd = id % kXcds, loc = id / kXcds;
-        logical = p.tile_offset + (xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc);
-    } else {
-        logical = p.tile_offset + unit / p.tail_slices;
-    }
+    // logical tile -> (tile_m, tile_n): bands of GROUP row tiles across all column blocks; with
+    // sub_tiles > 1 the walk and tiles_m are those of tiles sub_tiles times as tall as MS
     constexpr int GROUP = NMSPMM_GROUP;
     int tile_m, tile_n;
     {
@@ -162,7 +148,7 @@ spmm_direct_kernel(const DirectParams p)
     const int h = lane >> 5;
     const int j = lane & 31;
     const int M = p.M, N = p.N, lda = p.lda;
-    const int bi = (tile_m * p.sub_tiles + sub) * MS + wr * MW;  // first row of this wave (may be >= M: loads nothing)
+    const int bi = (tile_m * sub_tiles + sub) * MS + wr * MW;  // first row of this wave (may be >= M: loads nothing)
     const int bj = tile_n * NS + vec * 32;
 
     const float* const Ablk = p.A + min(bi, lda);
@@ -314,6 +300,53 @@ spmm_direct_kernel(const DirectParams p)
     }
 }
 
+// Workgroup `id` of a launch whose workgroups all compute the same kind of unit.  Whole tiles: a
+// walk that gives each XCD (consecutive ids go to different XCDs) a contiguous run of the
+// p.head_units logical tiles.  In a launch of K slices (p.tail_slices > 1) consecutive ids are the
+// slices of one tile, in a launch of pieces along M (p.sub_tiles > 1) the pieces of one tile.
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+__device__ __forceinline__ void direct_uniform_launch(const DirectParams& p, const int id)
+{
+    const bool tail_unit = p.tail_slices > 1;
+    int logical, sub = 0;
+    if (p.sub_tiles > 1) {
+        logical = p.tile_offset + id / p.sub_tiles;
+        sub = id % p.sub_tiles;
+    } else if (tail_unit) {
+        logical = p.tile_offset + id / p.tail_slices;
+    } else {
+        const int total = p.head_units;
+        const int q = total / kXcds, r = total % kXcds;
+        const int xcd = id % kXcds, loc = id / kXcds;
+        logical = p.tile_offset + (xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc);
+    }
+    direct_unit<KS, WS, QS, WR, RM, HIGH>(p, logical, sub, p.sub_tiles, tail_unit, id);
+}
+
+#define NMSPMM_DIRECT_BOUNDS __launch_bounds__(64 * QS * WR, RM == 8 ? 2 : (HIGH && WS == 16) ? 4 : NMSPMM_OCC)
+
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+__global__ void NMSPMM_DIRECT_BOUNDS spmm_direct_kernel(const DirectParams p)
+{
+    direct_uniform_launch<KS, WS, QS, WR, RM, HIGH>(p, blockIdx.x);
+}
+
+// The first p.head_units workgroups compute whole tiles; the ones after them are the pieces, two
+// per tile along M, of the tiles from p.tail_offset on, computed on waves of RM / 2 blocks.  They
+// are dispatched last and fill the CUs that run out of whole tiles, in pieces fine enough to even
+// out the end of the launch (same sums in the same order as whole tiles, no scratch).
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+__global__ void NMSPMM_DIRECT_BOUNDS spmm_direct_mixed_kernel(const DirectParams p)
+{
+    const int id = blockIdx.x;
+    if (id >= p.head_units) {
+        const int u = id - p.head_units;
+        direct_unit<KS, WS, QS, WR, RM / 2, HIGH>(p, p.tail_offset + u / 2, u % 2, 2, false, u);
+        return;
+    }
+    direct_uniform_launch<KS, WS, QS, WR, RM, HIGH>(p, id);
+}
+
 // Sums the slices of the tail tiles in slice order into C (second pass of the tail split).  One
 // workgroup per tail tile; the tile is found by the same walk as in the main kernel.
 template <int MS, int NS>
@@ -371,16 +404,28 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     p.tile_offset = 0;
     p.tail_slices = 1;
     p.tail_ws = nullptr;
+    p.tail_offset = 0;
     p.sub_tiles = 1;
     // the plan counts tiles of RM blocks per wave; it applies when that is this tile shape
     const bool own_tail = plan.separate && RM == plan.blocks;
     const dim3 block(64 * QS * WR);
     dim3 grid(p.tiles_m * p.tiles_n, a.split_k, 1);
+    p.head_units = (int)grid.x;
     if (!own_tail) {
         spmm_direct_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, a.stream>>>(p);
         return hipGetLastError();
     }
-    // head tiles, then the leftover tiles in a launch of their own, whole or in slices
+    p.head_units = (int)plan.head;
+    if (plan.slices == 1 && plan.sub > 1 && plan.fused) {
+        // shorter waves for the leftovers, in the same launch: each leftover tile in two pieces
+        // along M, so that the pieces fill the CUs more evenly than whole tiles would
+        p.tail_offset = (int)plan.head;
+        grid.x = (unsigned)(plan.head + plan.tail * plan.sub);
+        if constexpr (RM == 4)
+            spmm_direct_mixed_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, a.stream>>>(p);
+        return hipGetLastError();
+    }
+    // head tiles, then the leftover tiles in a launch of their own, whole or in slices along K
     grid.x = (unsigned)plan.head;
     spmm_direct_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, a.stream>>>(p);
     hipError_t e = hipGetLastError();
@@ -388,10 +433,12 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
         return e;
     p.tile_offset = (int)plan.head;
     if (plan.slices == 1 && plan.sub > 1) {
-        // shorter waves for the leftovers: each tile in plan.sub pieces along M, so that the pieces
-        // fill the CUs more evenly than whole tiles would; same sums in the same order, no scratch
+        // shorter waves for the leftovers, in a launch of the kernel built for such waves (which
+        // more workgroups per CU can run): each tile in plan.sub pieces along M; same sums in the
+        // same order as whole tiles, no scratch
         p.sub_tiles = plan.sub;
         grid.x = (unsigned)(plan.tail * plan.sub);
+        p.head_units = (int)grid.x;
         if (RM / plan.sub == 4) {
             if constexpr (RM >= 8)
                 spmm_direct_kernel<KS, WS, QS, WR, 4, HIGH><<<grid, block, 0, a.stream>>>(p);
@@ -404,6 +451,7 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     p.tail_slices = plan.slices;
     p.tail_ws = plan.slices > 1 ? a.tail_ws : nullptr;
     grid.x = (unsigned)(plan.tail * plan.slices);
+    p.head_units = (int)grid.x;
     spmm_direct_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, a.stream>>>(p);
     e = hipGetLastError();
     if (e == hipSuccess && plan.slices > 1) {
@@ -429,6 +477,7 @@ static TailPlan tail_plan_for(const SpmmArgs& a, bool have_scratch)
     none.ws_bytes = 0;
     none.separate = false;
     none.sub = 1;
+    none.fused = false;
     if (a.split_k != 1 || NMSPMM_RM_TALL != 8)
         return none;
     TailPlan t = plan_tail(a.M, a.N, a.W / a.kept, a.kept, 128 / a.Ns);

@@ -243,16 +243,10 @@ def test_ragged_last_round_is_split_along_k_through_scratch(oracle, M, N, K, n, 
             assert scaled_max_error(C[r0:r1].cpu().numpy(), want) <= REL_TOL
 
 
-@pytest.mark.parametrize("M,N,K,n,m", [(4096, 8448, 256, 2, 4), (8192, 4224, 512, 1, 8), (2048, 11008, 256, 2, 4),
-                                       (4096, 11008, 4096, 1, 8), (1024, 24576, 4096, 2, 8), (2000, 11008, 256, 2, 4)])
-@pytest.mark.parametrize("Ns", [128, 64, 32])
-def test_leftover_tiles_in_a_launch_of_their_own(oracle, M, N, K, n, m, Ns):
-    """More tiles than the GPU holds at once, a ragged last round and too few windows to cut its
-    tiles along K: the leftovers run as a second launch, whole (the first two shapes) or as two or
-    four shorter pieces along M each (688 tiles of 256 rows on 512 slots: 176 leftovers in four
-    pieces; 1376: 352 in two; 768: 256 in two; the last shape with a ragged row count as well).
-    Every tile must still be computed exactly once, for every width of the column blocks (the
-    workgroup is then 1 x 4, 2 x 2 or 4 x 1 waves and the tile 128, 64 or 32 columns wide)."""
+def check_every_tile_once(oracle, M, N, K, n, m, Ns):
+    """Unsplit multiplication on the tile kernel; column sums of C against column sums computed
+    from the operands in fp64 (touches every tile), and the first and last rows against the
+    checker."""
     d = datagen.init_data(M, N, K, n, m, seed=M + K)
     window, kept, D, cinfo = preprocess_with_oracle(oracle, d, Ns)
     C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
@@ -271,6 +265,32 @@ def test_leftover_tiles_in_a_launch_of_their_own(oracle, M, N, K, n, m, Ns):
         ref = oracle.gemm_cpu(d["A_km"].reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), M, N, d["W"],
                               rows=(r0, r1)).reshape(M, N)[r0:r1]
         assert scaled_max_error(C[r0:r1].cpu().numpy(), ref) <= REL_TOL
+
+
+@pytest.mark.parametrize("M,N,K,n,m", [(4096, 8448, 256, 2, 4), (8192, 4224, 512, 1, 8), (2048, 11008, 256, 2, 4),
+                                       (4096, 11008, 4096, 1, 8), (1024, 24576, 4096, 2, 8), (2000, 11008, 256, 2, 4)])
+@pytest.mark.parametrize("Ns", [128, 64, 32])
+def test_leftover_tiles_in_a_launch_of_their_own(oracle, M, N, K, n, m, Ns):
+    """More tiles than the GPU holds at once, a ragged last round and too few windows to cut its
+    tiles along K: the leftovers run as a second launch, whole (the first two shapes) or as two or
+    four shorter pieces along M each (688 tiles of 256 rows on 512 slots: 176 leftovers in four
+    pieces; 1376: 352 in two; 768: 256 in two; the last shape with a ragged row count as well).
+    Every tile must still be computed exactly once, for every width of the column blocks (the
+    workgroup is then 1 x 4, 2 x 2 or 4 x 1 waves and the tile 128, 64 or 32 columns wide)."""
+    check_every_tile_once(oracle, M, N, K, n, m, Ns)
+
+
+@pytest.mark.parametrize("M,N,K,n,m", [(1024, 5120, 256, 2, 4), (2048, 5120, 512, 1, 8), (300, 2048, 256, 2, 8),
+                                       (2048, 6656, 512, 1, 8), (1000, 6656, 256, 3, 8), (1024, 5120, 128, 32, 32)])
+@pytest.mark.parametrize("Ns", [128, 64, 32])
+def test_last_layer_of_a_small_launch_in_pieces(oracle, M, N, K, n, m, Ns):
+    """Fewer tiles than the GPU holds at once: the tiles beyond the last multiple of 256 are
+    computed as two 64-row pieces each by the workgroups at the end of the same launch when they
+    cover at most half of the CUs (320 tiles of 128 rows: 64 in pieces; 640: 128; 48 with a ragged
+    row count: all of them, and the pieces beyond the last row store nothing; 832: 64 after three
+    whole layers) and whole otherwise (416: 160 leftovers).  Every tile exactly once, for every
+    width of the column blocks."""
+    check_every_tile_once(oracle, M, N, K, n, m, Ns)
 
 
 def test_llm_layer_shape_2of8(oracle):
