@@ -40,13 +40,11 @@ __host__ __device__ inline void split_windows(int nwin, int split_k, int z, int*
 }
 
 // Pipe time of a 256-row wave relative to a 128-row one: twice the rows with half the B and index
-// loads per MFMA (4 % less), except at 8 kept rows per window (1:8), where the four 128-row waves
-// per SIMD hide the gather's cache misses better than two tall ones (measured 1 to 7 % in favour
-// of the shorter waves on shapes of up to three rounds, 4 % at 4096 cubed; from five rounds on the
-// tall waves are 1 % ahead again, which this leaves on the table).  A finer table per layout
-// (2:8 is level at 4096 cubed) was tried and chose worse on large shapes, where the tall waves'
-// smaller traffic counts for more than one exact round shows.
-inline double tall_wave_cost(int kept) { return kept <= 8 ? 2.0 / 0.98 : 2.0 / 1.04; }
+// loads per MFMA.  Measured on eleven shapes from 2048 x 4096 x 4096 to 8192 cubed with every CU
+// busy: 3 to 12 % less at 2:4, 2 to 7 % at 2:8, 1 to 7 % at 1:8, growing with the size of the
+// problem (the tall waves' smaller traffic counts for more the longer the run); one figure per
+// layout is used.
+inline double tall_wave_cost(int kept) { return kept <= 8 ? 2.0 / 1.03 : 2.0 / 1.05; }
 
 // Leftover tiles of 256-row waves (two workgroups per CU) after at least one full round: `rest`
 // tiles, each `unit` seconds of a CU's pipes.  Left in the launch they land packed on the CUs that
@@ -82,12 +80,12 @@ inline double tall_tail_seconds(long long rest, double unit, int* pieces, int ma
 // k-steps x blocks MFMAs x 64 cycles of each of its CU's four matrix pipes (2.39 GHz; taller and
 // shorter waves differ by a few per cent in the loads they issue, tall_wave_cost).  A CU holds
 // four workgroups of 128-row waves or two of 256-row waves at once and they share its pipes, so
-// the 256 CUs retire the workgroups in rounds of 1024 or 512.  After one full round the leftovers
-// of 128-row waves spread over the CUs and cost as much as the busiest CU (a CU left with one
-// workgroup, one wave per SIMD, runs at about 0.9 of its rate); after two or more they land packed
-// on the CUs that happen to free up and cost a whole round, unless they are few enough to get a
-// launch of their own (plan_tail, unsplit reductions only).  Leftovers of 256-row waves:
-// tall_tail_seconds.  Constants fitted to sweeps on one MI355X (mean error 6 %).
+// the 256 CUs retire the workgroups in rounds of 1024 or 512.  Fewer workgroups than that spread
+// over the CUs and cost as much as the busiest CU (a CU left with one workgroup, one wave per
+// SIMD, runs at about 0.9 of its rate).  After full rounds the leftovers land packed on the CUs
+// that happen to free up first and cost a whole round, unless plan_tail (unsplit reductions only)
+// gives them a launch of shorter pieces: tall_tail_seconds for 256-row waves, the piece costs
+// below for 128-row ones.  Constants fitted to sweeps on one MI355X (mean error 6 %).
 inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks, int split)
 {
     const double per_window = kept * 53.5e-9 * (blocks == 8 ? tall_wave_cost(kept) : blocks == 2 ? 0.5 * 1.25 : 1.0);
@@ -96,20 +94,28 @@ inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks,
     const int slots = blocks == 8 ? 2 : blocks == 2 ? 6 : 4;
     const long long full = groups / (256 * slots), rest = groups % (256 * slots);
     const long long busiest = (rest + 255) / 256;
-    if (blocks == 4 && split == 1 && full == 0) {
-        // fewer tiles than the CUs hold at once: a last layer on at most half of the CUs runs as
-        // two 64-row pieces per tile (plan_tail).  Next to whole tiles a piece costs 0.55 of a
-        // tile; alone on its CU (one 64-row wave per SIMD) it hides little latency and costs 0.85
-        // of a tile, and as much as a tile on the 1:8 geometry
+    if (blocks == 4 && split == 1) {
+        // plan_tail computes the last tiles of such a launch as two 64-row pieces each.  Next to
+        // whole tiles a piece costs 0.55 of a tile; alone on its CU (one 64-row wave per SIMD) it
+        // hides less latency: 0.65 of a tile, 0.85 on the 1:8 geometry
+        const double lone = kept <= 8 ? 0.85 : 0.65;
         const long long whole = rest / 256, layer = rest % 256;
-        if (layer > 0 && layer <= 128)
-            return whole == 0 ? (kept <= 8 ? 1.03 : 0.85) * unit : (whole + 0.55) * unit;
+        if (full == 0 && layer > 0 && layer <= 128)
+            return whole == 0 ? lone * unit : (whole + 0.55) * unit;
+        if (full >= 1 && rest > 0 && rest <= 128 * slots) {
+            const long long busiest_piece = (2 * rest + 255) / 256;
+            return (double)full * slots * unit + (busiest_piece == 1 ? lone : 0.55 * busiest_piece) * unit + 10e-6;
+        }
     }
     double t = (double)full * slots * unit;
     if (busiest > 0 && blocks == 8 && split == 1 && full >= 1) {
         t += tall_tail_seconds(rest, unit, nullptr);  // plan_tail gives these leftovers a launch of shorter pieces
     } else if (busiest > 0) {
-        const double spread = busiest * unit / (busiest == 1 ? 0.9 : 1.0);
+        // one workgroup per CU: a 128-row wave alone on its SIMD runs at 0.9 of the rate; a 256-row
+        // wave with 16 or more kept rows per chunk keeps its pipe busy by itself (measured 3 to 5 %
+        // ahead of two 128-row workgroups per CU at 2:4 and 2:8, behind at 1:8 and 3:8)
+        const double lone_rate = blocks == 8 && kept >= 16 ? 1.0 : 0.9;
+        const double spread = busiest * unit / (busiest == 1 ? lone_rate : 1.0);
         if (full < 2)
             t += spread;
         else if (split == 1 && rest <= 128 * slots)
@@ -171,21 +177,31 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
     t.ws_bytes = 0;
     t.separate = false;
     t.fused = false;
-    if (t.blocks == 4 && tiles < slots && max_pieces >= 4) {
-        // Fewer tiles than the CUs hold at once: they spread one per CU, then two per CU, ..., and
-        // the launch lasts as long as the busiest CU.  A last layer that covers at most half of the
-        // CUs is computed as two 64-row pieces per tile, dispatched after the whole tiles in the
-        // same launch, so that it covers twice as many CUs for about half as long: measured +25 to
-        // +40 % up to 384 tiles, +17 % with two whole layers, +10 % with three (+6 % on the 1:8
-        // geometry when there is no whole layer: a lone 64-row wave per SIMD hides little latency).
-        const long long layer = tiles % 256;
-        if (layer == 0 || layer > 128)
-            return t;
+    if (t.blocks == 4 && max_pieces >= 4) {
+        // 128-row waves.  Fewer tiles than the CUs hold at once spread one per CU, then two per CU,
+        // ..., and the launch lasts as long as the busiest CU: a last layer that covers at most half
+        // of the CUs is computed as two 64-row pieces per tile, dispatched after the whole tiles in
+        // the same launch, so that it covers twice as many CUs for about half as long (+25 to +40 %
+        // up to 384 tiles, +17 % with two whole layers, +10 % with three).  After one or more full
+        // rounds the workgroups of a CU finish close together and the dispatcher refills a CU's four
+        // slots at once, so up to half a round of leftovers lands packed on a quarter of the CUs:
+        // as pieces in a launch of their own they spread (+12 to +33 % at 2:8, up to +13 % at 1:8,
+        // +6 to +21 % at 2:4 except around a quarter round, where whole tiles are 2 % better).
+        // More than half a round left over: only its last layer, as above (+2 to +5 %).
+        const long long rest = tiles % slots, layer = tiles % 256;
         t.separate = true;
-        t.fused = true;
-        t.head = tiles - layer;
-        t.tail = layer;
         t.sub = 2;
+        if (tiles >= slots && rest > 0 && rest <= slots / 2) {
+            t.tail = rest;  // in a launch of their own: at the end of the first they would land packed too
+        } else if (layer > 0 && layer <= 128) {
+            t.tail = layer;
+            t.fused = true;
+        } else {
+            t.separate = false;
+            t.sub = 1;
+            return t;
+        }
+        t.head = tiles - t.tail;
         return t;
     }
     const long long rest = tiles % slots;
@@ -201,9 +217,10 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
         t.tail = rest;
         t.sub = pieces;
     } else {
-        // 128-row waves, four workgroups per CU: the finer grain already fills the last round well
-        // after one full round (a launch of their own was measured 0 to 16 % SLOWER there).  In
-        // steady state (two or more full rounds) a launch of their own spreads few leftovers.
+        // 128-row form of the short-vector kernel (it has no 64-row pieces), four workgroups per
+        // CU: the finer grain already fills the last round well after one full round (a launch of
+        // their own was measured 0 to 16 % SLOWER there).  In steady state (two or more full
+        // rounds) a launch of their own spreads few leftovers.
         if (tiles < 2 * slots || rest > slots / 2)
             return t;
         t.separate = true;
@@ -223,7 +240,7 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
 
 // Whole multiplication on the tile kernel: 6 us per launch, C written at about 8 TB/s, the kernel,
 // and for a split the second pass that moves (2 * split + 1) * M * N floats at about 8 TB/s (the
-// slices are cache resident) plus its launch.
+// slices are cache resident) plus 4 us for its launch behind the first.
 inline double model_tile_seconds(int M, int N, int nwin, int kept, int split)
 {
     const double c_bytes = (double)M * N * sizeof(float);
@@ -232,7 +249,7 @@ inline double model_tile_seconds(int M, int N, int nwin, int kept, int split)
         blocks = 2;  // as launch_mfma does (the column-block width is taken to be 128)
     double t = 6e-6 + c_bytes / 8e12 + model_kernel_seconds(M, N, nwin, kept, blocks, split);
     if (split > 1)
-        t += (2.0 * split + 1.0) * c_bytes / 8e12 + 2e-6;
+        t += (2.0 * split + 1.0) * c_bytes / 8e12 + 4e-6;
     return t;
 }
 // Whole multiplication on the decode kernel (M <= 128): one workgroup per 32-column vector, 256

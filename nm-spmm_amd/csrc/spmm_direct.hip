@@ -28,6 +28,7 @@
 //    lane reads outside A or B without a branch; lanes whose rows lie beyond M read zeros or
 //    other rows' values into accumulators that are never stored.
 #include "internal.h"
+#include <type_traits>
 
 namespace nmspmm {
 
@@ -101,6 +102,12 @@ __device__ inline float buffer_load_f1(__amdgpu_buffer_rsrc_t r, uint32_t byte_o
 #ifndef NMSPMM_RM_TALL
 #define NMSPMM_RM_TALL 8
 #endif
+#ifndef NMSPMM_BDEPTH
+#define NMSPMM_BDEPTH 1
+#endif
+#ifndef NMSPMM_UNROLL2
+#define NMSPMM_UNROLL2 0
+#endif
 
 // KS: dense rows per window, WS: kept rows per window, QS: column vectors per preprocessed column
 // block (Ns = 32*QS), WR: waves along M, RM: 32-row blocks per wave (2, 4 or 8), HIGH:
@@ -163,10 +170,10 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
     const uint32_t row_bytes = (uint32_t)((size_t)lda * sizeof(float));
     const uint32_t a_vlane = (uint32_t)(j * IL * sizeof(float));  // this lane's run of IL rows inside the wave's rows
     const uint32_t b_chunk = (uint32_t)((size_t)CH * N * sizeof(float));
-    uint32_t b_off[CS];
-#pragma unroll
-    for (int s = 0; s < CS; ++s)
-        b_off[s] = (uint32_t)(((size_t)(2 * s + h) * N + j) * sizeof(float));
+    // B operand of k-step s: this lane's element of kept row 2s + h.  The lane part sits in one
+    // register, the k-step part is a scalar offset of the load
+    const uint32_t b_lane = (uint32_t)(((size_t)h * N + j) * sizeof(float));
+    const uint32_t b_step = (uint32_t)((size_t)2 * N * sizeof(float));
 
     // ---- index metadata: d_vec / ci_vec belong to the window whose operands are being loaded,
     // d_nxt / ci_nxt to the one after it
@@ -210,10 +217,15 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
         }
     };
 
+    // B operands are loaded BD chunks ahead of their use, A operands one chunk: B streams from HBM
+    // (each element is read by the few workgroups of one column block), A is mostly served by the
+    // L2.  With 8 kept rows per window a chunk is only 4 k-steps, a thousand matrix-pipe cycles,
+    // which covers an L2 hit but not an HBM miss when the wave has its SIMD to itself; two chunks do.
+    constexpr int BD = (NMSPMM_BDEPTH >= 2 && NCH == 1 && WS == 8) ? 2 : 1;
     afrag_t a_op[CS];
-    float b_op[CS];
-    // operands of k-step s of chunk c of the window the descriptors point at
-    auto load_step = [&](int c, int s, __amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb) {
+    float b_op[BD][CS];
+    // A operand of k-step s of chunk c of the window the descriptor points at
+    auto load_a = [&](int s, __amdgpu_buffer_rsrc_t ra) {
         const uint32_t off = a_off[s];
         if constexpr (RM == 8) {
             a_op[s].lo = buffer_load_f4(ra, off);
@@ -223,7 +235,6 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
         } else {
             a_op[s] = buffer_load_f2(ra, off);
         }
-        b_op[s] = buffer_load_f1(rb, b_off[s], c * b_chunk);
     };
 
     floatx16 acc[RM];
@@ -234,18 +245,31 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
             acc[b][v] = 0.0f;
 
     if (w_count > 0) {
+        // the loads are issued in the order of the loop (index metadata of the window after, then
+        // the operands), so that the wait counts the compiler places at the loop head for the
+        // metadata leave the operand loads in flight on the first pass as on every other
         load_meta(w_begin);
         take_meta();
+        load_meta(min(w_begin + 1, w_last));
         resolve_ranks();
         form_offsets(0);
         const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)w_begin * KS * lda, a_bytes);
         const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)w_begin * WS * N, b_bytes);
 #pragma unroll
-        for (int s = 0; s < CS; ++s)
-            load_step(0, s, ra, rb);
-        load_meta(min(w_begin + 1, w_last));
+        for (int s = 0; s < CS; ++s) {
+            load_a(s, ra);
+            b_op[0][s] = buffer_load_f1(rb, b_lane, s * b_step);
+        }
+        if constexpr (BD == 2) {
+            const __amdgpu_buffer_rsrc_t rb1 = make_rsrc(Bvec + (size_t)min(w_begin + 1, w_last) * WS * N, b_bytes);
+#pragma unroll
+            for (int s = 0; s < CS; ++s)
+                b_op[1][s] = buffer_load_f1(rb1, b_lane, s * b_step);
+        }
     }
-    for (int t = 0; t < w_count; ++t) {
+    // window t of this workgroup; PAR (a compile-time 0 or 1) selects the B operand set it uses
+    auto window = [&](const int t, auto par) {
+        constexpr int PAR = decltype(par)::value;
         const int w = w_begin + t;
         const int wn = min(w + 1, w_last);  // the last window reloads itself; nothing consumes it
 #pragma unroll
@@ -262,17 +286,39 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
             const int cl = wrap ? 0 : c + 1;
             form_offsets(cl);
             const __amdgpu_buffer_rsrc_t ra = make_rsrc(Ablk + (size_t)wl * KS * lda, a_bytes);
-            const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)wl * WS * N, b_bytes);
+            const int wb = BD == 2 ? min(w + 2, w_last) : wl;
+            const __amdgpu_buffer_rsrc_t rb = make_rsrc(Bvec + (size_t)wb * WS * N, b_bytes);
 #pragma unroll
             for (int s = 0; s < CS; ++s) {
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int b = 0; b < RM; ++b)
-                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_get(a_op[s], b), b_op[s], acc[b], 0, 0, 0);
+                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_get(a_op[s], b), b_op[PAR][s], acc[b], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
-                load_step(cl, s, ra, rb);
+                load_a(s, ra);
+                b_op[PAR][s] = buffer_load_f1(rb, b_lane, s * b_step + cl * b_chunk);
             }
         }
+    };
+    if constexpr (BD == 2) {
+        int t = 0;
+        for (; t + 1 < w_count; t += 2) {
+            window(t, std::integral_constant<int, 0>());
+            window(t + 1, std::integral_constant<int, 1>());
+        }
+        if (t < w_count)
+            window(t, std::integral_constant<int, 0>());
+    } else if constexpr (NMSPMM_UNROLL2 && NCH == 1 && WS == 8) {
+        int t = 0;
+        for (; t + 1 < w_count; t += 2) {
+            window(t, std::integral_constant<int, 0>());
+            window(t + 1, std::integral_constant<int, 0>());
+        }
+        if (t < w_count)
+            window(t, std::integral_constant<int, 0>());
+    } else {
+        for (int t = 0; t < w_count; ++t)
+            window(t, std::integral_constant<int, 0>());
     }
 
     // ---- epilogue: MFMA result register v of lane (h, j) is row 8*(v/4) + 4*h + v%4 of the block,

@@ -44,7 +44,7 @@ def test_split_suggestion():
     assert L.nmspmm_suggest_split_k(4096, 4096, 2048, 16) == 1      # 4096 waves already
     assert L.nmspmm_suggest_split_k(160, 4096, 2048, 16) in (4, 8)  # 64 workgroups for 256 CUs, 128 windows
     assert L.nmspmm_suggest_split_k(64, 8192, 2048, 16) == 1        # the decode kernel needs no split
-    assert L.nmspmm_suggest_split_k(512, 4096, 1024, 16) == 2
+    assert L.nmspmm_suggest_split_k(512, 4096, 1024, 16) in (1, 2)  # 128 tiles: as 256 pieces along M, or two slices
     assert L.nmspmm_suggest_split_k(192, 512, 128, 16) in (1, 2, 4, 8)  # never more slices than windows
     assert L.nmspmm_suggest_split_k(4096, 4096, 16, 16) == 1        # one window cannot be split
     assert L.nmspmm_suggest_split_k(8, 8192, 1024, 8) == 1          # decode kernel reduces in the workgroup

@@ -215,7 +215,7 @@ def test_auto_entry_point_chooses_the_split_itself(oracle, M, N, K, n, m, sparsi
     check(oracle, d, C.cpu().numpy())
 
 
-@pytest.mark.parametrize("M,N,K,n,m", [(8192, 4224, 1024, 2, 4), (4096, 8448, 1024, 1, 8), (8192, 4224, 2048, 2, 8)])
+@pytest.mark.parametrize("M,N,K,n,m", [(8192, 4224, 1024, 2, 4), (4096, 8448, 1024, 3, 8), (8192, 4224, 2048, 2, 8)])
 @pytest.mark.parametrize("Ns", [128, 64, 32])
 def test_ragged_last_round_is_split_along_k_through_scratch(oracle, M, N, K, n, m, Ns):
     """More tiles than the GPU holds at once and a ragged last round: with scratch the tiles of that
