@@ -97,8 +97,9 @@ inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks,
     if (blocks == 4 && split == 1) {
         // plan_tail computes the last tiles of such a launch as two 64-row pieces each.  Next to
         // whole tiles a piece costs 0.55 of a tile; alone on its CU (one 64-row wave per SIMD) it
-        // hides less latency: 0.65 of a tile, 0.85 on the 1:8 geometry
-        const double lone = kept <= 8 ? 0.85 : 0.65;
+        // hides less latency: 0.65 of a tile, 0.7 on the 1:8 geometry (in its form that loads B two
+        // windows ahead)
+        const double lone = kept <= 8 ? 0.7 : 0.65;
         const long long whole = rest / 256, layer = rest % 256;
         if (full == 0 && layer > 0 && layer <= 128)
             return whole == 0 ? lone * unit : (whole + 0.55) * unit;

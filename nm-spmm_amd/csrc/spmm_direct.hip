@@ -35,6 +35,7 @@ namespace nmspmm {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kXcds = 8;
+constexpr int kCus = 256;
 
 struct DirectParams {
     const float* A;
@@ -102,17 +103,20 @@ __device__ inline float buffer_load_f1(__amdgpu_buffer_rsrc_t r, uint32_t byte_o
 #ifndef NMSPMM_RM_TALL
 #define NMSPMM_RM_TALL 8
 #endif
-#ifndef NMSPMM_BDEPTH
-#define NMSPMM_BDEPTH 1
-#endif
-#ifndef NMSPMM_UNROLL2
-#define NMSPMM_UNROLL2 0
-#endif
+
+// Tile shapes that exist in a second form for launches of at most one workgroup per CU, where
+// each wave has its SIMD to itself (direct_unit's DEEP).
+template <int WS, int RM, bool HIGH>
+constexpr bool has_lone_form()
+{
+    return (HIGH && WS == 8 && RM <= 4) || (!HIGH && WS == 16 && RM == 4);
+}
 
 // KS: dense rows per window, WS: kept rows per window, QS: column vectors per preprocessed column
 // block (Ns = 32*QS), WR: waves along M, RM: 32-row blocks per wave (2, 4 or 8), HIGH:
-// high-sparsity layout (D holds ranks into the window's column_info list).
-template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+// high-sparsity layout (D holds ranks into the window's column_info list), DEEP: B operands are
+// loaded two windows ahead (for launches that leave each wave alone on its SIMD).
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH, bool DEEP = false>
 __device__ __forceinline__ void direct_unit(const DirectParams& p, const int logical, const int sub, const int sub_tiles,
                                             const bool tail_unit, const int unit)
 {
@@ -219,9 +223,16 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
 
     // B operands are loaded BD chunks ahead of their use, A operands one chunk: B streams from HBM
     // (each element is read by the few workgroups of one column block), A is mostly served by the
-    // L2.  With 8 kept rows per window a chunk is only 4 k-steps, a thousand matrix-pipe cycles,
-    // which covers an L2 hit but not an HBM miss when the wave has its SIMD to itself; two chunks do.
-    constexpr int BD = (NMSPMM_BDEPTH >= 2 && NCH == 1 && WS == 8) ? 2 : 1;
+    // L2.  A chunk of a 128-row wave is 4 to 8 k-steps, one to two thousand matrix-pipe cycles,
+    // which covers an L2 hit but not always an HBM miss; two chunks do.  Measured on waves of 64
+    // and 128 rows: 16 and 12 kept rows of 32, 3 to 12 % faster while a CU holds one or two
+    // workgroups, level beyond (the 128-row wave with 16 kept rows would pass 128 registers and
+    // lose its fourth workgroup per CU, so it takes the deeper form only when asked, DEEP); 8 kept
+    // rows of 64, 4 to 20 % faster while each wave has its SIMD to itself and 2 to 5 % slower
+    // otherwise (DEEP again); 16 kept rows of 64 run out of registers with it.  256-row waves
+    // are level either way and keep one.
+    constexpr bool kAlwaysDeep = !HIGH && NCH == 1 && RM <= 4 && !(WS == 16 && RM == 4);
+    constexpr int BD = (kAlwaysDeep || (DEEP && has_lone_form<WS, RM, HIGH>())) ? 2 : 1;
     afrag_t a_op[CS];
     float b_op[BD][CS];
     // A operand of k-step s of chunk c of the window the descriptor points at
@@ -308,14 +319,6 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
         }
         if (t < w_count)
             window(t, std::integral_constant<int, 0>());
-    } else if constexpr (NMSPMM_UNROLL2 && NCH == 1 && WS == 8) {
-        int t = 0;
-        for (; t + 1 < w_count; t += 2) {
-            window(t, std::integral_constant<int, 0>());
-            window(t + 1, std::integral_constant<int, 0>());
-        }
-        if (t < w_count)
-            window(t, std::integral_constant<int, 0>());
     } else {
         for (int t = 0; t < w_count; ++t)
             window(t, std::integral_constant<int, 0>());
@@ -350,7 +353,7 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
 // walk that gives each XCD (consecutive ids go to different XCDs) a contiguous run of the
 // p.head_units logical tiles.  In a launch of K slices (p.tail_slices > 1) consecutive ids are the
 // slices of one tile, in a launch of pieces along M (p.sub_tiles > 1) the pieces of one tile.
-template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH, bool DEEP = false>
 __device__ __forceinline__ void direct_uniform_launch(const DirectParams& p, const int id)
 {
     const bool tail_unit = p.tail_slices > 1;
@@ -366,7 +369,7 @@ __device__ __forceinline__ void direct_uniform_launch(const DirectParams& p, con
         const int xcd = id % kXcds, loc = id / kXcds;
         logical = p.tile_offset + (xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc);
     }
-    direct_unit<KS, WS, QS, WR, RM, HIGH>(p, logical, sub, p.sub_tiles, tail_unit, id);
+    direct_unit<KS, WS, QS, WR, RM, HIGH, DEEP>(p, logical, sub, p.sub_tiles, tail_unit, id);
 }
 
 #define NMSPMM_DIRECT_BOUNDS __launch_bounds__(64 * QS * WR, RM == 8 ? 2 : (HIGH && WS == 16) ? 4 : NMSPMM_OCC)
@@ -377,20 +380,27 @@ __global__ void NMSPMM_DIRECT_BOUNDS spmm_direct_kernel(const DirectParams p)
     direct_uniform_launch<KS, WS, QS, WR, RM, HIGH>(p, blockIdx.x);
 }
 
+// The same with B loaded two windows ahead, for launches of at most one workgroup per CU.
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+__global__ void NMSPMM_DIRECT_BOUNDS spmm_direct_lone_kernel(const DirectParams p)
+{
+    direct_uniform_launch<KS, WS, QS, WR, RM, HIGH, true>(p, blockIdx.x);
+}
+
 // The first p.head_units workgroups compute whole tiles; the ones after them are the pieces, two
 // per tile along M, of the tiles from p.tail_offset on, computed on waves of RM / 2 blocks.  They
 // are dispatched last and fill the CUs that run out of whole tiles, in pieces fine enough to even
 // out the end of the launch (same sums in the same order as whole tiles, no scratch).
-template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH, bool DEEP = false>
 __global__ void NMSPMM_DIRECT_BOUNDS spmm_direct_mixed_kernel(const DirectParams p)
 {
     const int id = blockIdx.x;
     if (id >= p.head_units) {
         const int u = id - p.head_units;
-        direct_unit<KS, WS, QS, WR, RM / 2, HIGH>(p, p.tail_offset + u / 2, u % 2, 2, false, u);
+        direct_unit<KS, WS, QS, WR, RM / 2, HIGH, DEEP>(p, p.tail_offset + u / 2, u % 2, 2, false, u);
         return;
     }
-    direct_uniform_launch<KS, WS, QS, WR, RM, HIGH>(p, id);
+    direct_uniform_launch<KS, WS, QS, WR, RM, HIGH, DEEP>(p, id);
 }
 
 // Sums the slices of the tail tiles in slice order into C (second pass of the tail split).  One
@@ -427,6 +437,23 @@ tail_reduce_kernel(const float* __restrict__ ws, float* __restrict__ C, int M, i
     }
 }
 
+// One launch of uniform workgroups.  A launch of at most one workgroup per CU (each wave alone on
+// its SIMD) takes the form that loads B two windows ahead where the tile shape has one.
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
+static hipError_t launch_uniform(const dim3 grid, const dim3 block, hipStream_t stream, const DirectParams& p)
+{
+    bool lone = false;
+    if constexpr (has_lone_form<WS, RM, HIGH>())
+        lone = (long long)grid.x * grid.y <= kCus;
+    if (lone) {
+        if constexpr (has_lone_form<WS, RM, HIGH>())
+            spmm_direct_lone_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, stream>>>(p);
+    } else {
+        spmm_direct_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, stream>>>(p);
+    }
+    return hipGetLastError();
+}
+
 template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
 static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
 {
@@ -457,24 +484,25 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     const dim3 block(64 * QS * WR);
     dim3 grid(p.tiles_m * p.tiles_n, a.split_k, 1);
     p.head_units = (int)grid.x;
-    if (!own_tail) {
-        spmm_direct_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, a.stream>>>(p);
-        return hipGetLastError();
-    }
+    if (!own_tail)
+        return launch_uniform<KS, WS, QS, WR, RM, HIGH>(grid, block, a.stream, p);
     p.head_units = (int)plan.head;
     if (plan.slices == 1 && plan.sub > 1 && plan.fused) {
         // shorter waves for the leftovers, in the same launch: each leftover tile in two pieces
         // along M, so that the pieces fill the CUs more evenly than whole tiles would
         p.tail_offset = (int)plan.head;
         grid.x = (unsigned)(plan.head + plan.tail * plan.sub);
-        if constexpr (RM == 4)
-            spmm_direct_mixed_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, a.stream>>>(p);
+        if constexpr (RM == 4) {
+            if (has_lone_form<WS, RM, HIGH>() && grid.x <= (unsigned)kCus)
+                spmm_direct_mixed_kernel<KS, WS, QS, WR, RM, HIGH, has_lone_form<WS, RM, HIGH>()><<<grid, block, 0, a.stream>>>(p);
+            else
+                spmm_direct_mixed_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, a.stream>>>(p);
+        }
         return hipGetLastError();
     }
     // head tiles, then the leftover tiles in a launch of their own, whole or in slices along K
     grid.x = (unsigned)plan.head;
-    spmm_direct_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, a.stream>>>(p);
-    hipError_t e = hipGetLastError();
+    hipError_t e = launch_uniform<KS, WS, QS, WR, RM, HIGH>(grid, block, a.stream, p);
     if (e != hipSuccess)
         return e;
     p.tile_offset = (int)plan.head;
@@ -487,19 +515,18 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
         p.head_units = (int)grid.x;
         if (RM / plan.sub == 4) {
             if constexpr (RM >= 8)
-                spmm_direct_kernel<KS, WS, QS, WR, 4, HIGH><<<grid, block, 0, a.stream>>>(p);
+                return launch_uniform<KS, WS, QS, WR, 4, HIGH>(grid, block, a.stream, p);
         } else {
             if constexpr (RM >= 4)
-                spmm_direct_kernel<KS, WS, QS, WR, 2, HIGH><<<grid, block, 0, a.stream>>>(p);
+                return launch_uniform<KS, WS, QS, WR, 2, HIGH>(grid, block, a.stream, p);
         }
-        return hipGetLastError();
+        return hipErrorInvalidValue;
     }
     p.tail_slices = plan.slices;
     p.tail_ws = plan.slices > 1 ? a.tail_ws : nullptr;
     grid.x = (unsigned)(plan.tail * plan.slices);
     p.head_units = (int)grid.x;
-    spmm_direct_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, a.stream>>>(p);
-    e = hipGetLastError();
+    e = launch_uniform<KS, WS, QS, WR, RM, HIGH>(grid, block, a.stream, p);
     if (e == hipSuccess && plan.slices > 1) {
         tail_reduce_kernel<MS, NS><<<dim3((unsigned)plan.tail), dim3(256), 0, a.stream>>>(
             a.tail_ws, a.C, a.M, a.N, p.tiles_m, p.tiles_n, (int)plan.head, plan.slices);
