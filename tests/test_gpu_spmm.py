@@ -293,6 +293,30 @@ def test_last_layer_of_a_small_launch_in_pieces(oracle, M, N, K, n, m, Ns):
     check_every_tile_once(oracle, M, N, K, n, m, Ns)
 
 
+@pytest.mark.parametrize("M,N,K,n,m", [(1024, 4096, 320, 1, 8), (1024, 4096, 64, 1, 8), (512, 4096, 320, 1, 8), (768, 4096, 128, 1, 8),
+                                       (200, 4096, 448, 1, 8), (1024, 4096, 96, 2, 4), (1024, 4096, 32, 2, 4), (384, 4096, 160, 2, 4),
+                                       (2048, 4096, 96, 3, 8), (512, 4096, 32, 3, 8), (2048, 4096, 160, 12, 32)])
+@pytest.mark.parametrize("Ns", [128, 64, 32])
+def test_waves_that_load_b_two_windows_ahead(oracle, M, N, K, n, m, Ns):
+    """64- and 128-row waves load their B operands two windows ahead: at 3:8 always, at 1:8 and 2:4
+    in launches of at most one workgroup per CU (256 whole tiles; 128 or 96 tiles as 256 or 192
+    pieces; 192 whole tiles; 64-row waves for a ragged row count).  The window loop is then
+    unrolled by two: one, two, three, five and seven windows per workgroup.  Every tile exactly
+    once, for every width of the column blocks."""
+    check_every_tile_once(oracle, M, N, K, n, m, Ns)
+
+
+@pytest.mark.parametrize("split_k", [2, 3])
+@pytest.mark.parametrize("M,n,m", [(512, 3, 8), (256, 1, 8), (384, 2, 4)])
+def test_split_slices_of_unequal_length_two_windows_ahead(oracle, M, n, m, split_k):
+    """Seven windows (K = 448 at 1:8, whose windows are 64 rows; K = 224 otherwise) cut into two or
+    three slices: slices of odd and even length on the window loop unrolled by two."""
+    d = datagen.init_data(M, 1024, 448 if m == 8 and n == 1 else 224, n, m, seed=M + split_k)
+    got, fam = run_gpu(oracle, d, 128, split_k=split_k)
+    assert fam == "mfma"
+    check(oracle, d, got)
+
+
 def test_llm_layer_shape_2of8(oracle):
     """One LLM-layer shape (M = 512, K = 4096, Ncols = 11008, 2:8, N(0,1) x N(0,0.02^2))."""
     d = datagen.init_data(512, 11008, 4096, 2, 8, seed=3001, dist="normal", b_scale=0.02)
