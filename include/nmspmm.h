@@ -192,6 +192,12 @@ int nmspmm_gemm_high_sparsity(int tile, const float* A, const float* B, const in
  * geometry and the layout as nmspmm_pattern_from_sparsity does, column_info is required for the
  * high-sparsity layout and ignored otherwise. */
 int nmspmm_suggest_split_k(int M, int N, int W, int kept);
+/* No counterpart in the reference.  Rows per workgroup (128 or 64) when an unsplit multiplication
+ * (split_k == 1) of this shape on the matrix-core kernel is computed with the reduction shared
+ * between the four waves of each workgroup and added up in LDS (problems of few tiles; no
+ * workspace, one launch), 0 when it is computed tile by tile or the arguments are invalid.
+ * Informational: the choice is the library's. */
+int nmspmm_waves_along_k_rows(int M, int N, int W, int kept);
 int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int32_t* column_info,
                      float* C, int M, int N, int K, int W, float sparsity, void* stream);
 

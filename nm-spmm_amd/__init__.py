@@ -67,6 +67,7 @@ def lib():
         L.nmspmm_workspace_bytes_rowmajor.argtypes = [c_int] * 4
         L.nmspmm_spmm_rowmajor.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, c_void_p]
         L.nmspmm_suggest_split_k.argtypes = [c_int] * 4
+        L.nmspmm_waves_along_k_rows.argtypes = [c_int] * 4
         L.nmspmm_gemm_auto.argtypes = [c_void_p] * 5 + [c_int] * 4 + [c_float, c_void_p]
         L.nmspmm_release.restype = c_int
         _lib = L
@@ -189,6 +190,12 @@ def spmm_rowmajor(A_rm, B, D, cinfo, C, M, N, K, W, window, kept, workspace, vec
 
 def suggest_split_k(M, N, W, kept):
     return lib().nmspmm_suggest_split_k(M, N, W, kept)
+
+
+def waves_along_k_rows(M, N, W, kept):
+    """128 or 64 when an unsplit multiplication of this shape shares the reduction between the
+    waves of a workgroup, 0 otherwise."""
+    return lib().nmspmm_waves_along_k_rows(M, N, W, kept)
 
 
 def gemm_auto(A, B, D, cinfo, C, M, N, K, W, sparsity):

@@ -580,6 +580,13 @@ int nmspmm_suggest_split_k(int M, int N, int W, int kept)
     return best;
 }
 
+int nmspmm_waves_along_k_rows(int M, int N, int W, int kept)
+{
+    if (M <= 0 || N <= 0 || W <= 0 || kept <= 0 || W % kept != 0)
+        return 0;
+    return inner_split_pays(M, N, W / kept, kept) ? plan_inner(M, N, W / kept, kept).rows : 0;
+}
+
 int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C,
                      int M, int N, int K, int W, float sparsity, void* stream)
 {

@@ -239,6 +239,59 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
     return t;
 }
 
+// The launch with four waves along K (spmm_direct_inner_kernel): one workgroup per 128 or 64 rows
+// of one 32-column vector, each of its four waves over a quarter of the windows, partial sums
+// added in LDS.  It cuts the reduction without scratch or a second pass, for problems of at most
+// 256 tiles of 128 x 128 (measured on 96 shapes, M = 192 ... 1024, against the best of the splits
+// 1, 2, 4, 8 of the tile kernel: 2 to 56 % faster up to 256 tiles, 0 to 16 % slower at 512).
+// Two workgroups of 128-row waves fit a CU (64 KB of LDS each), so they retire in rounds of 512:
+// up to 256 run one per CU (at 0.9 of the rate, one wave per SIMD), up to 512 two per CU, and the
+// leftovers of full rounds land two per CU on the CUs that free up first (768 workgroups take as
+// long as 1024, measured) unless they are at most 128 (then 1.2 of a workgroup's time, measured).
+// Workgroups of 64-row waves (32 KB) spread evenly, a layer per 256, and cost 0.56 of the taller
+// ones each.
+struct InnerPlan {
+    bool pays;     // eligible at all
+    int rows;      // 128 or 64 rows per workgroup
+    double seconds;  // modelled kernel time
+};
+inline InnerPlan plan_inner(int M, int N, int nwin, int kept)
+{
+    InnerPlan r;
+    r.pays = false;
+    r.rows = 128;
+    r.seconds = 0.0;
+    const long long tiles = (long long)((M + 127) / 128) * ((N + 127) / 128);
+    if (tiles > 256 || nwin < 8 || M <= 32)
+        return r;
+    const long long vecs = N / 32;
+    const long long g4 = (long long)((M + 127) / 128) * vecs, g2 = (long long)((M + 63) / 64) * vecs;
+    const long long full = g4 / 512, rest = g4 % 512, b2 = (g2 + 255) / 256;
+    double c4;
+    if (full == 0)
+        c4 = rest <= 256 ? 1.0 / 0.9 : 2.0;
+    else
+        c4 = 2.0 * full + (rest == 0 ? 0.0 : rest <= 128 ? 1.2 : 2.0);
+    const double c2 = 0.56 * (b2 == 1 ? 1.0 / 0.9 : (double)b2);
+    const double unit = kept * 53.5e-9 * ((nwin + 3) / 4);
+    r.pays = true;
+    r.rows = c2 < c4 ? 64 : 128;
+    r.seconds = (c2 < c4 ? c2 : c4) * unit + 1e-6;
+    return r;
+}
+
+// Whether an unsplit multiplication takes the launch with four waves along K.
+inline bool inner_split_pays(int M, int N, int nwin, int kept)
+{
+    const InnerPlan inner = plan_inner(M, N, nwin, kept);
+    if (!inner.pays)
+        return false;
+    int blocks = choose_wave_blocks(M, N, nwin, kept, 1);
+    if (blocks == 4 && short_waves_pay(M))
+        blocks = 2;
+    return inner.seconds < model_kernel_seconds(M, N, nwin, kept, blocks, 1);
+}
+
 // Whole multiplication on the tile kernel: 6 us per launch, C written at about 8 TB/s, the kernel,
 // and for a split the second pass that moves (2 * split + 1) * M * N floats at about 8 TB/s (the
 // slices are cache resident) plus 4 us for its launch behind the first.
@@ -248,7 +301,13 @@ inline double model_tile_seconds(int M, int N, int nwin, int kept, int split)
     int blocks = choose_wave_blocks(M, N, nwin, kept, split);
     if (blocks == 4 && short_waves_pay(M))
         blocks = 2;  // as launch_mfma does (the column-block width is taken to be 128)
-    double t = 6e-6 + c_bytes / 8e12 + model_kernel_seconds(M, N, nwin, kept, blocks, split);
+    double kernel = model_kernel_seconds(M, N, nwin, kept, blocks, split);
+    if (split == 1) {
+        const InnerPlan inner = plan_inner(M, N, nwin, kept);
+        if (inner.pays && inner.seconds < kernel)
+            kernel = inner.seconds;  // launch_mfma takes that launch then
+    }
+    double t = 6e-6 + c_bytes / 8e12 + kernel;
     if (split > 1)
         t += (2.0 * split + 1.0) * c_bytes / 8e12 + 4e-6;
     return t;

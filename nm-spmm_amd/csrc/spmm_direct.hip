@@ -115,8 +115,11 @@ constexpr bool has_lone_form()
 // KS: dense rows per window, WS: kept rows per window, QS: column vectors per preprocessed column
 // block (Ns = 32*QS), WR: waves along M, RM: 32-row blocks per wave (2, 4 or 8), HIGH:
 // high-sparsity layout (D holds ranks into the window's column_info list), DEEP: B operands are
-// loaded two windows ahead (for launches that leave each wave alone on its SIMD).
-template <int KS, int WS, int QS, int WR, int RM, bool HIGH, bool DEEP = false>
+// loaded two windows ahead (for launches that leave each wave alone on its SIMD), KW: waves along
+// K.  With KW > 1 (WR == 1) the workgroup's KW waves compute the same RM*32 rows of ONE 32-column
+// vector, each over its share of the windows, and add their results up through LDS in wave order;
+// QS then only describes the index layout, and the tile walk counts vectors, not column blocks.
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH, bool DEEP = false, int KW = 1>
 __device__ __forceinline__ void direct_unit(const DirectParams& p, const int logical, const int sub, const int sub_tiles,
                                             const bool tail_unit, const int unit)
 {
@@ -145,27 +148,32 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
         tile_m = first_m + in_band % rows;
         tile_n = in_band / rows;
     }
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    static_assert(KW == 1 || WR == 1, "waves along K share their rows");
     int w_begin, w_count;
-    if (!tail_unit)
+    if constexpr (KW > 1)
+        split_windows(p.nwin, KW, wave, &w_begin, &w_count);
+    else if (!tail_unit)
         split_windows(p.nwin, p.split_k, blockIdx.y, &w_begin, &w_count);
     else
         split_windows(p.nwin, p.tail_slices, unit % p.tail_slices, &w_begin, &w_count);
     const int w_last = w_begin + w_count - 1;
 
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int vec = wave % QS;
-    const int wr = wave / QS;
+    // column vector inside its preprocessed column block, and that block
+    const int vec = KW > 1 ? tile_n % QS : wave % QS;
+    const int wr = KW > 1 ? 0 : wave / QS;
+    const int block_n = KW > 1 ? tile_n / QS : tile_n;
     const int h = lane >> 5;
     const int j = lane & 31;
     const int M = p.M, N = p.N, lda = p.lda;
     const int bi = (tile_m * sub_tiles + sub) * MS + wr * MW;  // first row of this wave (may be >= M: loads nothing)
-    const int bj = tile_n * NS + vec * 32;
+    const int bj = block_n * NS + vec * 32;
 
     const float* const Ablk = p.A + min(bi, lda);
     const float* const Bvec = p.B + bj;
-    const int32_t* const Dblk = p.D + (size_t)tile_n * p.W * QS;
-    const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)tile_n * p.nwin * KS : nullptr;
+    const int32_t* const Dblk = p.D + (size_t)block_n * p.W * QS;
+    const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)block_n * p.nwin * KS : nullptr;
     // extents: the last dense row of a window ends with its lda floats (rows between M and lda are
     // padding that may be read and is never stored), the last kept row of B with this vector's 32
     // columns
@@ -338,6 +346,44 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
     const __amdgpu_buffer_rsrc_t rc = make_rsrc(c_base, c_bytes);
     const uint32_t c_lane = (uint32_t)(((size_t)4 * IL * h * pitch + j) * sizeof(float));
     const uint32_t n_bytes = (uint32_t)((size_t)pitch * sizeof(float));
+    if constexpr (KW > 1) {
+        // Waves along K: every wave leaves its sums in LDS, and the groups of four result registers
+        // are dealt out to the waves, group g to wave g % KW, which adds the KW partial sums in wave
+        // order (the order of the windows) and stores the group's four rows.
+        static_assert(RM <= 4, "64 KB of LDS");
+        __shared__ float4 partial[KW][RM * 4][64];
+#pragma unroll
+        for (int b = 0; b < RM; ++b)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                partial[wave][b * 4 + q][lane] = make_float4(acc[b][4 * q], acc[b][4 * q + 1], acc[b][4 * q + 2], acc[b][4 * q + 3]);
+        __syncthreads();
+#pragma unroll
+        for (int b = 0; b < RM; ++b) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int g = b * 4 + q;
+                if (g % KW != wave)
+                    continue;
+                float4 sum = partial[0][g][lane];
+#pragma unroll
+                for (int z = 1; z < KW; ++z) {
+                    const float4 t = partial[z][g][lane];
+                    sum.x += t.x;
+                    sum.y += t.y;
+                    sum.z += t.z;
+                    sum.w += t.w;
+                }
+                const float out4[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t row = (b / 4) * 128 + IL * (8 * q + i) + (b % IL);
+                    __builtin_amdgcn_raw_buffer_store_b32(__float_as_int(out4[i]), rc, c_lane + row * n_bytes, 0, 0);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
 #pragma unroll
@@ -353,7 +399,7 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
 // walk that gives each XCD (consecutive ids go to different XCDs) a contiguous run of the
 // p.head_units logical tiles.  In a launch of K slices (p.tail_slices > 1) consecutive ids are the
 // slices of one tile, in a launch of pieces along M (p.sub_tiles > 1) the pieces of one tile.
-template <int KS, int WS, int QS, int WR, int RM, bool HIGH, bool DEEP = false>
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH, bool DEEP = false, int KW = 1>
 __device__ __forceinline__ void direct_uniform_launch(const DirectParams& p, const int id)
 {
     const bool tail_unit = p.tail_slices > 1;
@@ -369,7 +415,7 @@ __device__ __forceinline__ void direct_uniform_launch(const DirectParams& p, con
         const int xcd = id % kXcds, loc = id / kXcds;
         logical = p.tile_offset + (xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc);
     }
-    direct_unit<KS, WS, QS, WR, RM, HIGH, DEEP>(p, logical, sub, p.sub_tiles, tail_unit, id);
+    direct_unit<KS, WS, QS, WR, RM, HIGH, DEEP, KW>(p, logical, sub, p.sub_tiles, tail_unit, id);
 }
 
 #define NMSPMM_DIRECT_BOUNDS __launch_bounds__(64 * QS * WR, RM == 8 ? 2 : (HIGH && WS == 16) ? 4 : NMSPMM_OCC)
@@ -385,6 +431,15 @@ template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
 __global__ void NMSPMM_DIRECT_BOUNDS spmm_direct_lone_kernel(const DirectParams p)
 {
     direct_uniform_launch<KS, WS, QS, WR, RM, HIGH, true>(p, blockIdx.x);
+}
+
+// Four waves along K: one workgroup per RM*32 rows of one 32-column vector (p.tiles_n counts
+// vectors), the reduction over K split between its waves and finished in LDS.  For problems of so
+// few tiles that the reduction has to be cut to fill the GPU: no scratch, no second pass.
+template <int KS, int WS, int QS, int RM, bool HIGH, bool DEEP>
+__global__ void __launch_bounds__(256, 2) spmm_direct_inner_kernel(const DirectParams p)
+{
+    direct_uniform_launch<KS, WS, QS, 1, RM, HIGH, DEEP, 4>(p, blockIdx.x);
 }
 
 // The first p.head_units workgroups compute whole tiles; the ones after them are the pieces, two
@@ -535,6 +590,61 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     return e;
 }
 
+#ifndef NMSPMM_INNER
+#define NMSPMM_INNER 1
+#endif
+#ifndef NMSPMM_INNER_RM
+#define NMSPMM_INNER_RM 0
+#endif
+
+// The launch with four waves along K (spmm_direct_inner_kernel), on 128- or 64-row tiles as
+// plan_inner chooses.
+template <int KS, int WS, int QS, bool HIGH>
+static hipError_t launch_inner(const SpmmArgs& a)
+{
+    const long long vecs = a.N / 32;
+    const int rows = NMSPMM_INNER_RM != 0 ? NMSPMM_INNER_RM * 32 : plan_inner(a.M, a.N, a.W / WS, WS).rows;
+    const bool tall = rows == 128;
+    DirectParams p;
+    p.A = a.A;
+    p.B = a.B;
+    p.D = a.D;
+    p.cinfo = a.cinfo;
+    p.out = a.C;
+    p.slice_elems = 0;
+    p.M = a.M;
+    p.lda = a.lda;
+    p.N = a.N;
+    p.W = a.W;
+    p.nwin = a.W / WS;
+    p.split_k = 1;
+    p.tiles_m = (a.M + rows - 1) / rows;
+    p.tiles_n = (int)vecs;
+    p.tile_offset = 0;
+    p.tail_slices = 1;
+    p.tail_ws = nullptr;
+    p.tail_offset = 0;
+    p.sub_tiles = 1;
+    const long long groups = (long long)p.tiles_m * p.tiles_n;
+    if (groups > 0x7fffffffLL)
+        return hipErrorInvalidValue;
+    p.head_units = (int)groups;
+    const dim3 grid((unsigned)groups), block(256);
+    const bool lone = groups <= kCus;
+    if (tall) {
+        if (lone && has_lone_form<WS, 4, HIGH>())
+            spmm_direct_inner_kernel<KS, WS, QS, 4, HIGH, has_lone_form<WS, 4, HIGH>()><<<grid, block, 0, a.stream>>>(p);
+        else
+            spmm_direct_inner_kernel<KS, WS, QS, 4, HIGH, false><<<grid, block, 0, a.stream>>>(p);
+    } else {
+        if (lone && has_lone_form<WS, 2, HIGH>())
+            spmm_direct_inner_kernel<KS, WS, QS, 2, HIGH, has_lone_form<WS, 2, HIGH>()><<<grid, block, 0, a.stream>>>(p);
+        else
+            spmm_direct_inner_kernel<KS, WS, QS, 2, HIGH, false><<<grid, block, 0, a.stream>>>(p);
+    }
+    return hipGetLastError();
+}
+
 // Every workgroup has four waves: 1 x 4, 2 x 2 or 4 x 1 (rows x column vectors), chosen by the
 // column-block width the indices were preprocessed for.  A wave is 256 or 128 rows tall, whichever
 // the run-time model expects to finish first: the taller wave halves the B and index loads per
@@ -566,6 +676,13 @@ static TailPlan tail_plan_for(const SpmmArgs& a, bool have_scratch)
 template <int KS, int WS, bool HIGH>
 static hipError_t launch_ns(const SpmmArgs& a)
 {
+    if (a.split_k == 1 && a.W / WS >= 4 && (NMSPMM_INNER == 2 || (NMSPMM_INNER == 1 && inner_split_pays(a.M, a.N, a.W / WS, WS)))) {
+        switch (a.Ns) {
+        case 128: return launch_inner<KS, WS, 4, HIGH>(a);
+        case 64: return launch_inner<KS, WS, 2, HIGH>(a);
+        case 32: return launch_inner<KS, WS, 1, HIGH>(a);
+        }
+    }
     const TailPlan plan = tail_plan_for(a, true);
     const bool tall = NMSPMM_RM_TALL == 8 && plan.blocks == 8;
     if (!tall && a.Ns == 128 && short_waves_pay(a.M))

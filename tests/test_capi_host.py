@@ -42,7 +42,8 @@ def test_library_exports_the_cxx_drop_in_functions():
 def test_split_suggestion():
     L = nmspmm.lib()
     assert L.nmspmm_suggest_split_k(4096, 4096, 2048, 16) == 1      # 4096 waves already
-    assert L.nmspmm_suggest_split_k(160, 4096, 2048, 16) in (4, 8)  # 64 workgroups for 256 CUs, 128 windows
+    assert L.nmspmm_suggest_split_k(160, 4096, 2048, 16) == 1       # 64 tiles, 128 windows: the four waves of a workgroup share the reduction
+    assert L.nmspmm_suggest_split_k(2048, 12288, 16384, 16) == 1    # 1536 tiles fill the GPU
     assert L.nmspmm_suggest_split_k(64, 8192, 2048, 16) == 1        # the decode kernel needs no split
     assert L.nmspmm_suggest_split_k(512, 4096, 1024, 16) in (1, 2)  # 128 tiles: as 256 pieces along M, or two slices
     assert L.nmspmm_suggest_split_k(192, 512, 128, 16) in (1, 2, 4, 8)  # never more slices than windows

@@ -209,7 +209,8 @@ def test_auto_entry_point_chooses_the_split_itself(oracle, M, N, K, n, m, sparsi
     split = nmspmm.suggest_split_k(M, N, d["W"], kept)
     assert 1 <= split <= 16 and (d["W"] // kept) // split >= 1
     if M == 160 and K == 2048:
-        assert split > 1          # 64 workgroups for 256 CUs: the reduction must be split
+        # 16 tiles for 256 CUs: the reduction must be cut, between workgroups or inside them
+        assert split > 1 or nmspmm.waves_along_k_rows(M, N, d["W"], kept) > 0
     if M == 2048 or M <= 32:
         assert split == 1
     check(oracle, d, C.cpu().numpy())
@@ -304,6 +305,26 @@ def test_waves_that_load_b_two_windows_ahead(oracle, M, N, K, n, m, Ns):
     unrolled by two: one, two, three, five and seven windows per workgroup.  Every tile exactly
     once, for every width of the column blocks."""
     check_every_tile_once(oracle, M, N, K, n, m, Ns)
+
+
+@pytest.mark.parametrize("M,N,K,n,m,rows", [(256, 2048, 512, 2, 4, 64), (512, 4096, 1024, 1, 8, 128), (192, 1024, 1024, 2, 8, 64),
+                                            (1000, 2048, 1056, 3, 8, 128), (300, 1024, 352, 32, 32, 64), (132, 2048, 512, 2, 4, 64),
+                                            (768, 4096, 2112, 1, 8, 64), (256, 8192, 2112, 2, 8, 128)])
+@pytest.mark.parametrize("Ns", [128, 64, 32])
+def test_reduction_shared_between_the_waves_of_a_workgroup(oracle, M, N, K, n, m, rows, Ns):
+    """Problems of few tiles: one workgroup per 128 or 64 rows of one 32-column vector, its four
+    waves each over a quarter of the windows (33 and eleven windows: unequal quarters), partial
+    sums added in LDS.  Ragged row counts, every index layout, every width of the column blocks;
+    every tile exactly once."""
+    window, kept, _ = kernel_geometry(n, m)
+    assert nmspmm.waves_along_k_rows(M, N, K // window * kept, kept) == rows
+    check_every_tile_once(oracle, M, N, K, n, m, Ns)
+
+
+def test_larger_problems_stay_on_whole_tiles():
+    assert nmspmm.waves_along_k_rows(2048, 4096, 2048, 16) == 0    # 512 tiles
+    assert nmspmm.waves_along_k_rows(256, 2048, 64, 16) == 0       # four windows: nothing to share
+    assert nmspmm.waves_along_k_rows(0, 2048, 64, 16) == 0
 
 
 @pytest.mark.parametrize("split_k", [2, 3])
