@@ -5,7 +5,8 @@
 // Design for gfx950 (64-lane waves, v_mfma_f32_32x32x2_f32):
 //  * A 32-column index vector is exactly the N extent of one 32x32x2 MFMA, so one wave owns one
 //    column vector and RM row blocks of 32 rows, and is independent of every other wave: no LDS,
-//    no barrier.
+//    no barrier (the one exception: problems of few tiles, where the four waves of a workgroup
+//    share the reduction of one vector and add their sums up in LDS at the end).
 //  * The A operand of one MFMA is A[row][k] with lane = (row % 32, k half): lanes 0-31 take kept
 //    row 2s of the window, lanes 32-63 kept row 2s+1, and each half reads the dense row of A that
 //    *its* index selects.  A is column-major, so that is M contiguous floats: the gather is a
