@@ -591,6 +591,9 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     return e;
 }
 
+// Tuning builds: NMSPMM_INNER 0 never takes the launch with waves along K, 2 takes it for every
+// unsplit call (1: where the run-time model expects it to win); NMSPMM_INNER_RM 2 or 4 fixes its
+// wave height (0: the model's choice).
 #ifndef NMSPMM_INNER
 #define NMSPMM_INNER 1
 #endif
