@@ -46,6 +46,22 @@ __host__ __device__ inline void split_windows(int nwin, int split_k, int z, int*
 // layout is used.
 inline double tall_wave_cost(int kept) { return kept <= 8 ? 2.0 / 1.03 : 2.0 / 1.05; }
 
+#ifndef NMSPMM_TAIL_ALONG_K
+#define NMSPMM_TAIL_ALONG_K 1
+#endif
+// Whether the last layer of a launch of fewer tiles than the GPU holds at once is computed by
+// workgroups whose four waves share the reduction (four per tile, each a quarter of a tile's time
+// and alone on its CU) rather than as two 64-row pieces per tile (0.55 of a tile's time each).
+// Measured on 156 shapes of 288 to 640 tiles against the pieces: 10 to 13 % faster with one whole
+// layer and at most 64 tiles after it (5 to 7 % at 1:8); level to 5 % slower with 65 to 128 tiles
+// after it (two such workgroups per CU), and -7 to +3 % after two whole layers (that kernel's LDS
+// lets a CU hold two workgroups only), so it is taken in the first case.  (Without a whole layer
+// the whole problem takes the launch with waves along K, plan_inner.)
+inline bool tail_along_k(long long tiles, int nwin)
+{
+    return NMSPMM_TAIL_ALONG_K != 0 && tiles > 256 && tiles <= 320 && nwin >= 8;
+}
+
 // Leftover tiles of 256-row waves (two workgroups per CU) after at least one full round: `rest`
 // tiles, each `unit` seconds of a CU's pipes.  Left in the launch they land packed on the CUs that
 // free up first and the last round lasts as long as a full one (measured: 2752 tiles on 512 slots
@@ -101,8 +117,11 @@ inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks,
         // windows ahead)
         const double lone = kept <= 8 ? 0.7 : 0.65;
         const long long whole = rest / 256, layer = rest % 256;
-        if (full == 0 && layer > 0 && layer <= 128)
+        if (full == 0 && layer > 0 && layer <= 128) {
+            if (tail_along_k(rest, nwin))  // a quarter of a tile each, one per CU at 0.9 of the rate
+                return (whole + 0.25 / 0.9) * unit + 1e-6;
             return whole == 0 ? lone * unit : (whole + 0.55) * unit;
+        }
         if (full >= 1 && rest > 0 && rest <= 128 * slots) {
             const long long busiest_piece = (2 * rest + 255) / 256;
             return (double)full * slots * unit + (busiest_piece == 1 ? lone : 0.55 * busiest_piece) * unit + 10e-6;
@@ -158,6 +177,8 @@ struct TailPlan {
     int sub;         // > 1: the tail tiles run as `sub` pieces along M each, on waves of blocks / sub blocks
     size_t ws_bytes; // scratch needed
     bool fused;      // the pieces along M are part of the launch of the whole tiles, after them
+    bool along_k;    // fused, and the tail tiles run as four workgroups each (one per 128 rows of one
+                     // 32-column vector) whose four waves share the reduction, instead of pieces along M
     bool separate;   // without scratch: give the tail tiles a launch of their own (they then spread
                      // one or two per CU instead of landing packed on the CUs that free up last)
 };
@@ -178,6 +199,7 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
     t.ws_bytes = 0;
     t.separate = false;
     t.fused = false;
+    t.along_k = false;
     if (t.blocks == 4 && max_pieces >= 4) {
         // 128-row waves.  Fewer tiles than the CUs hold at once spread one per CU, then two per CU,
         // ..., and the launch lasts as long as the busiest CU: a last layer that covers at most half
@@ -197,6 +219,7 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
         } else if (layer > 0 && layer <= 128) {
             t.tail = layer;
             t.fused = true;
+            t.along_k = tail_along_k(tiles, nwin);
         } else {
             t.separate = false;
             t.sub = 1;

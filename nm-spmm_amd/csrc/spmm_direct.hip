@@ -151,7 +151,6 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
     }
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    static_assert(KW == 1 || WR == 1, "waves along K share their rows");
     int w_begin, w_count;
     if constexpr (KW > 1)
         split_windows(p.nwin, KW, wave, &w_begin, &w_count);
@@ -161,14 +160,18 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
         split_windows(p.nwin, p.tail_slices, unit % p.tail_slices, &w_begin, &w_count);
     const int w_last = w_begin + w_count - 1;
 
-    // column vector inside its preprocessed column block, and that block
-    const int vec = KW > 1 ? tile_n % QS : wave % QS;
-    const int wr = KW > 1 ? 0 : wave / QS;
-    const int block_n = KW > 1 ? tile_n / QS : tile_n;
+    // column vector inside its preprocessed column block, and that block.  With waves along K the
+    // workgroup is either one vector of a walk over vectors, or (sub_tiles == 0) unit `sub` of the
+    // WR * QS units, 128 rows of one vector each, of a whole tile of the walk over tiles
+    const bool tile_unit = KW > 1 && sub_tiles == 0;
+    const int vec = KW > 1 ? (tile_unit ? sub % QS : tile_n % QS) : wave % QS;
+    const int wr = KW > 1 ? (tile_unit ? sub / QS : 0) : wave / QS;
+    const int block_n = KW > 1 && !tile_unit ? tile_n / QS : tile_n;
     const int h = lane >> 5;
     const int j = lane & 31;
     const int M = p.M, N = p.N, lda = p.lda;
-    const int bi = (tile_m * sub_tiles + sub) * MS + wr * MW;  // first row of this wave (may be >= M: loads nothing)
+    const int bi = tile_unit ? tile_m * MS + wr * MW            // first row of this wave (may be >= M: loads nothing)
+                             : (tile_m * sub_tiles + sub) * MS + wr * MW;
     const int bj = block_n * NS + vec * 32;
 
     const float* const Ablk = p.A + min(bi, lda);
@@ -443,6 +446,22 @@ __global__ void __launch_bounds__(256, 2) spmm_direct_inner_kernel(const DirectP
     direct_uniform_launch<KS, WS, QS, 1, RM, HIGH, DEEP, 4>(p, blockIdx.x);
 }
 
+// The first p.head_units workgroups compute whole tiles; the ones after them the tiles from
+// p.tail_offset on, four workgroups per tile, each 128 rows of one 32-column vector with the
+// reduction shared between its four waves.  They are dispatched last and give the CUs that run out
+// of whole tiles a quarter of a tile each.
+template <int KS, int WS, int QS, int WR, bool HIGH>
+__global__ void __launch_bounds__(256, 2) spmm_direct_mixed_inner_kernel(const DirectParams p)
+{
+    const int id = blockIdx.x;
+    if (id >= p.head_units) {
+        const int u = id - p.head_units;
+        direct_unit<KS, WS, QS, WR, 4, HIGH, false, 4>(p, p.tail_offset + u / 4, u % 4, 0, false, u);
+        return;
+    }
+    direct_uniform_launch<KS, WS, QS, WR, 4, HIGH>(p, id);
+}
+
 // The first p.head_units workgroups compute whole tiles; the ones after them are the pieces, two
 // per tile along M, of the tiles from p.tail_offset on, computed on waves of RM / 2 blocks.  They
 // are dispatched last and fill the CUs that run out of whole tiles, in pieces fine enough to even
@@ -547,6 +566,12 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
         // shorter waves for the leftovers, in the same launch: each leftover tile in two pieces
         // along M, so that the pieces fill the CUs more evenly than whole tiles would
         p.tail_offset = (int)plan.head;
+        if (plan.along_k) {
+            grid.x = (unsigned)(plan.head + plan.tail * 4);
+            if constexpr (RM == 4)
+                spmm_direct_mixed_inner_kernel<KS, WS, QS, WR, HIGH><<<grid, block, 0, a.stream>>>(p);
+            return hipGetLastError();
+        }
         grid.x = (unsigned)(plan.head + plan.tail * plan.sub);
         if constexpr (RM == 4) {
             if (has_lone_form<WS, RM, HIGH>() && grid.x <= (unsigned)kCus)
@@ -665,6 +690,7 @@ static TailPlan tail_plan_for(const SpmmArgs& a, bool have_scratch)
     none.separate = false;
     none.sub = 1;
     none.fused = false;
+    none.along_k = false;
     if (a.split_k != 1 || NMSPMM_RM_TALL != 8)
         return none;
     TailPlan t = plan_tail(a.M, a.N, a.W / a.kept, a.kept, 128 / a.Ns);

@@ -281,13 +281,13 @@ def test_leftover_tiles_in_a_launch_of_their_own(oracle, M, N, K, n, m, Ns):
     check_every_tile_once(oracle, M, N, K, n, m, Ns)
 
 
-@pytest.mark.parametrize("M,N,K,n,m", [(1024, 5120, 256, 2, 4), (2048, 5120, 512, 1, 8), (300, 2048, 256, 2, 8),
+@pytest.mark.parametrize("M,N,K,n,m", [(1024, 5120, 128, 2, 4), (2048, 5120, 512, 1, 8), (300, 2048, 256, 2, 8),
                                        (2048, 6656, 512, 1, 8), (1000, 6656, 256, 3, 8), (1024, 5120, 128, 32, 32)])
 @pytest.mark.parametrize("Ns", [128, 64, 32])
 def test_last_layer_of_a_small_launch_in_pieces(oracle, M, N, K, n, m, Ns):
     """Fewer tiles than the GPU holds at once: the tiles beyond the last multiple of 256 are
     computed as two 64-row pieces each by the workgroups at the end of the same launch when they
-    cover at most half of the CUs (320 tiles of 128 rows: 64 in pieces; 640: 128; 48 with a ragged
+    cover at most half of the CUs (320 tiles of 128 rows and four windows: 64 in pieces; 640: 128; 48 with a ragged
     row count: all of them, and the pieces beyond the last row store nothing; 832: 64 after three
     whole layers) and whole otherwise (416: 160 leftovers).  Every tile exactly once, for every
     width of the column blocks."""
@@ -336,6 +336,18 @@ def test_split_slices_of_unequal_length_two_windows_ahead(oracle, M, n, m, split
     got, fam = run_gpu(oracle, d, 128, split_k=split_k)
     assert fam == "mfma"
     check(oracle, d, got)
+
+
+@pytest.mark.parametrize("M,N,K,n,m", [(1024, 5120, 256, 2, 4), (1152, 4096, 1024, 2, 8), (1000, 4608, 352, 3, 8), (1280, 4096, 704, 1, 8),
+                                       (1024, 4608, 288, 32, 32)])
+@pytest.mark.parametrize("Ns", [128, 64, 32])
+def test_last_layer_of_a_small_launch_with_the_reduction_shared(oracle, M, N, K, n, m, Ns):
+    """257 to 320 tiles of 128 rows and at least eight windows: the tiles beyond the first 256 are
+    computed by four workgroups each at the end of the same launch, 128 rows of one 32-column
+    vector with the reduction shared between the four waves (eight, nine, eleven and sixteen
+    windows; a ragged row count).  Every tile exactly once, for every width of the column blocks
+    (the whole tile is then 128 x 128, 256 x 64 or 512 x 32)."""
+    check_every_tile_once(oracle, M, N, K, n, m, Ns)
 
 
 def test_llm_layer_shape_2of8(oracle):
