@@ -10,12 +10,17 @@
 //   * the three preprocessing calls take HOST pointers and work in place;
 //   * the eight launchers take DEVICE pointers, enqueue on the default stream and return at once;
 //   * a launcher given a sparsity of the other family prints "Not support! ..." and does nothing;
-//     a sparsity outside {0, 0.5, 0.625, 0.75, 0.875} does nothing.
-// Difference: with SPLIT_K > 1 the result overwrites C (workspace reduction) instead of being
-// atomically added to a caller-zeroed C; callers that zero C first see the same values.
+//     a sparsity outside {0, 0.5, 0.625, 0.75, 0.875} does nothing;
+//   * SPLIT_K == 1 overwrites C, SPLIT_K > 1 adds the product to what C holds (the reference
+//     kernels' atomicAdd epilogue, src/kernel_64x128_8x8.cu:235-251): zero C before a split call.
+//     Here the slices are summed in a fixed order through a workspace, so the result is
+//     reproducible bit for bit.
 #ifndef NM_SPMM_DROP_IN_H
 #define NM_SPMM_DROP_IN_H
 
+// The reference header brings the GPU runtime API to its includers (include/NM-SpMM.h:4-5 include
+// <cuda.h> and <cuda_runtime.h>); this one brings HIP's, so a driver needs no include of its own.
+#include <hip/hip_runtime.h>
 #include <iostream>
 
 // Adjacent columns of B that share one index pattern (reference include/NM-SpMM.h:8).

@@ -141,8 +141,9 @@ size_t nmspmm_tail_workspace_bytes(int M, int N, int W, int kept);
 /* General entry point: C = A . B for one (window, kept, vec_len, Ns) geometry.
  * column_info == NULL selects the low-sparsity layout (all window rows staged), non-NULL the
  * high-sparsity layout (only the rows column_info lists are staged, D holds ranks).
- * split_k > 1 requires `workspace` of at least nmspmm_workspace_bytes(); unlike the reference's
- * atomicAdd reduction (include/ptx.h:34-40) C is overwritten, not accumulated into.  With
+ * split_k > 1 requires `workspace` of at least nmspmm_workspace_bytes(); C is overwritten
+ * whatever the split (the reference's atomicAdd reduction, include/ptx.h:34-40, adds to C when
+ * SPLIT_K > 1: nmspmm_spmm_ex with NMSPMM_ACCUMULATE does that).  With
  * split_k == 1 the workspace is optional: NULL, or nmspmm_tail_workspace_bytes() bytes (16-byte
  * aligned) that enable the tail split; a smaller one is ignored.
  * Requirements: N % Ns == 0, Ns % vec_len == 0, W % kept == 0, 1 <= split_k <= W / kept,
@@ -150,6 +151,17 @@ size_t nmspmm_tail_workspace_bytes(int M, int N, int W, int kept);
 int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t* column_info,
                 float* C, int M, int N, int K, int W, int window, int kept, int vec_len, int Ns,
                 int split_k, void* workspace, size_t workspace_bytes, void* stream);
+
+/* nmspmm_spmm with flags.  NMSPMM_ACCUMULATE: with split_k > 1 the sum of the reduction slices is
+ * added to what C holds, C += A . B, exactly what the reference kernels do with their atomicAdd
+ * epilogue (src/kernel_64x128_8x8.cu:235-242; deterministic here: C, then the slices in order);
+ * with split_k == 1 C is overwritten, as in the reference (:243-251).  Any other flag bit:
+ * NMSPMM_ERR_BAD_SHAPE. */
+#define NMSPMM_ACCUMULATE 1u
+int nmspmm_spmm_ex(const float* A, const float* B, const int32_t* D, const int32_t* column_info,
+                   float* C, int M, int N, int K, int W, int window, int kept, int vec_len, int Ns,
+                   int split_k, void* workspace, size_t workspace_bytes, unsigned flags,
+                   void* stream);
 
 /* Row-major A (M x K, K contiguous per row: activations as a model produces them).  No
  * counterpart: the reference kernels demand column-major A (reference
@@ -173,9 +185,14 @@ int nmspmm_spmm_rowmajor(const float* A_rowmajor, const float* B, const int32_t*
  * (reference include/NM-SpMM.h:14,17,20,23) and ..._high_sparsity (:15,18,21,24): `tile` is the
  * nmspmm_tile of the named entry point, `sparsity` selects the geometry as
  * nmspmm_pattern_from_sparsity does, vec_len is 32.  A sparsity that belongs to the other path
- * returns NMSPMM_ERR_WRONG_PATH (the reference prints "Not support!" there).  When split_k > 1
- * the library uses a per-device workspace that it grows on demand and keeps until
- * nmspmm_release(); calls sharing a device must then be issued on one stream at a time. */
+ * returns NMSPMM_ERR_WRONG_PATH (the reference prints "Not support!" there).  As in the reference,
+ * split_k == 1 overwrites C and split_k > 1 adds the product to what C holds (NMSPMM_ACCUMULATE),
+ * so a caller zeroes C before a split call.
+ * Shared state: none when split_k == 1 (any number of streams and threads, and the call can be
+ * recorded into a HIP graph).  When split_k > 1 the slices go to a per-device workspace that the
+ * library grows on demand (hipMalloc, so not under graph capture unless an earlier call has
+ * already grown it to the size) and keeps until nmspmm_release(); split calls that share a device
+ * must be issued on one stream at a time, or they overwrite each other's slices. */
 int nmspmm_gemm_low_sparsity(int tile, const float* A, const float* B, const int32_t* D, float* C,
                              int M, int N, int K, int W, float sparsity, int split_k, void* stream);
 int nmspmm_gemm_high_sparsity(int tile, const float* A, const float* B, const int32_t* D,

@@ -19,6 +19,7 @@ STATUS_NAMES = {
     8: "NMSPMM_ERR_ALIGNMENT",
 }
 TILE_SMALL, TILE_MEDIUM, TILE_LARGE, TILE_HUGE = 32, 64, 64, 128
+ACCUMULATE = 1  # flag of spmm_ex: with split_k > 1 the product is added to what C holds
 
 
 class NmSpmmError(RuntimeError):
@@ -60,6 +61,7 @@ def lib():
         L.nmspmm_workspace_bytes.restype = c_size_t
         L.nmspmm_workspace_bytes.argtypes = [c_int] * 3
         L.nmspmm_spmm.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, c_void_p]
+        L.nmspmm_spmm_ex.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, ctypes.c_uint, c_void_p]
         L.nmspmm_gemm_low_sparsity.argtypes = [c_int] + [c_void_p] * 4 + [c_int] * 4 + [c_float, c_int, c_void_p]
         L.nmspmm_gemm_high_sparsity.argtypes = [c_int] + [c_void_p] * 5 + [c_int] * 4 + [c_float, c_int, c_void_p]
         L.nmspmm_transpose_device.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p]
@@ -156,6 +158,13 @@ def spmm(A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len=32, Ns=128, split_
     _check("nmspmm_spmm",
            lib().nmspmm_spmm(_ptr(A), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(C), M, N, K, W, window, kept, vec_len,
                              Ns, split_k, _ptr(workspace), ws_bytes, _stream()))
+
+
+def spmm_ex(A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len=32, Ns=128, split_k=1, workspace=None, flags=0):
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _check("nmspmm_spmm_ex",
+           lib().nmspmm_spmm_ex(_ptr(A), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(C), M, N, K, W, window, kept, vec_len,
+                                Ns, split_k, _ptr(workspace), ws_bytes, flags, _stream()))
 
 
 def gemm_low_sparsity(tile, A, B, D, C, M, N, K, W, sparsity, split_k=1):

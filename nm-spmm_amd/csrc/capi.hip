@@ -5,6 +5,7 @@
 
 #include <cmath>
 #include <mutex>
+#include <vector>
 
 using namespace nmspmm;
 
@@ -15,6 +16,7 @@ thread_local const char* g_last_kernel = "none";
 struct Workspace {
     void* ptr = nullptr;
     size_t bytes = 0;
+    std::vector<void*> retired;  // outgrown buffers: launches already enqueued may still use them
 };
 constexpr int kMaxDevices = 64;
 Workspace g_workspace[kMaxDevices];
@@ -31,7 +33,10 @@ int check_index_shape(int W, int Q)
     return (W > 0 && Q > 0) ? NMSPMM_OK : NMSPMM_ERR_BAD_SHAPE;
 }
 
-// Grows (never shrinks) the calling device's cached workspace.
+// Grows (never shrinks) the calling device's cached workspace.  An outgrown buffer is kept until
+// nmspmm_release(): another thread may have taken its address a moment ago and not launched yet,
+// and launches already enqueued read it, so it is neither freed nor waited for here.  Growth is
+// at least geometric, which bounds what the retired buffers hold to the size of the live one.
 int cached_workspace(size_t bytes, void** out)
 {
     int dev = 0;
@@ -40,18 +45,19 @@ int cached_workspace(size_t bytes, void** out)
     std::lock_guard<std::mutex> lock(g_workspace_mutex);
     Workspace& ws = g_workspace[dev];
     if (ws.bytes < bytes) {
-        if (ws.ptr) {
-            if (hipDeviceSynchronize() != hipSuccess)
+        const size_t want = bytes > 2 * ws.bytes ? bytes : 2 * ws.bytes;
+        void* grown = nullptr;
+        if (hipMalloc(&grown, want) != hipSuccess) {
+            (void)hipGetLastError();
+            if (want == bytes || hipMalloc(&grown, bytes) != hipSuccess)
                 return NMSPMM_ERR_HIP;
-            (void)hipFree(ws.ptr);
-            ws.ptr = nullptr;
-            ws.bytes = 0;
+            ws.bytes = bytes;
+        } else {
+            ws.bytes = want;
         }
-        if (hipMalloc(&ws.ptr, bytes) != hipSuccess) {
-            ws.ptr = nullptr;
-            return NMSPMM_ERR_HIP;
-        }
-        ws.bytes = bytes;
+        if (ws.ptr)
+            ws.retired.push_back(ws.ptr);
+        ws.ptr = grown;
     }
     *out = ws.ptr;
     return NMSPMM_OK;
@@ -349,8 +355,11 @@ size_t nmspmm_workspace_bytes(int M, int N, int split_k)
 constexpr int kNotTaken = -1000;
 static int spmm_impl(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C, int M,
                      int N, int K, int W, int window, int kept, int vec_len, int Ns, int split_k, void* workspace,
-                     size_t workspace_bytes, void* stream, int lda, bool dry_run, int* lda_out, bool a_rowmajor = false)
+                     size_t workspace_bytes, void* stream, int lda, bool dry_run, int* lda_out, bool a_rowmajor = false,
+                     unsigned flags = 0)
 {
+    if (flags & ~(unsigned)NMSPMM_ACCUMULATE)
+        return NMSPMM_ERR_BAD_SHAPE;
     if (!A || !B || !D || !C)
         return NMSPMM_ERR_NULL_POINTER;
     if (M <= 0 || N <= 0 || K <= 0 || W <= 0)
@@ -389,6 +398,7 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     a.vec_len = vec_len;
     a.Ns = Ns;
     a.split_k = split_k;
+    a.accumulate = (flags & NMSPMM_ACCUMULATE) != 0 && split_k > 1;
     // without a split the workspace, if any, serves the tail split of the tile kernel
     const bool scratch = split_k == 1 && workspace != nullptr && aligned16(workspace);
     a.tail_ws = scratch ? (float*)workspace : nullptr;
@@ -437,7 +447,7 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     if (e != hipSuccess)
         return NMSPMM_ERR_HIP;
     if (split_k > 1) {
-        e = launch_splitk_reduce(a.partial, C, (size_t)M * N, a.slice_stride, split_k, a.stream);
+        e = launch_splitk_reduce(a.partial, C, (size_t)M * N, a.slice_stride, split_k, a.accumulate, a.stream);
         if (e != hipSuccess)
             return NMSPMM_ERR_HIP;
     }
@@ -509,9 +519,18 @@ int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t*
                      workspace_bytes, stream, M, false, nullptr);
 }
 
+int nmspmm_spmm_ex(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C, int M,
+                   int N, int K, int W, int window, int kept, int vec_len, int Ns, int split_k, void* workspace,
+                   size_t workspace_bytes, unsigned flags, void* stream)
+{
+    return spmm_impl(A, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k, workspace,
+                     workspace_bytes, stream, M, false, nullptr, false, flags);
+}
+
+// `flags`: NMSPMM_ACCUMULATE for the reference launchers' replacements, whose SPLIT_K > 1 adds to C.
 static int named_gemm(int want_high, int tile, const float* A, const float* B, const int32_t* D,
                       const int32_t* column_info, float* C, int M, int N, int K, int W, float sparsity,
-                      int split_k, void* stream)
+                      int split_k, unsigned flags, void* stream)
 {
     int window, kept, is_high;
     const int st = nmspmm_pattern_from_sparsity(sparsity, &window, &kept, &is_high);
@@ -529,29 +548,31 @@ static int named_gemm(int want_high, int tile, const float* A, const float* B, c
         return NMSPMM_ERR_BAD_SHAPE;
     if (split_k < 1 || split_k > W / kept)
         return NMSPMM_ERR_BAD_SPLIT;
+    // Only a split reduction uses the library's per-device workspace.  (The optional scratch that
+    // cuts a few leftover tiles along K, nmspmm_tail_workspace_bytes, is for callers of nmspmm_spmm
+    // who own it: unsplit calls here touch no shared memory and may run on any number of streams.)
     void* ws = nullptr;
-    size_t ws_bytes = split_k > 1 ? nmspmm_workspace_bytes(M, N, split_k)
-                                  : (tile == 128 ? nmspmm_tail_workspace_bytes(M, N, W, kept) : 0);
+    const size_t ws_bytes = nmspmm_workspace_bytes(M, N, split_k);
     if (ws_bytes > 0) {
         const int rc = cached_workspace(ws_bytes, &ws);
         if (rc != NMSPMM_OK)
             return rc;
     }
-    return nmspmm_spmm(A, B, D, want_high ? column_info : nullptr, C, M, N, K, W, window, kept, 32, tile, split_k,
-                       ws, ws_bytes, stream);
+    return nmspmm_spmm_ex(A, B, D, want_high ? column_info : nullptr, C, M, N, K, W, window, kept, 32, tile,
+                          split_k, ws, ws_bytes, flags, stream);
 }
 
 int nmspmm_gemm_low_sparsity(int tile, const float* A, const float* B, const int32_t* D, float* C, int M, int N,
                              int K, int W, float sparsity, int split_k, void* stream)
 {
-    return named_gemm(0, tile, A, B, D, nullptr, C, M, N, K, W, sparsity, split_k, stream);
+    return named_gemm(0, tile, A, B, D, nullptr, C, M, N, K, W, sparsity, split_k, NMSPMM_ACCUMULATE, stream);
 }
 
 int nmspmm_gemm_high_sparsity(int tile, const float* A, const float* B, const int32_t* D,
                               const int32_t* column_info, float* C, int M, int N, int K, int W, float sparsity,
                               int split_k, void* stream)
 {
-    return named_gemm(1, tile, A, B, D, column_info, C, M, N, K, W, sparsity, split_k, stream);
+    return named_gemm(1, tile, A, B, D, column_info, C, M, N, K, W, sparsity, split_k, NMSPMM_ACCUMULATE, stream);
 }
 
 int nmspmm_suggest_split_k(int M, int N, int W, int kept)
@@ -599,7 +620,7 @@ int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int
     const int split_k = nmspmm_suggest_split_k(M, N, W, kept);
     if (split_k < 1)
         return NMSPMM_ERR_BAD_SHAPE;
-    return named_gemm(is_high, NMSPMM_TILE_HUGE, A, B, D, column_info, C, M, N, K, W, sparsity, split_k, stream);
+    return named_gemm(is_high, NMSPMM_TILE_HUGE, A, B, D, column_info, C, M, N, K, W, sparsity, split_k, 0, stream);
 }
 
 int nmspmm_release(void)
@@ -609,12 +630,20 @@ int nmspmm_release(void)
     int prev = 0;
     const bool have_dev = hipGetDevice(&prev) == hipSuccess;
     for (int d = 0; d < kMaxDevices; ++d) {
-        if (!g_workspace[d].ptr)
+        Workspace& ws = g_workspace[d];
+        if (!ws.ptr && ws.retired.empty())
             continue;
-        if (hipSetDevice(d) != hipSuccess || hipFree(g_workspace[d].ptr) != hipSuccess)
+        // hipFree waits for the work enqueued on the device before it releases the memory
+        if (hipSetDevice(d) != hipSuccess)
             rc = NMSPMM_ERR_HIP;
-        g_workspace[d].ptr = nullptr;
-        g_workspace[d].bytes = 0;
+        if (ws.ptr && hipFree(ws.ptr) != hipSuccess)
+            rc = NMSPMM_ERR_HIP;
+        for (void* old : ws.retired)
+            if (hipFree(old) != hipSuccess)
+                rc = NMSPMM_ERR_HIP;
+        ws.retired.clear();
+        ws.ptr = nullptr;
+        ws.bytes = 0;
     }
     if (have_dev)
         (void)hipSetDevice(prev);

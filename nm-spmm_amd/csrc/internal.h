@@ -24,6 +24,8 @@ struct SpmmArgs {
                            // the one-block decode kernels only)
     int window, kept, vec_len, Ns;
     int split_k;
+    bool accumulate;       // split_k > 1 only: the sum of the slices is added to what C holds (the
+                           // reference's atomicAdd reduction, include/ptx.h:34-40) instead of replacing it
     float* tail_ws;        // optional scratch for splitting the tiles of a ragged last round (split_k == 1)
     size_t tail_ws_bytes;
     hipStream_t stream;
@@ -364,9 +366,10 @@ hipError_t launch_skinny(const SpmmArgs& a);
 bool simt_supported(const SpmmArgs& a);
 hipError_t launch_simt(const SpmmArgs& a);
 
-// Sums split_k slices of `partial` into C in slice order (spmm_simt.hip).
+// Sums split_k slices of `partial` in slice order (spmm_simt.hip) and stores the sum to C, or,
+// with `accumulate`, adds it to what C holds.
 hipError_t launch_splitk_reduce(const float* partial, float* C, size_t elems, size_t slice_stride,
-                                int split_k, hipStream_t stream);
+                                int split_k, bool accumulate, hipStream_t stream);
 
 // Index preprocessing kernels (preprocess.hip).
 hipError_t launch_trans_index(int32_t* dDT, int W, int Q, int pN, int pM, hipStream_t stream);

@@ -97,7 +97,10 @@ hipError_t launch_simt(const SpmmArgs& a)
     return hipGetLastError();
 }
 
-// C[e] = partial[0][e] + partial[1][e] + ... in slice order (deterministic, unlike atomics).
+// C[e] = partial[0][e] + partial[1][e] + ... in slice order (deterministic, unlike atomics); with
+// ACC the chain starts from what C[e] holds, as the reference's atomicAdd reduction into the
+// caller's C does (include/ptx.h:34-40, src/kernel_64x128_8x8.cu:235-242).
+template <bool ACC>
 __global__ void __launch_bounds__(256)
 splitk_reduce_kernel(const float* __restrict__ partial, float* __restrict__ C, size_t elems,
                      size_t slice_stride, int split_k)
@@ -106,6 +109,13 @@ splitk_reduce_kernel(const float* __restrict__ partial, float* __restrict__ C, s
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n4; e += stride) {
         float4 s = reinterpret_cast<const float4*>(partial)[e];
+        if (ACC) {
+            const float4 c = reinterpret_cast<const float4*>(C)[e];
+            s.x = c.x + s.x;
+            s.y = c.y + s.y;
+            s.z = c.z + s.z;
+            s.w = c.w + s.w;
+        }
         for (int z = 1; z < split_k; ++z) {
             const float4 v = reinterpret_cast<const float4*>(partial + (size_t)z * slice_stride)[e];
             s.x += v.x;
@@ -118,7 +128,7 @@ splitk_reduce_kernel(const float* __restrict__ partial, float* __restrict__ C, s
     // tail (elems not a multiple of 4)
     if (blockIdx.x == 0 && threadIdx.x < (elems & 3)) {
         const size_t e = n4 * 4 + threadIdx.x;
-        float s = partial[e];
+        float s = ACC ? C[e] + partial[e] : partial[e];
         for (int z = 1; z < split_k; ++z)
             s += partial[(size_t)z * slice_stride + e];
         C[e] = s;
@@ -126,7 +136,7 @@ splitk_reduce_kernel(const float* __restrict__ partial, float* __restrict__ C, s
 }
 
 hipError_t launch_splitk_reduce(const float* partial, float* C, size_t elems, size_t slice_stride,
-                                int split_k, hipStream_t stream)
+                                int split_k, bool accumulate, hipStream_t stream)
 {
     const size_t n4 = elems / 4;
     size_t blocks = (n4 + 255) / 256;
@@ -134,8 +144,12 @@ hipError_t launch_splitk_reduce(const float* partial, float* C, size_t elems, si
         blocks = 1;
     if (blocks > 256 * 16)
         blocks = 256 * 16;
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, partial, C,
-                       elems, slice_stride, split_k);
+    if (accumulate)
+        hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, partial, C,
+                           elems, slice_stride, split_k);
+    else
+        hipLaunchKernelGGL(splitk_reduce_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, partial, C,
+                           elems, slice_stride, split_k);
     return hipGetLastError();
 }
 

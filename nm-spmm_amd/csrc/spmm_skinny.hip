@@ -34,6 +34,7 @@ struct SkinnyParams {
     // element (i, k) of A lies i * a_row_stride + k * a_k_stride bytes into its a_bytes bytes:
     // (4, 4 * lda) for the column-major operand, (4 * lda, 4) for a row-major one (up to 32 rows)
     uint32_t a_row_stride, a_k_stride, a_bytes;
+    int accumulate;  // the result is added to what C holds instead of replacing it
 };
 
 __device__ inline __amdgpu_buffer_rsrc_t sk_rsrc(const void* base, uint32_t bytes)
@@ -235,8 +236,10 @@ spmm_skinny_kernel(const SkinnyParams p)
             for (int x = 1; x < kSkinnyWaves; ++x)
                 s += red[x][v][lane];
             const int row = RB * (8 * (v / 4) + 4 * h + (v % 4)) + b;
-            if (row < M)
-                p.C[(size_t)row * N + (size_t)vec_g * 32 + j] = s;
+            if (row < M) {
+                float* const dst = p.C + (size_t)row * N + (size_t)vec_g * 32 + j;
+                *dst = p.accumulate ? *dst + s : s;
+            }
         }
     }
 }
@@ -380,8 +383,10 @@ spmm_skinny16_kernel(const SkinnyParams p)
         for (int y = 1; y < kSkinnyWaves; ++y)
             s += red[y][x][lane];
         const int row = 4 * kq + (x % 4);
-        if (row < M)
-            p.C[(size_t)row * N + (size_t)vec_g * 32 + 2 * jl + x / 4] = s;
+        if (row < M) {
+            float* const dst = p.C + (size_t)row * N + (size_t)vec_g * 32 + 2 * jl + x / 4;
+            *dst = p.accumulate ? *dst + s : s;
+        }
     }
 }
 
@@ -403,6 +408,7 @@ static hipError_t launch_qs(const SpmmArgs& a)
     p.a_row_stride = (uint32_t)(a.a_rowmajor ? a.lda * sizeof(float) : sizeof(float));
     p.a_k_stride = (uint32_t)(a.a_rowmajor ? sizeof(float) : a.lda * sizeof(float));
     p.a_bytes = (uint32_t)((size_t)(a.a_rowmajor ? a.M : a.K) * a.lda * sizeof(float));
+    p.accumulate = (a.accumulate && a.split_k > 1) ? 1 : 0;
     const dim3 grid(a.N / 32), block(64 * kSkinnyWaves);
     switch (a.Ns) {
     case 128: spmm_skinny_kernel<KS, WS, 4, HIGH, RB, U><<<grid, block, 0, a.stream>>>(p); break;
@@ -431,6 +437,7 @@ static hipError_t launch_qs16(const SpmmArgs& a)
     p.a_row_stride = (uint32_t)(a.a_rowmajor ? a.lda * sizeof(float) : sizeof(float));
     p.a_k_stride = (uint32_t)(a.a_rowmajor ? sizeof(float) : a.lda * sizeof(float));
     p.a_bytes = (uint32_t)((size_t)(a.a_rowmajor ? a.M : a.K) * a.lda * sizeof(float));
+    p.accumulate = (a.accumulate && a.split_k > 1) ? 1 : 0;
     const dim3 grid(a.N / 32), block(64 * kSkinnyWaves);
     switch (a.Ns) {
     case 128: spmm_skinny16_kernel<KS, WS, 4, HIGH, U><<<grid, block, 0, a.stream>>>(p); break;

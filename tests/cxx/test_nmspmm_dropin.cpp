@@ -3,12 +3,13 @@
 // preprocessing in place, copy, launch by tile name), one run per tile whose divisibility holds.
 // Differences: operands are seeded and signed, the CPU check is the checker library
 // (oracle/libnm_oracle.so), the comparison is the scaled max error bound 1e-4, and the exit code
-// reports failure.
+// reports failure.  C does not start from zero: with SPLIT_K > 1 the launchers add to what C holds
+// (reference src/kernel_64x128_8x8.cu:235-242), so C starts from seeded values on both sides; with
+// SPLIT_K == 1 they overwrite (:243-251), so the device C starts from NaNs.
 //
-//   test_nmspmm_dropin M N K [pruning_M sparsity [SPLIT_K]]
-#include "NM-SpMM.h"
-
-#include <hip/hip_runtime.h>
+//   test_nmspmm_dropin M N K [pruning_M sparsity [SPLIT_K [warm_up iter]]]
+// (the argument forms of the reference driver, tests/test_nmspmm.cu:169-192)
+#include "NM-SpMM.h"  // brings the HIP runtime API, as the reference header brings CUDA's
 
 #include <algorithm>
 #include <cmath>
@@ -41,7 +42,7 @@ static float next_unit() { return (float)(next_u32() & 0xFFFFFF) / 8388608.0f - 
     } while (0)
 
 static bool run_tile(const char* name, LowFn low, HighFn high, int Ns, int M, int N, int K, int pruning_M,
-                     float sparsity, int split_k)
+                     float sparsity, int split_k, int warm_up, int iters)
 {
     const bool is_high = std::fabs(sparsity - 0.75f) < 1e-6f || std::fabs(sparsity - 0.875f) < 1e-6f;
     const int W = (int)(K * (1.0f - sparsity));
@@ -88,7 +89,12 @@ static bool run_tile(const char* name, LowFn low, HighFn high, int Ns, int M, in
     HIP_OK(hipMalloc(&dci, ci_ints * 4));
     HIP_OK(hipMemcpy(dA, A.data(), A.size() * 4, hipMemcpyHostToDevice));
     HIP_OK(hipMemcpy(dB, BT.data(), BT.size() * 4, hipMemcpyHostToDevice));
-    HIP_OK(hipMemset(dC, 0, Cgpu.size() * 4));
+    if (split_k > 1) {
+        for (float& x : Cref) x = next_unit();
+        HIP_OK(hipMemcpy(dC, Cref.data(), Cgpu.size() * 4, hipMemcpyHostToDevice));
+    } else {
+        HIP_OK(hipMemset(dC, 0xFF, Cgpu.size() * 4));
+    }
     HIP_OK(hipMemcpy(dD, DT.data(), DT.size() * 4, hipMemcpyHostToDevice));
     HIP_OK(hipMemcpy(dci, column_info.data(), ci_ints * 4, hipMemcpyHostToDevice));
 
@@ -115,7 +121,12 @@ static bool run_tile(const char* name, LowFn low, HighFn high, int Ns, int M, in
     hipEvent_t e0, e1;
     HIP_OK(hipEventCreate(&e0));
     HIP_OK(hipEventCreate(&e1));
-    const int iters = 20;
+    for (int i = 0; i < warm_up; ++i) {
+        if (!is_high)
+            low(dA, dB, dD, dC, M, N, K, W, sparsity, split_k);
+        else
+            high(dA, dB, dD, dci, dC, M, N, K, W, sparsity, split_k);
+    }
     HIP_OK(hipEventRecord(e0));
     for (int i = 0; i < iters; ++i) {
         if (!is_high)
@@ -151,15 +162,17 @@ static void auto_high(float* A, float* B, int* D, int* column_info, float* C, in
 
 int main(int argc, char** argv)
 {
-    int M = 512, N = 512, K = 512, pruning_M = 32, split_k = 1;
+    int M = 512, N = 512, K = 512, pruning_M = 32, split_k = 1, warm_up = 5, iters = 20;
     float sparsity = 0.5f;
-    if (argc != 1 && argc != 4 && argc != 6 && argc != 7) {
-        std::printf("Usage: %s M N K [pruning_M sparsity [SPLIT_K]]\n", argv[0]);
+    if (argc != 1 && argc != 4 && argc != 6 && argc != 7 && argc != 9) {
+        std::printf("Usage: %s M N K [pruning_M sparsity [SPLIT_K [warm_up iter]]]\n", argv[0]);
         return -1;
     }
     if (argc >= 4) { M = std::atoi(argv[1]); N = std::atoi(argv[2]); K = std::atoi(argv[3]); }
     if (argc >= 6) { pruning_M = std::atoi(argv[4]); sparsity = (float)std::atof(argv[5]); }
     if (argc >= 7) split_k = std::atoi(argv[6]);
+    if (argc >= 9) { warm_up = std::atoi(argv[7]); iters = std::atoi(argv[8]); }
+    if (warm_up < 0 || iters < 1) { std::printf("warm_up >= 0 and iter >= 1 expected\n"); return -1; }
     std::printf("M = %d, N = %d, K = %d, pruning_M = %d, sparsity = %f, SPLIT_K = %d\n", M, N, K, pruning_M, sparsity, split_k);
     const float allowed[] = {0.0f, 0.5f, 0.625f, 0.75f, 0.875f};
     bool known = false;
@@ -168,17 +181,18 @@ int main(int argc, char** argv)
     if (K % pruning_M != 0) { std::printf("K is not an integer multiple of pruning_M!!!\n"); return -3; }
 
     int failures = 0, runs = 0;
-    struct Tile { const char* name; LowFn low; HighFn high; int Ns; } tiles[] = {
-        {"small", &nmGEMM_small_matrices_low_sparsity, &nmGEMM_small_matrices_high_sparsity, 32},
-        {"medium", &nmGEMM_medium_matrices_low_sparsity, &nmGEMM_medium_matrices_high_sparsity, 64},
-        {"large", &nmGEMM_large_matrices_low_sparsity, &nmGEMM_large_matrices_high_sparsity, 64},
-        {"huge", &nmGEMM_huge_matrices_low_sparsity, &nmGEMM_huge_matrices_high_sparsity, 128},
-        {"nmGEMM (split chosen by the library)", &auto_low, &auto_high, 128},
+    // nmGEMM picks the split itself and always overwrites C: it is checked as a SPLIT_K == 1 call
+    struct Tile { const char* name; LowFn low; HighFn high; int Ns; bool takes_split; } tiles[] = {
+        {"small", &nmGEMM_small_matrices_low_sparsity, &nmGEMM_small_matrices_high_sparsity, 32, true},
+        {"medium", &nmGEMM_medium_matrices_low_sparsity, &nmGEMM_medium_matrices_high_sparsity, 64, true},
+        {"large", &nmGEMM_large_matrices_low_sparsity, &nmGEMM_large_matrices_high_sparsity, 64, true},
+        {"huge", &nmGEMM_huge_matrices_low_sparsity, &nmGEMM_huge_matrices_high_sparsity, 128, true},
+        {"nmGEMM (split chosen by the library)", &auto_low, &auto_high, 128, false},
     };
     for (const Tile& t : tiles) {
         if (N % t.Ns != 0) continue;
         ++runs;
-        if (!run_tile(t.name, t.low, t.high, t.Ns, M, N, K, pruning_M, sparsity, split_k)) ++failures;
+        if (!run_tile(t.name, t.low, t.high, t.Ns, M, N, K, pruning_M, sparsity, t.takes_split ? split_k : 1, warm_up, iters)) ++failures;
     }
     std::printf("\n%d tile runs, %d failures\n", runs, failures);
     return failures == 0 && runs > 0 ? 0 : 1;

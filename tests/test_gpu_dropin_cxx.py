@@ -20,6 +20,8 @@ BIN = os.path.join(ROOT, "tests", "cxx", "test_nmspmm_dropin")
     ["256", "256", "512", "32", "0.75"],
     ["128", "256", "512", "32", "0.875", "4"],
     ["16", "256", "512", "32", "0.875"],
+    ["16", "256", "512", "32", "0.75", "4"],           # decode-sized rows, split call: adds to C
+    ["512", "512", "1024", "32", "0.5", "4", "2", "3"],  # the reference driver's nine-argument form
 ], ids=" ".join)
 def test_reference_style_driver(args):
     assert os.path.exists(BIN), "build the driver first: make -C tests/cxx"

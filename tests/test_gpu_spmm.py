@@ -100,6 +100,58 @@ def test_split_k_through_workspace(oracle, split_k, n, m, Ns):
     assert scaled_max_error(got, one) <= REL_TOL
 
 
+@pytest.mark.parametrize("split_k", [1, 2, 4])
+@pytest.mark.parametrize("M,N,K,n,m,family", [(160, 256, 1280, 2, 4, "mfma"), (256, 512, 1024, 1, 8, "mfma"),
+                                             (132, 256, 768, 3, 8, "mfma"), (16, 256, 1024, 2, 8, "skinny"),
+                                             (32, 512, 1024, 1, 8, "skinny"), (64, 8192, 512, 1, 8, "skinny"),
+                                             (7, 256, 1152, 2, 4, "skinny")])
+def test_split_k_adds_to_c_like_the_reference(oracle, M, N, K, n, m, family, split_k):
+    """The reference kernels store with SPLIT_K == 1 and atomicAdd into the caller's C with
+    SPLIT_K > 1 (src/kernel_64x128_8x8.cu:235-251).  With NMSPMM_ACCUMULATE, and through the named
+    launchers, a split call on a non-zero C equals the checker's accumulate-into-C result, and an
+    unsplit call overwrites; without the flag every call overwrites."""
+    d = datagen.init_data(M, N, K, n, m, seed=7 * M + split_k)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    rng = np.random.default_rng(M + split_k)
+    C0 = rng.uniform(-4.0, 4.0, (M, N)).astype(np.float32)
+    A, B, Dd = dev(d["A_km"]), dev(d["BT"]), dev(D)
+    ci = None if cinfo is None else dev(cinfo)
+    ws = None
+    if split_k > 1:
+        ws = torch.full((nmspmm.workspace_bytes(M, N, split_k) // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    args = (d["A_km"].reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), M, N, d["W"])
+    product = oracle.gemm_cpu(*args).reshape(M, N)
+    added = oracle.gemm_cpu(*args, C=C0.reshape(-1).copy()).reshape(M, N)
+    want = added if split_k > 1 else product
+    sparsity = 1.0 - n / m
+
+    C = dev(C0)
+    nmspmm.spmm_ex(A, B, Dd, ci, C, M, N, K, d["W"], window, kept, 32, 128, split_k, ws, nmspmm.ACCUMULATE)
+    torch.cuda.synchronize()
+    if M <= 32 or M > 128:  # between, the two kernels compete and the split decides
+        assert nmspmm.last_kernel() == family
+    assert scaled_max_error(C.cpu().numpy(), want) <= REL_TOL
+
+    C = dev(C0)
+    if cinfo is None:
+        nmspmm.gemm_low_sparsity(128, A, B, Dd, C, M, N, K, d["W"], sparsity, split_k)
+    else:
+        nmspmm.gemm_high_sparsity(128, A, B, Dd, ci, C, M, N, K, d["W"], sparsity, split_k)
+    torch.cuda.synchronize()
+    assert scaled_max_error(C.cpu().numpy(), want) <= REL_TOL
+
+    C = dev(C0)
+    nmspmm.spmm(A, B, Dd, ci, C, M, N, K, d["W"], window, kept, 32, 128, split_k, ws)
+    torch.cuda.synchronize()
+    assert scaled_max_error(C.cpu().numpy(), product) <= REL_TOL
+
+
+def test_unknown_flag_bits_are_rejected():
+    with pytest.raises(nmspmm.NmSpmmError, match="BAD_SHAPE"):
+        x = torch.zeros(64 * 64, dtype=torch.float32, device="cuda")
+        nmspmm.spmm_ex(x, x, x.int(), None, x, 32, 32, 32, 16, 32, 16, 32, 32, 1, None, 2)
+
+
 @pytest.mark.parametrize("M", [1, 2, 8, 13, 16, 30, 32])
 @pytest.mark.parametrize("n,m", [(1, 8), (2, 8), (2, 4), (3, 8), (32, 32)])
 @pytest.mark.parametrize("Ns", [128, 64, 32])
