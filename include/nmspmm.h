@@ -163,6 +163,22 @@ int nmspmm_spmm_ex(const float* A, const float* B, const int32_t* D, const int32
                    int split_k, void* workspace, size_t workspace_bytes, unsigned flags,
                    void* stream);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  nmspmm_spmm with the
+ * split-K slices in a fixed device-resident array of NMSPMM_NOALLOC_MAX_BYTES that belongs to the
+ * library (each GPU the library runs on holds one such array from the first use of the library on
+ * it until the process ends): no workspace argument, and no hipMalloc, hipFree or other
+ * allocating call on any path.  nmspmm_workspace_bytes(M, N, split_k) beyond that size:
+ * NMSPMM_ERR_WORKSPACE, nothing launched.  split_k == 1 uses no scratch at all.  C is
+ * overwritten; results are bit-identical to nmspmm_spmm with a caller-owned workspace.  All calls
+ * on a GPU share that GPU's array (the kernels overwrite every slice element they later read, so
+ * nothing needs clearing between calls): split calls that overlap in time on one GPU, from
+ * different streams or threads, race on it and must be serialised by the caller. */
+#define NMSPMM_NOALLOC_MAX_BYTES (32u << 20)
+int nmspmm_spmm_noalloc(const float* A, const float* B, const int32_t* D, const int32_t* column_info,
+                        float* C, int M, int N, int K, int W, int window, int kept, int vec_len,
+                        int Ns, int split_k, void* stream);
+
 /* Row-major A (M x K, K contiguous per row: activations as a model produces them).  No
  * counterpart: the reference kernels demand column-major A (reference
  * src/kernel_64x128_8x8.cu:15), i.e. a transpose before every layer.  nmspmm_transpose_device

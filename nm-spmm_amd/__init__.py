@@ -62,6 +62,7 @@ def lib():
         L.nmspmm_workspace_bytes.argtypes = [c_int] * 3
         L.nmspmm_spmm.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, c_void_p]
         L.nmspmm_spmm_ex.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, ctypes.c_uint, c_void_p]
+        L.nmspmm_spmm_noalloc.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p]
         L.nmspmm_gemm_low_sparsity.argtypes = [c_int] + [c_void_p] * 4 + [c_int] * 4 + [c_float, c_int, c_void_p]
         L.nmspmm_gemm_high_sparsity.argtypes = [c_int] + [c_void_p] * 5 + [c_int] * 4 + [c_float, c_int, c_void_p]
         L.nmspmm_transpose_device.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p]
@@ -165,6 +166,16 @@ def spmm_ex(A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len=32, Ns=128, spl
     _check("nmspmm_spmm_ex",
            lib().nmspmm_spmm_ex(_ptr(A), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(C), M, N, K, W, window, kept, vec_len,
                                 Ns, split_k, _ptr(workspace), ws_bytes, flags, _stream()))
+
+
+NOALLOC_MAX_BYTES = 32 << 20  # NMSPMM_NOALLOC_MAX_BYTES
+
+
+def spmm_noalloc(A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len=32, Ns=128, split_k=1):
+    """spmm with the split-K slices in the library's fixed device-resident scratch: allocates nothing."""
+    _check("nmspmm_spmm_noalloc",
+           lib().nmspmm_spmm_noalloc(_ptr(A), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(C), M, N, K, W, window, kept,
+                                     vec_len, Ns, split_k, _stream()))
 
 
 def gemm_low_sparsity(tile, A, B, D, C, M, N, K, W, sparsity, split_k=1):

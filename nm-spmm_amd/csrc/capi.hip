@@ -22,6 +22,32 @@ constexpr int kMaxDevices = 64;
 Workspace g_workspace[kMaxDevices];
 std::mutex g_workspace_mutex;
 
+// Split-K slices for nmspmm_spmm_noalloc: device memory that exists from the moment the code object
+// is loaded on a GPU until the process ends, one copy per GPU, so that entry point never allocates.
+// Host code must not use the array's name as an address (on the host it is only a handle):
+// noalloc_scratch() asks the runtime for the device address, once per device.
+static __device__ __align__(256) unsigned char scratch[NMSPMM_NOALLOC_MAX_BYTES];
+void* g_scratch_ptr[64] = {};
+std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device, or nullptr when the runtime cannot give it.
+void* noalloc_scratch()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        return nullptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 size_t slice_stride(int M, int N) { return (((size_t)M * N + 3) / 4) * 4; }
@@ -525,6 +551,29 @@ int nmspmm_spmm_ex(const float* A, const float* B, const int32_t* D, const int32
 {
     return spmm_impl(A, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k, workspace,
                      workspace_bytes, stream, M, false, nullptr, false, flags);
+}
+
+int nmspmm_spmm_noalloc(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C,
+                        int M, int N, int K, int W, int window, int kept, int vec_len, int Ns, int split_k,
+                        void* stream)
+{
+    // every argument is checked before the scratch is looked up, so the error paths need no GPU
+    // (the dry run only validates; C stands in for a workspace that is large enough and aligned)
+    const int st = spmm_impl(A, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k,
+                             split_k > 1 ? (void*)C : nullptr, (size_t)-1, stream, M, true, nullptr);
+    if (st != NMSPMM_OK)
+        return st;
+    const size_t need = nmspmm_workspace_bytes(M, N, split_k);
+    if (need > (size_t)NMSPMM_NOALLOC_MAX_BYTES)
+        return NMSPMM_ERR_WORKSPACE;
+    void* ws = nullptr;
+    if (need > 0) {
+        ws = noalloc_scratch();
+        if (!ws)
+            return NMSPMM_ERR_HIP;
+    }
+    return spmm_impl(A, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k, ws, need, stream, M,
+                     false, nullptr);
 }
 
 // `flags`: NMSPMM_ACCUMULATE for the reference launchers' replacements, whose SPLIT_K > 1 adds to C.

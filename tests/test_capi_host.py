@@ -101,6 +101,30 @@ def test_spmm_rejects_bad_arguments_without_a_gpu():
     assert spmm_status(A=FAKE + 4) == 8
 
 
+def test_noalloc_entry_rejects_bad_arguments_without_a_gpu():
+    """The entry point that allocates nothing: same checks as nmspmm_spmm, and a split whose slices
+    exceed the library's fixed scratch (NMSPMM_NOALLOC_MAX_BYTES, 32 MiB) is refused, all before
+    the GPU is touched."""
+    L = nmspmm.lib()
+    call = lambda **kw: L.nmspmm_spmm_noalloc(kw.get("A", FAKE), FAKE, FAKE, None, FAKE, kw.get("M", 128),
+                                              kw.get("N", 128), kw.get("K", 128), kw.get("W", 64), 32, 16, 32, 128,
+                                              kw.get("split", 1), None)
+    assert call(A=None) == 1
+    assert call(N=96) == 2
+    assert call(split=0) == 5 and call(split=5) == 5
+    assert call(A=FAKE + 4) == 8
+    assert nmspmm.workspace_bytes(1024, 4096, 4) > nmspmm.NOALLOC_MAX_BYTES
+    assert call(M=1024, N=4096, K=1024, W=512, split=4) == 6
+    assert call(M=1 << 20, N=4096, K=1024, W=512, split=16) == 6
+
+
+def test_spmm_ex_rejects_unknown_flags_without_a_gpu():
+    L = nmspmm.lib()
+    args = [FAKE, FAKE, FAKE, None, FAKE, 128, 128, 128, 64, 32, 16, 32, 128, 1, None, 0]
+    assert L.nmspmm_spmm_ex(*args, 2, None) == 2
+    assert L.nmspmm_spmm_ex(FAKE, FAKE, FAKE, None, None, 128, 128, 128, 64, 32, 16, 32, 128, 1, None, 0, 1, None) == 1
+
+
 def test_named_entry_points_reject_the_other_family():
     L = nmspmm.lib()
     low = lambda s, tile=128: L.nmspmm_gemm_low_sparsity(tile, FAKE, FAKE, FAKE, FAKE, 128, 128, 128, 64, s, 1, None)
