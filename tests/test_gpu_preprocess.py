@@ -47,6 +47,7 @@ def test_device_forms_match_reference_golden(path):
     (4096, 4096, 2, 4, 32, 3), (4096, 4096, 1, 8, 32, 3), (4096, 4096, 2, 8, 32, 3), (4096, 4096, 3, 8, 32, 2),
     (11008, 4096, 2, 8, 32, 3), (4096, 11008, 2, 8, 32, 3), (4096, 4096, 8, 32, 32, 1), (4096, 4096, 4, 32, 32, 1),
     (1024, 1024, 2, 4, 4, 3), (512, 512, 2, 4, 8, 4),
+    (4096, 4096, 2, 4, 4, 0),   # 2:4 with vector length 4 at full size: the 2048 x 1024 (8 MiB) index buffer as generated
 ])
 def test_full_size_index_buffers_bit_exact_vs_checker(oracle, N, K, n, m, vl, times):
     d = datagen.init_data(4, N, K, n, m, vec_len=vl, seed=N + K + n)

@@ -182,9 +182,12 @@ def test_operands_off_a_sixteen_byte_boundary_are_rejected(oracle, M):
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 32])
-def test_decode_shape_8192(oracle, M):
-    """One full-size config-4 shape: K = Ncols = 8192 at 1:8."""
-    d = datagen.init_data(M, 8192, 8192, 1, 8, seed=40 + M, dist="normal", b_scale=0.02)
+@pytest.mark.parametrize("n,m", [(1, 8), (2, 8)])
+@pytest.mark.parametrize("K,N", [(8192, 8192), (4096, 14336)])
+def test_decode_shapes_at_full_size(oracle, M, n, m, K, N):
+    """The sixteen decode cases at full size (K = Ncols = 8192 and K = 4096, Ncols = 14336; 1:8 and
+    2:8; B ~ N(0, 0.02^2)), all of C against the checker."""
+    d = datagen.init_data(M, N, K, n, m, seed=40 + M + n, dist="normal", b_scale=0.02)
     got, fam = run_gpu(oracle, d, 128)
     assert fam == "skinny"
     check(oracle, d, got)
@@ -296,11 +299,11 @@ def test_ragged_last_round_is_split_along_k_through_scratch(oracle, M, N, K, n, 
             assert scaled_max_error(C[r0:r1].cpu().numpy(), want) <= REL_TOL
 
 
-def check_every_tile_once(oracle, M, N, K, n, m, Ns):
+def check_every_tile_once(oracle, M, N, K, n, m, Ns, **gen):
     """Unsplit multiplication on the tile kernel; column sums of C against column sums computed
     from the operands in fp64 (touches every tile), and the first and last rows against the
     checker."""
-    d = datagen.init_data(M, N, K, n, m, seed=M + K)
+    d = datagen.init_data(M, N, K, n, m, seed=M + K, **gen)
     window, kept, D, cinfo = preprocess_with_oracle(oracle, d, Ns)
     C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
     nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), None if cinfo is None else dev(cinfo), C, M, N, K, d["W"], window,
@@ -408,6 +411,53 @@ def test_llm_layer_shape_2of8(oracle):
     got, fam = run_gpu(oracle, d, 128)
     assert fam == "mfma"
     check(oracle, d, got)
+
+
+@pytest.mark.parametrize("M", [512, 2048, 8192])
+@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 11008), (11008, 4096)])
+def test_llm_layer_shapes_at_full_size(oracle, M, K, N):
+    """The nine prefill-sized LLM-layer shapes at 2:8, A ~ N(0,1), B ~ N(0, 0.02^2).  K = 11008 is
+    172 windows of 64 rows, not a power of two; Ncols = 11008 is 86 column blocks.  Column sums in
+    fp64 touch every tile, the first and last rows are compared with the checker."""
+    check_every_tile_once(oracle, M, N, K, 2, 8, 128, dist="normal", b_scale=0.02)
+
+
+@pytest.mark.parametrize("n,m", [(4, 32), (8, 32), (16, 32), (3, 8)])
+def test_full_size_4096_cubed_remaining_patterns(oracle, n, m):
+    """The fine-grained patterns (windows of 32 as generated, one widening for 4:32 and 8:32) and
+    3:8 at M = Ncols = K = 4096."""
+    check_every_tile_once(oracle, 4096, 4096, 4096, n, m, 128)
+
+
+def test_full_size_4096_cubed_2of4_with_vectors_of_four_columns(oracle):
+    """2:4 with index vectors of 4 columns at M = Ncols = K = 4096: 2048 x 1024 indices (8 MiB), the
+    expanding matrix-core kernel.  Column sums in fp64 over all of C; sampled rows against the
+    checker."""
+    M = N = K = 4096
+    vl, n, m = 4, 2, 4
+    d = datagen.init_data(M, N, K, n, m, vec_len=vl, seed=5004)
+    W, Q = d["W"], d["Q"]
+    DT = dev(d["DT"].reshape(-1))
+    D = torch.empty_like(DT)
+    nmspmm.preprocess_low_device(DT, D, W, Q, 128, vl)
+    want_D = d["DT"].reshape(-1).copy()
+    oracle.preprocess_low(want_D, W, Q, 128, vl)
+    assert np.array_equal(D.cpu().numpy(), want_D)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), D, None, C, M, N, K, W, m, n, vl, 128)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == "short" and bool(torch.isfinite(C).all())
+    dense = torch.zeros((K, N), dtype=torch.float64, device="cuda")
+    rows = (torch.arange(W, device="cuda") // n * m)[:, None] + dev(d["DT"]).long()
+    dense[rows.repeat_interleave(vl, dim=1), torch.arange(N, device="cuda")[None, :].expand(W, -1)] = dev(d["BT"]).double()
+    want = dev(d["A_km"]).double().sum(dim=1) @ dense
+    got = C.double().sum(dim=0)
+    assert float(((got - want).abs() / want.abs().clamp_min(want.pow(2).mean().sqrt())).max()) <= REL_TOL
+    rows_s = np.array([0, 1, 127, 128, 2047, 2048, M - 129, M - 2, M - 1])
+    A_rows = np.ascontiguousarray(d["A_km"][:, rows_s])
+    ref = oracle.gemm_cpu(A_rows.reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), len(rows_s), N, W,
+                          vl).reshape(len(rows_s), N)
+    assert scaled_max_error(C[torch.from_numpy(rows_s).cuda()].cpu().numpy(), ref) <= REL_TOL
 
 
 @pytest.mark.parametrize("n,m", [(2, 4), (2, 8), (1, 8)])
