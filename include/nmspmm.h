@@ -152,16 +152,40 @@ int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t*
                 float* C, int M, int N, int K, int W, int window, int kept, int vec_len, int Ns,
                 int split_k, void* workspace, size_t workspace_bytes, void* stream);
 
-/* nmspmm_spmm with flags.  NMSPMM_ACCUMULATE: with split_k > 1 the sum of the reduction slices is
- * added to what C holds, C += A . B, exactly what the reference kernels do with their atomicAdd
- * epilogue (src/kernel_64x128_8x8.cu:235-242; deterministic here: C, then the slices in order);
- * with split_k == 1 C is overwritten, as in the reference (:243-251).  Any other flag bit:
- * NMSPMM_ERR_BAD_SHAPE. */
+/* nmspmm_spmm with flags and the optional row list.
+ * NMSPMM_ACCUMULATE: with split_k > 1 the sum of the reduction slices is added to what C holds,
+ * C += A . B, exactly what the reference kernels do with their atomicAdd epilogue
+ * (src/kernel_64x128_8x8.cu:235-242; deterministic here: C, then the slices in order); with
+ * split_k == 1 C is overwritten, as in the reference (:243-251).
+ * NMSPMM_STREAM_B: B is loaded with the non-temporal hint, for weights that will not be read again
+ * before they would have left the caches anyway (a decode step walks through every layer of a
+ * model: gigabytes between two uses of one B).  Only the decode kernel on the row list honours
+ * it; measured there: faster when B comes from HBM, slower when a loop re-reads one B that fits
+ * the 256 MB Infinity Cache.  Any other flag bit: NMSPMM_ERR_BAD_SHAPE.
+ * row_index: NULL, or the row list nmspmm_row_index_device() made from these same D / column_info
+ * (16-byte aligned).  With it, M <= 32 runs on the decode kernel that reads the list instead of
+ * D and column_info; larger M ignore it. */
 #define NMSPMM_ACCUMULATE 1u
+#define NMSPMM_STREAM_B 2u
 int nmspmm_spmm_ex(const float* A, const float* B, const int32_t* D, const int32_t* column_info,
-                   float* C, int M, int N, int K, int W, int window, int kept, int vec_len, int Ns,
-                   int split_k, void* workspace, size_t workspace_bytes, unsigned flags,
-                   void* stream);
+                   const int32_t* row_index, float* C, int M, int N, int K, int W, int window,
+                   int kept, int vec_len, int Ns, int split_k, void* workspace,
+                   size_t workspace_bytes, unsigned flags, void* stream);
+
+/* No counterpart in the reference: a second, kernel-friendly form of the index metadata for the
+ * memory-bound decode sizes, derived from the reference-layout buffers, which stay bit-exact and
+ * remain what every other kernel reads.  The reference kernels find a row of A through two
+ * dependent loads (the rank in D, then the window's column_info list, src/kernel_64x128_8x8.cu:371);
+ * the row list holds the absolute dense row per (32-column vector, kept row):
+ *   row_index[(v * G + g) * 16 + kq * 4 + t] = 1 + k(16 g + 4 t + kq, v),  0 where 16 g + 4 t + kq >= W
+ * G = ceil(W / 16), v = column / 32, k(r, v) = (r / kept) * window + the window-local row that
+ * D (through column_info on the high-sparsity layout) gives for kept row r of vector v.
+ * nmspmm_row_index_ints: int32 the list holds, (N / 32) * G * 16 (0 for invalid arguments).
+ * nmspmm_row_index_device: builds it on the GPU from D [N/Ns][W][Ns/32] and, when non-NULL,
+ * column_info [N/Ns][W/kept][window]; vec_len is 32; asynchronous on `stream`. */
+size_t nmspmm_row_index_ints(int W, int N);
+int nmspmm_row_index_device(const int32_t* dD, const int32_t* d_column_info, int W, int N, int window,
+                            int kept, int Ns, int32_t* d_row_index, void* stream);
 
 /* No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  nmspmm_spmm with the
@@ -238,7 +262,7 @@ int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int
 int nmspmm_release(void);
 
 /* Name of the kernel family the last successful nmspmm_spmm call on this thread dispatched to
- * ("mfma", "short", "skinny", "simt"), for tests and profiles.  Never NULL. */
+ * ("mfma", "short", "skinny", "decode", "simt"), for tests and profiles.  Never NULL. */
 const char* nmspmm_last_kernel(void);
 
 #ifdef __cplusplus

@@ -20,6 +20,7 @@ STATUS_NAMES = {
 }
 TILE_SMALL, TILE_MEDIUM, TILE_LARGE, TILE_HUGE = 32, 64, 64, 128
 ACCUMULATE = 1  # flag of spmm_ex: with split_k > 1 the product is added to what C holds
+STREAM_B = 2    # flag of spmm_ex: B is loaded with the non-temporal hint (decode kernel on the row list)
 
 
 class NmSpmmError(RuntimeError):
@@ -61,7 +62,10 @@ def lib():
         L.nmspmm_workspace_bytes.restype = c_size_t
         L.nmspmm_workspace_bytes.argtypes = [c_int] * 3
         L.nmspmm_spmm.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, c_void_p]
-        L.nmspmm_spmm_ex.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, ctypes.c_uint, c_void_p]
+        L.nmspmm_spmm_ex.argtypes = [c_void_p] * 6 + [c_int] * 9 + [c_void_p, c_size_t, ctypes.c_uint, c_void_p]
+        L.nmspmm_row_index_ints.restype = c_size_t
+        L.nmspmm_row_index_ints.argtypes = [c_int] * 2
+        L.nmspmm_row_index_device.argtypes = [c_void_p, c_void_p] + [c_int] * 5 + [c_void_p, c_void_p]
         L.nmspmm_spmm_noalloc.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p]
         L.nmspmm_gemm_low_sparsity.argtypes = [c_int] + [c_void_p] * 4 + [c_int] * 4 + [c_float, c_int, c_void_p]
         L.nmspmm_gemm_high_sparsity.argtypes = [c_int] + [c_void_p] * 5 + [c_int] * 4 + [c_float, c_int, c_void_p]
@@ -161,11 +165,22 @@ def spmm(A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len=32, Ns=128, split_
                              Ns, split_k, _ptr(workspace), ws_bytes, _stream()))
 
 
-def spmm_ex(A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len=32, Ns=128, split_k=1, workspace=None, flags=0):
+def spmm_ex(A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len=32, Ns=128, split_k=1, workspace=None, flags=0,
+            row_index=None):
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     _check("nmspmm_spmm_ex",
-           lib().nmspmm_spmm_ex(_ptr(A), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(C), M, N, K, W, window, kept, vec_len,
-                                Ns, split_k, _ptr(workspace), ws_bytes, flags, _stream()))
+           lib().nmspmm_spmm_ex(_ptr(A), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(row_index), _ptr(C), M, N, K, W, window,
+                                kept, vec_len, Ns, split_k, _ptr(workspace), ws_bytes, flags, _stream()))
+
+
+def row_index_ints(W, N):
+    return lib().nmspmm_row_index_ints(W, N)
+
+
+def row_index_device(D, cinfo, W, N, window, kept, Ns, row_index):
+    """Row list for the decode kernel from the preprocessed D (and column_info)."""
+    _check("nmspmm_row_index_device",
+           lib().nmspmm_row_index_device(_ptr(D), _ptr(cinfo), W, N, window, kept, Ns, _ptr(row_index), _stream()))
 
 
 NOALLOC_MAX_BYTES = 32 << 20  # NMSPMM_NOALLOC_MAX_BYTES

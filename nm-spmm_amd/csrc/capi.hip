@@ -382,9 +382,9 @@ constexpr int kNotTaken = -1000;
 static int spmm_impl(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C, int M,
                      int N, int K, int W, int window, int kept, int vec_len, int Ns, int split_k, void* workspace,
                      size_t workspace_bytes, void* stream, int lda, bool dry_run, int* lda_out, bool a_rowmajor = false,
-                     unsigned flags = 0)
+                     unsigned flags = 0, const int32_t* row_index = nullptr)
 {
-    if (flags & ~(unsigned)NMSPMM_ACCUMULATE)
+    if (flags & ~(unsigned)(NMSPMM_ACCUMULATE | NMSPMM_STREAM_B))
         return NMSPMM_ERR_BAD_SHAPE;
     if (!A || !B || !D || !C)
         return NMSPMM_ERR_NULL_POINTER;
@@ -410,6 +410,8 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     a.B = B;
     a.D = D;
     a.cinfo = column_info;
+    a.row_index = row_index;
+    a.stream_b = (flags & NMSPMM_STREAM_B) != 0;
     a.C = C;
     a.partial = split_k > 1 ? (float*)workspace : nullptr;
     a.slice_stride = slice_stride(M, N);
@@ -442,9 +444,15 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     if (dry_run)
         return NMSPMM_OK;
 
-    if (a_rowmajor && !(M <= 32 && skinny_supported(a)))
+    if (a_rowmajor && !(M <= 32 && (skinny_supported(a) || decode_supported(a))))
         return kNotTaken;
     hipError_t e;
+    if (decode_supported(a)) {
+        // decode sizes with the row list: one launch, reduction inside the workgroup
+        e = launch_decode(a);
+        g_last_kernel = "decode";
+        return e == hipSuccess ? NMSPMM_OK : NMSPMM_ERR_HIP;
+    }
     // up to 32 rows the decode kernel always wins; up to 128 it competes with the tile kernel at
     // the caller's split
 #ifdef NMSPMM_FORCE_DECODE  // tuning builds: the decode kernel wherever it applies
@@ -545,12 +553,37 @@ int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t*
                      workspace_bytes, stream, M, false, nullptr);
 }
 
-int nmspmm_spmm_ex(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C, int M,
-                   int N, int K, int W, int window, int kept, int vec_len, int Ns, int split_k, void* workspace,
-                   size_t workspace_bytes, unsigned flags, void* stream)
+int nmspmm_spmm_ex(const float* A, const float* B, const int32_t* D, const int32_t* column_info,
+                   const int32_t* row_index, float* C, int M, int N, int K, int W, int window, int kept, int vec_len,
+                   int Ns, int split_k, void* workspace, size_t workspace_bytes, unsigned flags, void* stream)
 {
+    if (row_index && ((uintptr_t)row_index & 15u))
+        return NMSPMM_ERR_ALIGNMENT;
     return spmm_impl(A, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k, workspace,
-                     workspace_bytes, stream, M, false, nullptr, false, flags);
+                     workspace_bytes, stream, M, false, nullptr, false, flags, row_index);
+}
+
+size_t nmspmm_row_index_ints(int W, int N)
+{
+    if (W <= 0 || N <= 0 || N % 32 != 0)
+        return 0;
+    return (size_t)(N / 32) * (size_t)((W + 15) / 16) * 16;
+}
+
+int nmspmm_row_index_device(const int32_t* dD, const int32_t* d_column_info, int W, int N, int window, int kept,
+                            int Ns, int32_t* d_row_index, void* stream)
+{
+    if (!dD || !d_row_index)
+        return NMSPMM_ERR_NULL_POINTER;
+    if (window <= 0 || kept <= 0 || kept > window)
+        return NMSPMM_ERR_BAD_PATTERN;
+    if (W <= 0 || N <= 0 || Ns <= 0 || Ns % 32 != 0 || N % Ns != 0 || W % kept != 0)
+        return NMSPMM_ERR_BAD_SHAPE;
+    if ((long long)(W / kept) * window >= (1LL << 31) - 1)
+        return NMSPMM_ERR_BAD_SHAPE;
+    return launch_row_index(dD, d_column_info, d_row_index, W, N, window, kept, Ns, (hipStream_t)stream) == hipSuccess
+               ? NMSPMM_OK
+               : NMSPMM_ERR_HIP;
 }
 
 int nmspmm_spmm_noalloc(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C,
@@ -607,7 +640,7 @@ static int named_gemm(int want_high, int tile, const float* A, const float* B, c
         if (rc != NMSPMM_OK)
             return rc;
     }
-    return nmspmm_spmm_ex(A, B, D, want_high ? column_info : nullptr, C, M, N, K, W, window, kept, 32, tile,
+    return nmspmm_spmm_ex(A, B, D, want_high ? column_info : nullptr, nullptr, C, M, N, K, W, window, kept, 32, tile,
                           split_k, ws, ws_bytes, flags, stream);
 }
 

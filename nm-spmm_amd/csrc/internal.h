@@ -14,6 +14,8 @@ struct SpmmArgs {
     const float* B;        // row-major W x N
     const int32_t* D;      // [N/Ns][W][Ns/vec_len]
     const int32_t* cinfo;  // [N/Ns][W/kept][window] or nullptr (low-sparsity layout)
+    const int32_t* row_index;  // optional row list [N/32][ceil(W/16)][4][4] (spmm_decode.hip) or nullptr
+    bool stream_b;         // B is loaded with the non-temporal hint (decode kernel on the row list)
     float* C;              // row-major M x N
     float* partial;        // split_k slices of slice_stride floats when split_k > 1, else nullptr
     size_t slice_stride;   // M * N rounded up to a multiple of 4
@@ -361,6 +363,13 @@ hipError_t launch_short(const SpmmArgs& a);
 // Decode-sized path (spmm_skinny.hip): M <= 32, the reference geometries, no workspace needed.
 bool skinny_supported(const SpmmArgs& a);
 hipError_t launch_skinny(const SpmmArgs& a);
+
+// Decode-sized path on the row list (spmm_decode.hip): M <= 32 and a.row_index given.
+bool decode_supported(const SpmmArgs& a);
+hipError_t launch_decode(const SpmmArgs& a);
+// Row list from the preprocessed D (and column_info on the high-sparsity layout).
+hipError_t launch_row_index(const int32_t* D, const int32_t* cinfo, int32_t* R, int W, int N, int window, int kept,
+                            int Ns, hipStream_t stream);
 
 // Generic SIMT path (spmm_simt.hip): any window/kept, vec_len in {4, 8, 16, 32}, any M.
 bool simt_supported(const SpmmArgs& a);

@@ -1,0 +1,257 @@
+// Decode-sized multiplication (M <= 32) on the row list: the index format this library adds for
+// the memory-bound case, next to the reference's D / column_info buffers (which stay as they are).
+//
+// The reference layout makes a kernel chase two dependent loads before it can ask for a row of A:
+// the window's ranks in D, then the window's column_info list (reference
+// src/kernel_64x128_8x8.cu:371 and include/utils.h:82-95 for the meaning).  At decode sizes the
+// whole launch lasts a few memory latencies, so that chain is a quarter of the run time.  The row
+// list stores, per 32-column vector and kept row, the absolute dense row of A, in the order the
+// lanes of this kernel consume it:
+//
+//   row_index[(v * G + g) * 16 + kq * 4 + t] = 1 + k(16 g + 4 t + kq, v),   0 where there is no such kept row
+//
+// with G = ceil(W / 16) groups of 16 kept rows per vector and k(r, v) the dense row that kept row
+// r of vector v multiplies.  One 128-bit load per lane hands lane quarter kq the rows of its next
+// four k-steps; no lane exchange, no second table, and the layout no longer depends on the window
+// geometry or on Ns.
+//
+// Kernel: one workgroup per 32-column vector, 16 waves; wave w takes the groups w, w + 16, ... (so
+// the waves of a workgroup, and with them the whole GPU, read one band of adjacent rows of B at a
+// time).  A k-step is four kept rows on v_mfma_f32_16x16x4_f32: lane (kq, jl) = (l / 16, l % 16)
+// loads B[4 s + kq][2 jl .. 2 jl + 1] with one 64-bit load (four 128-byte row segments per wave and
+// instruction, each byte of B read once) and A[jl][row]; even and odd columns accumulate in two
+// MFMA tiles.  17 to 32 rows take a second pair of tiles for the other 16 rows with the same B
+// operands.  The waves add their tiles up through LDS in wave order (deterministic, one launch,
+// no workspace).  Measured on the MI355X: more than one group per wave in flight does not help (the
+// 16 waves of a CU keep 32 KB of B in flight, which covers the latency at the rate the fabric
+// delivers), so the loop is: load a group, multiply it.
+#include "internal.h"
+
+namespace nmspmm {
+
+typedef float dfloatx4 __attribute__((ext_vector_type(4)));
+typedef int dintx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kDecodeWaves = 16;
+
+struct DecodeParams {
+    const float* A;
+    const float* B;
+    const int32_t* R;
+    float* C;
+    int M, N, W, G;
+    // element (i, k) of A lies i * a_row_stride + k * a_k_stride bytes into its a_bytes bytes
+    uint32_t a_row_stride, a_k_stride, a_bytes, b_bytes;
+    int accumulate;
+};
+
+__device__ inline __amdgpu_buffer_rsrc_t dc_rsrc(const void* base, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+
+// HB: 16-row halves (1: M <= 16, 2: M <= 32).  PAIRS (HB == 2, column-major A with an even pitch):
+// one 64-bit load fetches rows 2 jl and 2 jl + 1 for the two halves, instead of two loads of rows
+// jl and jl + 16.  NT: B is loaded with the non-temporal hint (it is not kept in the caches).
+template <int HB, bool PAIRS, bool NT>
+__global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const DecodeParams p)
+{
+    constexpr int kAux = NT ? 2 : 0;
+    __shared__ float red[kDecodeWaves][8 * HB][64];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kq = lane >> 4, jl = lane & 15;
+    const int v = blockIdx.x;
+    const int M = p.M, N = p.N;
+
+    // every offset that relies on the descriptor's range check is a vector offset: the scalar
+    // offset of a buffer load is not part of that check
+    const __amdgpu_buffer_rsrc_t rb = dc_rsrc(p.B + (size_t)v * 32, p.b_bytes);
+    const __amdgpu_buffer_rsrc_t rr = dc_rsrc(p.R + (size_t)v * p.G * 16, (uint32_t)p.G * 64u);
+    const __amdgpu_buffer_rsrc_t ra = dc_rsrc(p.A, p.a_bytes);
+    const uint32_t a_stride = p.a_k_stride;
+    // the list holds row + 1: entry 0 (no such kept row, or a read beyond the list) puts the offset
+    // below zero, which is out of range and loads 0; so does a lane whose row of C does not exist
+    uint32_t a_lane[HB];
+    if (PAIRS) {
+        a_lane[0] = (2 * jl < M ? (uint32_t)jl * 8u : 0x80000000u) - a_stride;
+    } else {
+#pragma unroll
+        for (int hb = 0; hb < HB; ++hb)
+            a_lane[hb] = (jl + 16 * hb < M ? (uint32_t)(jl + 16 * hb) * p.a_row_stride : 0x80000000u) - a_stride;
+    }
+    const uint32_t b_lane = (uint32_t)(((size_t)kq * N + 2 * jl) * sizeof(float));
+    const uint32_t b_step = (uint32_t)((size_t)4 * N * sizeof(float));
+
+    dfloatx4 acc_e[HB], acc_o[HB];
+#pragma unroll
+    for (int hb = 0; hb < HB; ++hb) {
+        acc_e[hb] = {0.0f, 0.0f, 0.0f, 0.0f};
+        acc_o[hb] = {0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    auto load_rows = [&](int g) -> dintx4 {
+        const auto x = __builtin_amdgcn_raw_buffer_load_b128(rr, (uint32_t)(g * 64 + kq * 16), 0, 0);
+        dintx4 r = {(int)x[0], (int)x[1], (int)x[2], (int)x[3]};
+        return r;
+    };
+
+    dintx4 rows = load_rows(wave);
+    for (int g = wave; g < p.G; g += kDecodeWaves) {
+        float2 b[4];
+        float a[4][HB];
+        const uint32_t b_group = b_lane + (uint32_t)g * 4u * b_step;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            // rows at or beyond W (the tail of the last group) lie beyond the descriptor: 0
+            const auto x = __builtin_amdgcn_raw_buffer_load_b64(rb, b_group + t * b_step, 0, kAux);
+            b[t] = make_float2(__int_as_float(x[0]), __int_as_float(x[1]));
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            if constexpr (PAIRS) {
+                const auto x = __builtin_amdgcn_raw_buffer_load_b64(ra, a_lane[0] + (uint32_t)rows[t] * a_stride, 0, 0);
+                a[t][0] = __int_as_float(x[0]);
+                a[t][1] = __int_as_float(x[1]);
+            } else {
+#pragma unroll
+                for (int hb = 0; hb < HB; ++hb)
+                    a[t][hb] = __int_as_float(
+                        __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane[hb] + (uint32_t)rows[t] * a_stride, 0, 0));
+            }
+        }
+        rows = load_rows(g + kDecodeWaves);  // beyond the list: zeros, never used
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int hb = 0; hb < HB; ++hb) {
+                acc_e[hb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t][hb], b[t].x, acc_e[hb], 0, 0, 0);
+                acc_o[hb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t][hb], b[t].y, acc_o[hb], 0, 0, 0);
+            }
+    }
+
+    // the waves' tiles are added in wave order.  Value x of a lane: register x % 4 of the even
+    // (x % 8 < 4) or odd columns of half x / 8; register r of lane (kq, jl) is tile row 4 kq + r
+#pragma unroll
+    for (int hb = 0; hb < HB; ++hb)
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            red[wave][8 * hb + x][lane] = acc_e[hb][x];
+            red[wave][8 * hb + 4 + x][lane] = acc_o[hb][x];
+        }
+    __syncthreads();
+    for (int x = wave; x < 8 * HB; x += kDecodeWaves) {
+        float s = red[0][x][lane];
+#pragma unroll
+        for (int y = 1; y < kDecodeWaves; ++y)
+            s += red[y][x][lane];
+        const int tile_row = 4 * kq + (x % 4);
+        const int row = PAIRS ? 2 * tile_row + x / 8 : 16 * (x / 8) + tile_row;
+        if (row < M) {
+            float* const dst = p.C + (size_t)row * N + (size_t)v * 32 + 2 * jl + (x % 8) / 4;
+            *dst = p.accumulate ? *dst + s : s;
+        }
+    }
+}
+
+bool decode_supported(const SpmmArgs& a)
+{
+    if (a.row_index == nullptr || a.M > 32 || a.vec_len != 32)
+        return false;
+    if (a.a_rowmajor) {
+        if (a.lda < a.K || (size_t)a.M * a.lda * sizeof(float) >= 0x80000000ull)
+            return false;
+    } else {
+        if (a.lda < a.M || (size_t)a.K * a.lda * sizeof(float) >= 0x80000000ull)
+            return false;
+    }
+    // 32-bit offsets into B from a vector's first column, and into a vector's part of the list
+    if ((size_t)a.W * a.N * sizeof(float) >= 0xffffffffull || (size_t)a.W * 4 + 64 >= 0xffffffffull)
+        return false;
+    return true;
+}
+
+hipError_t launch_decode(const SpmmArgs& a)
+{
+    DecodeParams p;
+    p.A = a.A;
+    p.B = a.B;
+    p.R = a.row_index;
+    p.C = a.C;
+    p.M = a.M;
+    p.N = a.N;
+    p.W = a.W;
+    p.G = (a.W + 15) / 16;
+    p.a_row_stride = (uint32_t)(a.a_rowmajor ? a.lda * sizeof(float) : sizeof(float));
+    p.a_k_stride = (uint32_t)(a.a_rowmajor ? sizeof(float) : a.lda * sizeof(float));
+    p.a_bytes = (uint32_t)((size_t)(a.a_rowmajor ? a.M : a.K) * a.lda * sizeof(float));
+    p.b_bytes = (uint32_t)(((size_t)(a.W - 1) * a.N + 32) * sizeof(float));
+    p.accumulate = (a.accumulate && a.split_k > 1) ? 1 : 0;
+    const dim3 grid(a.N / 32), block(64 * kDecodeWaves);
+    const bool pairs = a.M > 16 && !a.a_rowmajor && a.lda % 2 == 0 && a.M % 2 == 0;
+    if (a.M <= 16) {
+        if (a.stream_b)
+            spmm_decode_kernel<1, false, true><<<grid, block, 0, a.stream>>>(p);
+        else
+            spmm_decode_kernel<1, false, false><<<grid, block, 0, a.stream>>>(p);
+    } else if (pairs) {
+        if (a.stream_b)
+            spmm_decode_kernel<2, true, true><<<grid, block, 0, a.stream>>>(p);
+        else
+            spmm_decode_kernel<2, true, false><<<grid, block, 0, a.stream>>>(p);
+    } else {
+        if (a.stream_b)
+            spmm_decode_kernel<2, false, true><<<grid, block, 0, a.stream>>>(p);
+        else
+            spmm_decode_kernel<2, false, false><<<grid, block, 0, a.stream>>>(p);
+    }
+    return hipGetLastError();
+}
+
+// Builds the row list from the preprocessed buffers (D in its blocked layout, column_info on the
+// high-sparsity layout): one thread per list entry, writes coalesced.
+__global__ void __launch_bounds__(256)
+row_index_kernel(const int32_t* __restrict__ D, const int32_t* __restrict__ cinfo, int32_t* __restrict__ R, int W,
+                 int Q, int Qs, int window, int kept, int G)
+{
+    const size_t total = (size_t)Q * G * 16;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const int nwin = W / kept;
+    for (size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += stride) {
+        const int e = (int)(o % 16);
+        const size_t vg = o / 16;
+        const int g = (int)(vg % G);
+        const int v = (int)(vg / G);
+        const int kq = e / 4, t = e % 4;
+        const int r = 16 * g + 4 * t + kq;
+        int out = 0;
+        if (r < W) {
+            const int jb = v / Qs, c = v % Qs;
+            const int w = r / kept;
+            int local = D[((size_t)jb * W + r) * Qs + c];
+            if (cinfo != nullptr) {
+                // a rank outside the window's list marks a malformed index: no row
+                local = (unsigned)local < (unsigned)window ? cinfo[((size_t)jb * nwin + w) * window + local] : -1;
+            }
+            if ((unsigned)local < (unsigned)window)
+                out = 1 + w * window + local;
+        }
+        R[o] = out;
+    }
+}
+
+hipError_t launch_row_index(const int32_t* D, const int32_t* cinfo, int32_t* R, int W, int N, int window, int kept,
+                            int Ns, hipStream_t stream)
+{
+    const int Q = N / 32, G = (W + 15) / 16;
+    const size_t total = (size_t)Q * G * 16;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 256 * 32)
+        blocks = 256 * 32;
+    if (blocks < 1)
+        blocks = 1;
+    row_index_kernel<<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(D, cinfo, R, W, Q, Ns / 32, window, kept, G);
+    return hipGetLastError();
+}
+
+} // namespace nmspmm

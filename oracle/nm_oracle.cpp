@@ -14,6 +14,9 @@
 //   nm_oracle_decompress       scatter/gather round trip
 //   nm_oracle_compress         recovers generated (BT, DT) from their dense expansion, fp64 score
 //                              dominance of kept over dropped rows, constructed ties, sign symmetry
+//   nm_oracle_row_index        equals the generator's global rows (the D the reference's own CPU
+//                              path multiplies with, include/utils.h:60) entry by entry, on every
+//                              geometry and column-block width; padding entries are 0
 // No function here is "parity unpinned".
 //
 // Vocabulary (reference include/utils.h:10-66, include/NM-SpMM.h:8):
@@ -205,6 +208,35 @@ void nm_oracle_compress(const float* dense, int K, int N, int n, int m, int vec_
                 std::memcpy(BT + row * N + (size_t)a * vec_len, src, sizeof(float) * vec_len);
             }
         }
+    }
+}
+
+// The row list of the decode kernel (no reference counterpart; it restates how the reference
+// kernels address a row of A: src/kernel_64x128_8x8.cu:75-77 for the low-sparsity layout,
+// dense row = window * Ks + D[...]; :371 for the high-sparsity one, through column_info).
+// D is the preprocessed blocked buffer [N/Ns][W][Ns/32], column_info [N/Ns][W/kept][window] or
+// NULL.  R[(v * G + g) * 16 + kq * 4 + t] = 1 + dense row of kept row 16 g + 4 t + kq of vector v,
+// 0 beyond W; G = ceil(W / 16).
+void nm_oracle_row_index(const int32_t* D, const int32_t* column_info, int W, int N, int window, int kept, int Ns,
+                         int32_t* R)
+{
+    const int Q = N / 32, Qs = Ns / 32, G = (W + 15) / 16, nwin = W / kept;
+    for (int v = 0; v < Q; ++v) {
+        const int jb = v / Qs, c = v % Qs;
+        for (int g = 0; g < G; ++g)
+            for (int kq = 0; kq < 4; ++kq)
+                for (int t = 0; t < 4; ++t) {
+                    const int r = 16 * g + 4 * t + kq;
+                    int32_t out = 0;
+                    if (r < W) {
+                        const int w = r / kept;
+                        int32_t local = D[((int64_t)jb * W + r) * Qs + c];
+                        if (column_info)
+                            local = column_info[((int64_t)jb * nwin + w) * window + local];
+                        out = 1 + w * window + local;
+                    }
+                    R[((int64_t)v * G + g) * 16 + kq * 4 + t] = out;
+                }
     }
 }
 

@@ -45,7 +45,8 @@ class Oracle:
         lib.nm_oracle_gemm_cpu.argtypes = [_f32p, _f32p, _i32p, _f32p] + [_int] * 6
         lib.nm_oracle_decompress.argtypes = [_f32p, _i32p, _f32p] + [_int] * 4
         lib.nm_oracle_compress.argtypes = [_f32p] + [_int] * 5 + [_f32p, _i32p]
-        for f in ("trans_index", "preprocess_low", "preprocess_high", "gemm_cpu", "decompress", "compress"):
+        lib.nm_oracle_row_index.argtypes = [_i32p, ctypes.c_void_p] + [_int] * 5 + [_i32p]
+        for f in ("trans_index", "preprocess_low", "preprocess_high", "gemm_cpu", "decompress", "compress", "row_index"):
             getattr(lib, "nm_oracle_" + f).restype = None
         self.lib = lib
 
@@ -75,6 +76,13 @@ class Oracle:
         r0, r1 = (0, M) if rows is None else rows
         self.lib.nm_oracle_gemm_cpu(A, B, D, C, M, N, W, vec_len, r0, r1)
         return C
+
+    def row_index(self, D, cinfo, W, N, window, kept, Ns):
+        """Row list int32[(N/32) * ceil(W/16) * 16] from the preprocessed D (and column_info or None)."""
+        R = np.empty((N // 32) * ((W + 15) // 16) * 16, np.int32)
+        ci = None if cinfo is None else cinfo.ctypes.data_as(ctypes.c_void_p)
+        self.lib.nm_oracle_row_index(D, ci, W, N, window, kept, Ns, R)
+        return R
 
     def decompress(self, B, D, K, N, W, vec_len=32):
         dense = np.empty(K * N, np.float32)

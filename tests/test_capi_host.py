@@ -120,9 +120,24 @@ def test_noalloc_entry_rejects_bad_arguments_without_a_gpu():
 
 def test_spmm_ex_rejects_unknown_flags_without_a_gpu():
     L = nmspmm.lib()
-    args = [FAKE, FAKE, FAKE, None, FAKE, 128, 128, 128, 64, 32, 16, 32, 128, 1, None, 0]
-    assert L.nmspmm_spmm_ex(*args, 2, None) == 2
-    assert L.nmspmm_spmm_ex(FAKE, FAKE, FAKE, None, None, 128, 128, 128, 64, 32, 16, 32, 128, 1, None, 0, 1, None) == 1
+    args = [FAKE, FAKE, FAKE, None, None, FAKE, 128, 128, 128, 64, 32, 16, 32, 128, 1, None, 0]
+    assert L.nmspmm_spmm_ex(*args, 4, None) == 2
+    assert L.nmspmm_spmm_ex(FAKE, FAKE, FAKE, None, None, None, 128, 128, 128, 64, 32, 16, 32, 128, 1, None, 0, 1, None) == 1
+    args[4] = FAKE + 4   # a row list that is not 16-byte aligned
+    assert L.nmspmm_spmm_ex(*args, 0, None) == 8
+
+
+def test_row_list_entry_points_reject_bad_arguments_without_a_gpu():
+    L = nmspmm.lib()
+    assert nmspmm.row_index_ints(1024, 8192) == 256 * 64 * 16
+    assert nmspmm.row_index_ints(36, 128) == 4 * 3 * 16       # the last group is padded
+    assert nmspmm.row_index_ints(0, 128) == 0 and nmspmm.row_index_ints(64, 100) == 0
+    call = lambda **kw: L.nmspmm_row_index_device(kw.get("D", FAKE), FAKE, kw.get("W", 64), kw.get("N", 128),
+                                                   kw.get("window", 64), kw.get("kept", 16), kw.get("Ns", 128),
+                                                   kw.get("R", FAKE), None)
+    assert call(D=None) == 1 and call(R=None) == 1
+    assert call(kept=80) == 3
+    assert call(W=60) == 2 and call(N=96) == 2 and call(Ns=48) == 2
 
 
 def test_named_entry_points_reject_the_other_family():

@@ -1,0 +1,169 @@
+"""The row list (the decode-oriented index format) and the decode kernel that reads it, on the GPU
+through the C-ABI.  The list must equal the checker's bit for bit; the multiplication must match
+the checker's restatement of the reference's nmGEMM_on_cpu within the scaled max error 1e-4."""
+import numpy as np
+import pytest
+
+from conftest import REL_TOL, datagen, nmspmm, preprocess_with_oracle, scaled_max_error
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def gpu_row_list(D, cinfo, W, N, window, kept, Ns):
+    R = torch.full((nmspmm.row_index_ints(W, N),), -77, dtype=torch.int32, device="cuda")
+    nmspmm.row_index_device(dev(D), None if cinfo is None else dev(cinfo), W, N, window, kept, Ns, R)
+    torch.cuda.synchronize()
+    return R
+
+
+def want_c(oracle, d, C0=None):
+    return oracle.gemm_cpu(d["A_km"].reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), d["M"], d["N"], d["W"],
+                           C=None if C0 is None else C0.reshape(-1).copy()).reshape(d["M"], d["N"])
+
+
+def run_decode(oracle, d, Ns=128, flags=0, split_k=1, C0=None):
+    M, N, K, W = d["M"], d["N"], d["K"], d["W"]
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, Ns)
+    R = gpu_row_list(D, cinfo, W, N, window, kept, Ns)
+    assert np.array_equal(R.cpu().numpy(), oracle.row_index(D, cinfo, W, N, window, kept, Ns))
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda") if C0 is None else dev(C0)
+    ws = None
+    if split_k > 1:
+        ws = torch.empty(nmspmm.workspace_bytes(M, N, split_k) // 4, dtype=torch.float32, device="cuda")
+    nmspmm.spmm_ex(dev(d["A_km"]), dev(d["BT"]), dev(D), None if cinfo is None else dev(cinfo), C, M, N, K, W, window,
+                   kept, 32, Ns, split_k, ws, flags, R)
+    torch.cuda.synchronize()
+    return C.cpu().numpy(), nmspmm.last_kernel()
+
+
+@pytest.mark.parametrize("n,m", [(2, 4), (3, 8), (2, 8), (1, 8), (16, 32), (12, 32), (8, 32), (4, 32), (32, 32)])
+@pytest.mark.parametrize("Ns", [128, 64, 32])
+def test_row_list_bit_exact_every_pattern_and_block_width(oracle, n, m, Ns):
+    d = datagen.init_data(4, 512, 1024, n, m, seed=n + m + Ns)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, Ns)
+    got = gpu_row_list(D, cinfo, d["W"], d["N"], window, kept, Ns).cpu().numpy()
+    assert np.array_equal(got, oracle.row_index(D, cinfo, d["W"], d["N"], window, kept, Ns))
+    # and, independently of the checker, the generator's own global rows
+    assert np.array_equal(np.sort(got.reshape(d["Q"], -1), axis=1)[:, -d["W"]:], np.sort(d["D_cm"] + 1, axis=1))
+
+
+@pytest.mark.parametrize("N,K,n,m", [(8192, 8192, 1, 8), (8192, 8192, 2, 8), (14336, 4096, 1, 8), (14336, 4096, 2, 8),
+                                     (4096, 11008, 2, 8), (4096, 4096, 3, 8)])
+def test_row_list_bit_exact_at_full_size(oracle, N, K, n, m):
+    d = datagen.init_data(1, N, K, n, m, seed=N + K + n)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    got = gpu_row_list(D, cinfo, d["W"], N, window, kept, 128).cpu().numpy()
+    assert np.array_equal(got, oracle.row_index(D, cinfo, d["W"], N, window, kept, 128))
+
+
+@pytest.mark.parametrize("M", [1, 2, 7, 8, 13, 16, 17, 24, 31, 32])
+@pytest.mark.parametrize("n,m,K", [(1, 8, 1024), (2, 8, 1088), (2, 4, 1152), (3, 8, 96), (3, 8, 1120), (32, 32, 160), (4, 32, 960)])
+def test_decode_kernel_every_row_count(oracle, M, n, m, K):
+    """Row counts on both sides of 16 and 32, odd ones included (17 to 32 rows take one 64-bit
+    load of A per k-step when the row count is even, two 32-bit loads when it is odd); reductions
+    that give the 16 waves of a workgroup unequal shares, some none, and (3:8 with K = 96: 36 kept
+    rows) a last group of four rows."""
+    d = datagen.init_data(M, 256, K, n, m, seed=M + K, dist="normal", b_scale=0.02)
+    got, fam = run_decode(oracle, d)
+    assert fam == "decode"
+    assert np.isfinite(got).all() and scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
+
+
+@pytest.mark.parametrize("Ns", [64, 32])
+@pytest.mark.parametrize("M,n,m", [(5, 1, 8), (32, 2, 8), (16, 2, 4)])
+def test_decode_kernel_with_lists_from_other_block_widths(oracle, Ns, M, n, m):
+    d = datagen.init_data(M, 512, 512, n, m, seed=M + Ns)
+    got, fam = run_decode(oracle, d, Ns=Ns)
+    assert fam == "decode"
+    assert scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 32])
+@pytest.mark.parametrize("n,m", [(1, 8), (2, 8)])
+@pytest.mark.parametrize("K,N", [(8192, 8192), (4096, 14336)])
+def test_decode_shapes_at_full_size_on_the_row_list(oracle, M, n, m, K, N):
+    """The sixteen decode cases at full size, all of C against the checker, with and without the
+    non-temporal hint for B (same result bit for bit: only the cache policy of the loads differs)."""
+    d = datagen.init_data(M, N, K, n, m, seed=140 + M + n, dist="normal", b_scale=0.02)
+    got, fam = run_decode(oracle, d)
+    assert fam == "decode"
+    assert np.isfinite(got).all() and scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
+    streamed, fam = run_decode(oracle, d, flags=nmspmm.STREAM_B)
+    assert fam == "decode" and np.array_equal(streamed, got)
+
+
+@pytest.mark.parametrize("M", [3, 16, 20, 32])
+def test_decode_kernel_adds_to_c_when_asked_like_a_split_call_of_the_reference(oracle, M):
+    """split_k has no effect on how this kernel computes (one launch, reduction in the workgroup),
+    but a split call with NMSPMM_ACCUMULATE still adds to C, as the reference's split calls do."""
+    d = datagen.init_data(M, 256, 1024, 2, 8, seed=M)
+    rng = np.random.default_rng(M)
+    C0 = rng.uniform(-3.0, 3.0, (M, 256)).astype(np.float32)
+    got, fam = run_decode(oracle, d, flags=nmspmm.ACCUMULATE, split_k=4, C0=C0)
+    assert fam == "decode" and scaled_max_error(got, want_c(oracle, d, C0)) <= REL_TOL
+    got, _ = run_decode(oracle, d, flags=nmspmm.ACCUMULATE, split_k=1, C0=C0)
+    assert scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
+    got, _ = run_decode(oracle, d, flags=0, split_k=4, C0=C0)
+    assert scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
+
+
+def test_larger_row_counts_ignore_the_list(oracle):
+    d = datagen.init_data(48, 256, 512, 2, 8, seed=3)
+    got, fam = run_decode(oracle, d)
+    assert fam in ("skinny", "mfma")
+    assert scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
+
+
+def test_a_list_off_a_sixteen_byte_boundary_is_rejected(oracle):
+    d = datagen.init_data(4, 128, 256, 2, 8, seed=1)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    base = torch.zeros(nmspmm.row_index_ints(d["W"], 128) + 1, dtype=torch.int32, device="cuda")
+    C = torch.zeros((4, 128), dtype=torch.float32, device="cuda")
+    with pytest.raises(nmspmm.NmSpmmError, match="ALIGNMENT"):
+        nmspmm.spmm_ex(dev(d["A_km"]), dev(d["BT"]), dev(D), dev(cinfo), C, 4, 128, 256, d["W"], window, kept, 32, 128, 1,
+                       None, 0, base[1:])
+
+
+def test_decode_kernel_with_131072_column_vectors(oracle):
+    """Ncols = 2^22: 131072 workgroups, B rows 16 MiB apart."""
+    M, N, K = 4, 1 << 22, 64
+    d = datagen.init_data(M, N, K, 2, 4, seed=4445, dist="normal", b_scale=0.02)
+    got, fam = run_decode(oracle, d)
+    assert fam == "decode"
+    assert scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
+
+
+@pytest.mark.parametrize("M,n,m", [(8, 1, 8), (32, 2, 8)])
+def test_graph_replays_of_the_decode_kernel_equal_eager_calls(oracle, M, n, m):
+    N, K = 512, 1024
+    d = datagen.init_data(M, N, K, n, m, seed=M, dist="normal", b_scale=0.02)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    R = gpu_row_list(D, cinfo, d["W"], N, window, kept, 128)
+    A, B, Dd, ci = dev(d["A_km"]), dev(d["BT"]), dev(D), dev(cinfo)
+    C_g = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    C_e = torch.empty_like(C_g)
+
+    def call(C):
+        nmspmm.spmm_ex(A, B, Dd, ci, C, M, N, K, d["W"], window, kept, 32, 128, 1, None, 0, R)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(C_g)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(C_g)
+    for rep in range(3):
+        A.mul_(1.25)
+        C_g.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        call(C_e)
+        torch.cuda.synchronize()
+        assert torch.isfinite(C_g).all().item() and torch.equal(C_g, C_e), "replay %d" % rep
