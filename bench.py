@@ -2,23 +2,33 @@
 """Benchmark of the N:M sparse x dense fp32 multiplication on one MI355X.
 
 One "step" is one launch of the hot path (nmspmm_spmm through the C-ABI) on the square sweep of
-the baseline: M = Ncols = K = 4096, fp32, operands resident in HBM, at 2:4 (the headline value),
-3:8, 2:8 and 1:8 (reported under "sweep").  Prints ONE JSON line:
+the baseline: M = Ncols = K = 4096, fp32, operands resident in HBM, at 2:4 (the headline value).
+Prints ONE JSON line:
 
   value            useful TFLOP/s at 2:4 = 2*M*Ncols*W / t   (W = K*n/m)
-  roofline         the dominant kernel (spmm_direct_kernel at 2:4) against the fp32 MFMA peak
+  roofline         the dominant kernel (the tile kernel at 2:4) against the fp32 MFMA peak
   cpu_baseline     the reference project's own nmGEMM_on_cpu (oracle/_ref) on a row slice
-  sweep            per pattern: ms, useful and dense-equivalent TFLOP/s, speedup over the dense
-                   fp32 GEMM of the same shape (rocBLAS/hipBLASLt through torch.mm), and the GPU
-                   preprocessing time (the reference's call sequence, and the one-kernel entry)
+  sweep            3:8, 2:8, 1:8 beside 2:4: ms, useful TFLOP/s, speedup over the dense fp32 GEMM
+  configs          the baseline's other workloads, each timed in this run:
+                     llm     nine prefill-sized LLM-layer shapes at 2:8 against the dense fp32 GEMM
+                     decode  M in {1, 8, 16, 32} x two weight shapes x {1:8, 2:8}: microseconds and
+                             algorithmic GB/s against the 8 TB/s HBM bound, with B re-read from the
+                             caches ("hot") and streamed from HBM ("cold"), row list on and off
+                     fine    4:32, 8:32, 16:32 and 2:4 with 4-column vectors at 4096 cubed
+  preprocess       index preprocessing: one-kernel device call, the reference's call sequence on
+                   the device, the host-pointer drop-in calls (wall time, PCIe included), and the
+                   CPU restatement / the reference's own host code
+  dispatch         the library's split / kernel choice against the best of the splits 1, 2, 4, 8
 
 Timing uses HIP events on the stream the kernels are launched on (torch's current stream is the
-one handed to the C-ABI).
+one handed to the C-ABI); decode-sized launches are replayed from a HIP graph so that the host's
+launch rate does not enter.  --only selects parts (for profiling runs); the default runs all.
 """
 import argparse
 import importlib
 import json
 import os
+import re
 import sys
 import time
 
@@ -28,70 +38,23 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 FP32_MFMA_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBS = 8000.0
 M = N = K = 4096
 PATTERNS = [(2, 4), (3, 8), (2, 8), (1, 8)]  # first one is the headline
 NS = 128
+GEOMETRY = {(1, 1): (32, 32), (1, 2): (32, 16), (3, 8): (32, 12), (1, 4): (64, 16), (1, 8): (64, 8)}
+PARTS = ("sweep", "llm", "decode", "fine", "preprocess", "dispatch", "cpu")
 
 
 def geometry(n, m):
-    window, kept = {(2, 4): (32, 16), (3, 8): (32, 12), (2, 8): (64, 16), (1, 8): (64, 8)}[(n, m)]
-    times = {4: 3, 8: 2}[m] + (1 if window == 64 else 0)
+    """(window, kept, transIndex doublings) the kernels run an n:m pattern at."""
+    from math import gcd
+    g = gcd(n, m)
+    window, kept = GEOMETRY[(n // g, m // g)]
+    times, mm = 0, m
+    while mm < window:
+        mm, times = mm * 2, times + 1
     return window, kept, times
-
-
-class Case:
-    """Operands of one pattern, resident on the GPU, preprocessed by the GPU kernels."""
-
-    def __init__(self, torch, pkg, datagen, n, m, seed):
-        d = datagen.init_data(M, N, K, n, m, seed=seed)
-        self.d, self.n, self.m = d, n, m
-        self.W, self.Q = d["W"], d["Q"]
-        self.window, self.kept, times = geometry(n, m)
-        self.A = torch.from_numpy(d["A_km"]).cuda()
-        self.B = torch.from_numpy(d["BT"]).cuda()
-        self.C = torch.zeros((M, N), dtype=torch.float32, device="cuda")
-        DT0 = torch.from_numpy(d["DT"].reshape(-1).copy()).cuda()
-        self.cinfo = None
-        if self.window == 64:
-            self.cinfo = torch.empty(pkg.column_info_ints(self.W, self.kept, self.window, N, NS), dtype=torch.int32,
-                                     device="cuda")
-        self.D = torch.empty_like(DT0)
-        DT = torch.empty_like(DT0)
-
-        def preprocess():
-            DT.copy_(DT0)
-            pn, pm = n, m
-            for _ in range(times):
-                pn, pm = pkg.trans_index_device(DT, self.W, N, self.Q, pn, pm)
-            if self.cinfo is None:
-                pkg.preprocess_low_device(DT, self.D, self.W, self.Q, NS)
-            else:
-                pkg.preprocess_high_device(self.cinfo, pm, pn, DT, self.D, self.W, self.Q, N, NS)
-
-        preprocess()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(5):
-            preprocess()
-        e1.record()
-        torch.cuda.synchronize()
-        self.preprocess_ms = e0.elapsed_time(e1) / 5
-        # the same work by the one-kernel entry point (widening folded into the re-blocking pass)
-        pkg.preprocess_device(DT0, n, m, self.W, self.Q, N, NS, self.D, self.cinfo)
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(20):
-            pkg.preprocess_device(DT0, n, m, self.W, self.Q, N, NS, self.D, self.cinfo)
-        e1.record()
-        torch.cuda.synchronize()
-        self.preprocess_one_kernel_ms = e0.elapsed_time(e1) / 20
-
-    def launch(self, pkg):
-        pkg.spmm(self.A, self.B, self.D, self.cinfo, self.C, M, N, K, self.W, self.window, self.kept, 32, NS, 1, None)
-
-    def useful_flops(self):
-        return 2.0 * M * N * self.W
 
 
 PREWARM_S = 1.0
@@ -120,6 +83,107 @@ def time_launches(torch, fn, steps, warmup, prewarm_s=None):
     return e0.elapsed_time(e1) / steps, wall_ms
 
 
+def time_graph(torch, calls, replays=6, prewarm_s=0.15):
+    """Milliseconds per call of a HIP graph that holds the calls back to back, best of `replays`
+    (each replay is one event pair around the whole graph)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        calls[0]()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for c in calls:
+            c()
+    t_end = time.perf_counter() + prewarm_s
+    while time.perf_counter() < t_end:
+        graph.replay()
+        torch.cuda.synchronize()
+    best = 1e9
+    for _ in range(replays):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        best = min(best, e0.elapsed_time(e1) / len(calls))
+    del graph
+    return best
+
+
+class Case:
+    """Operands of one square-sweep pattern from the seeded host generator (the CPU baseline needs
+    the host arrays), resident on the GPU, preprocessed by the GPU kernels."""
+
+    def __init__(self, torch, pkg, datagen, n, m, seed):
+        d = datagen.init_data(M, N, K, n, m, seed=seed)
+        self.d, self.n, self.m = d, n, m
+        self.W, self.Q = d["W"], d["Q"]
+        self.window, self.kept, _ = geometry(n, m)
+        self.A = torch.from_numpy(d["A_km"]).cuda()
+        self.B = torch.from_numpy(d["BT"]).cuda()
+        self.C = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        DT0 = torch.from_numpy(d["DT"].reshape(-1).copy()).cuda()
+        self.cinfo = None
+        if self.window == 64:
+            self.cinfo = torch.empty(pkg.column_info_ints(self.W, self.kept, self.window, N, NS), dtype=torch.int32,
+                                     device="cuda")
+        self.D = torch.empty_like(DT0)
+        pkg.preprocess_device(DT0, n, m, self.W, self.Q, N, NS, self.D, self.cinfo)
+        torch.cuda.synchronize()
+
+    def launch(self, pkg):
+        pkg.spmm(self.A, self.B, self.D, self.cinfo, self.C, M, N, K, self.W, self.window, self.kept, 32, NS, 1, None)
+
+    def useful_flops(self):
+        return 2.0 * M * N * self.W
+
+
+class GpuOperands:
+    """Synthetic operands drawn on the GPU (values and per-vector patterns), preprocessed on the
+    GPU: for the workloads whose results are checked by the test-suite, not here."""
+
+    def __init__(self, torch, pkg, m_rows, n_cols, k, n, m, vec_len=32, normal=True, row_list=False):
+        self.M, self.N, self.K, self.n, self.m, self.vl = m_rows, n_cols, k, n, m, vec_len
+        self.W, self.Q = k // m * n, n_cols // vec_len
+        scale = 0.02 if normal else 1.0
+        if normal:
+            self.A = torch.randn((k, m_rows), dtype=torch.float32, device="cuda")
+            self.B = torch.randn((self.W, n_cols), dtype=torch.float32, device="cuda") * scale
+        else:
+            self.A = torch.rand((k, m_rows), dtype=torch.float32, device="cuda") * 2 - 1
+            self.B = torch.rand((self.W, n_cols), dtype=torch.float32, device="cuda") * 2 - 1
+        self.C = torch.zeros((m_rows, n_cols), dtype=torch.float32, device="cuda")
+        pick = torch.rand((k // m, self.Q, m), device="cuda").argsort(dim=2)[:, :, :n].sort(dim=2).values
+        self.DT = pick.permute(0, 2, 1).reshape(self.W, self.Q).to(torch.int32).contiguous()
+        del pick
+        self.D = torch.empty_like(self.DT)
+        self.cinfo = None
+        if vec_len == 32:
+            self.window, self.kept, _ = geometry(n, m)
+            if self.window == 64:
+                self.cinfo = torch.empty(pkg.column_info_ints(self.W, self.kept, self.window, n_cols, NS),
+                                         dtype=torch.int32, device="cuda")
+            pkg.preprocess_device(self.DT, n, m, self.W, self.Q, n_cols, NS, self.D, self.cinfo)
+        else:
+            self.window, self.kept = m, n
+            pkg.preprocess_low_device(self.DT, self.D, self.W, self.Q, NS, vec_len)
+        self.R = None
+        if row_list:
+            self.R = torch.empty(pkg.row_index_ints(self.W, n_cols), dtype=torch.int32, device="cuda")
+            pkg.row_index_device(self.D, self.cinfo, self.W, n_cols, self.window, self.kept, NS, self.R)
+        torch.cuda.synchronize()
+
+    def flops(self):
+        return 2.0 * self.M * self.N * self.W
+
+    def algorithmic_bytes(self):
+        b = 4.0 * (self.M * self.K + self.W * self.N + self.W * self.N / self.vl + self.M * self.N)
+        if self.cinfo is not None:
+            b += 4.0 * self.cinfo.numel()
+        return b
+
+
 def cpu_baseline(case, rows):
     """The reference's nmGEMM_on_cpu (compiled from the reference sources into oracle/_ref) on the
     first `rows` rows of the 2:4 workload; rows are independent, so rows/M of the job."""
@@ -132,26 +196,248 @@ def cpu_baseline(case, rows):
     orc = Oracle()
     A_sub = np.ascontiguousarray(d["A_km"][:, :rows]).reshape(-1)
     B, D = d["B_cm"].reshape(-1), d["D_cm"].reshape(-1)
-    # The reference prints its thread count with printf; keep stdout for the one JSON line.
-    sys.stdout.flush()
-    saved = os.dup(1)
-    os.dup2(2, 1)
-    try:
+    with stdout_to_stderr():  # the reference prints its thread count with printf
         t0 = time.perf_counter()
         if ref is not None:
             C = ref.gemm_cpu(A_sub, B, D, rows, N, K, case.W)
         else:
             C = orc.gemm_cpu(A_sub, B, D, rows, N, case.W)
         dt = time.perf_counter() - t0
-        import ctypes
-        ctypes.CDLL(None).fflush(None)
-    finally:
-        os.dup2(saved, 1)
-        os.close(saved)
     return C.reshape(rows, N), {
         "value": 2.0 * rows * N * case.W / dt / 1e12, "unit": "TFLOP/s (useful)", "cores": orc.threads(), "kind": kind,
         "sample": "rows [0,%d) of the M=%d 2:4 workload (rows are independent), %.1f s wall" % (rows, M, dt),
     }
+
+
+class stdout_to_stderr:
+    """Keeps stdout for the one JSON line while C code that prints runs."""
+
+    def __enter__(self):
+        sys.stdout.flush()
+        self.saved = os.dup(1)
+        os.dup2(2, 1)
+
+    def __exit__(self, *exc):
+        import ctypes
+        ctypes.CDLL(None).fflush(None)
+        os.dup2(self.saved, 1)
+        os.close(self.saved)
+
+
+def tile_kernel_name(pkg, case):
+    rows = pkg.tile_wave_rows(M, N, case.W, case.kept, NS, 1)
+    if rows == 0:
+        return "spmm_direct_inner_kernel (waves along K, %d rows)" % pkg.waves_along_k_rows(M, N, case.W, case.kept)
+    qs = NS // 32
+    return "spmm_direct_kernel<%d,%d,%d,%d,%d,%s>" % (case.window, case.kept, qs, 4 // qs, rows // 32,
+                                                     "true" if case.cinfo is not None else "false")
+
+
+def profiled_traffic():
+    """HBM-side bytes per launch of the headline kernel, from the tracked rocprofv3 counter summary
+    (FETCH_SIZE and WRITE_SIZE scaled by a plain copy); None when the file does not hold it."""
+    path = os.path.join(ROOT, "profiles", "spmm_direct_kernel_4096cubed_2of4.md")
+    try:
+        m = re.search(r"traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read())
+    except OSError:
+        return None, None
+    return (float(m.group(1)), os.path.relpath(path, ROOT)) if m else (None, None)
+
+
+def run_llm(torch, pkg):
+    """Config 3: nine prefill-sized layer shapes at 2:8, the library's own split, against torch.mm fp32."""
+    rows = []
+    for (k, n_cols) in ((4096, 4096), (4096, 11008), (11008, 4096)):
+        for m_rows in (512, 2048, 8192):
+            op = GpuOperands(torch, pkg, m_rows, n_cols, k, 2, 8)
+            split = pkg.suggest_split_k(m_rows, n_cols, op.W, op.kept)
+            ms, _ = time_launches(torch, lambda: pkg.gemm_auto(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k,
+                                                               op.W, 0.75), 30, 5, 0.2)
+            fam = pkg.last_kernel()
+            a = op.A.t().contiguous()
+            b = torch.randn((k, n_cols), dtype=torch.float32, device="cuda")
+            dms, _ = time_launches(torch, lambda: torch.mm(a, b, out=op.C), 20, 3, 0.2)
+            useful = op.flops() / ms / 1e9
+            rows.append({"M": m_rows, "K": k, "Ncols": n_cols, "pattern": "2:8", "kernel": fam, "split_k": split,
+                         "waves_along_k_rows": pkg.waves_along_k_rows(m_rows, n_cols, op.W, op.kept),
+                         "ms": round(ms, 4), "useful_tflops": round(useful, 1),
+                         "frac_fp32_mfma_peak": round(useful / FP32_MFMA_PEAK_TFLOPS, 3),
+                         "dense_ms": round(dms, 4), "speedup_vs_dense": round(dms / ms, 2),
+                         "speedup_over_ideal": round(dms / ms / 4.0, 3)})
+            del op, a, b
+    return rows
+
+
+def run_decode(torch, pkg, rows_list=(1, 8, 16, 32)):
+    """Config 4.  Per case: the decode kernel on the row list and the kernel on the reference-layout
+    indices, with one B re-read by every launch (it then sits in the 256 MB Infinity Cache: "hot")
+    and with launches that walk through copies of B adding up to more than 600 MB ("cold": every
+    byte of B comes from HBM, as in a model whose layers do not fit the cache), the latter also
+    with the non-temporal hint."""
+    out = []
+    for (k, n_cols) in ((8192, 8192), (4096, 14336)):
+        for (n, m) in ((1, 8), (2, 8)):
+            op = GpuOperands(torch, pkg, 32, n_cols, k, n, m, row_list=True)
+            b_bytes = op.B.numel() * 4
+            copies = [op.B] + [op.B.clone() for _ in range(int(640e6 // b_bytes))]
+            for m_rows in rows_list:
+                a = op.A[:, :m_rows].contiguous()
+                c = torch.empty((m_rows, n_cols), dtype=torch.float32, device="cuda")
+                op.M = m_rows
+
+                def call(b, flags, rl):
+                    return lambda: pkg.spmm_ex(a, b, op.D, op.cinfo, c, m_rows, n_cols, k, op.W, op.window, op.kept, 32,
+                                               NS, 1, None, flags, op.R if rl else None)
+
+                alg = op.algorithmic_bytes()
+                entry = {"M": m_rows, "K": k, "Ncols": n_cols, "pattern": "%d:%d" % (n, m),
+                         "algorithmic_bytes": int(alg)}
+                for label, flags, rl, cold in (("hot", 0, True, False), ("cold", 0, True, True),
+                                               ("cold_stream_hint", pkg.STREAM_B, True, True),
+                                               ("hot_reference_layout", 0, False, False),
+                                               ("cold_reference_layout", 0, False, True)):
+                    calls = [call(b, flags, rl) for b in (copies if cold else [op.B] * 20)]
+                    ms = time_graph(torch, calls)
+                    if label == "hot":
+                        entry["kernel"] = pkg.last_kernel()
+                    elif label == "hot_reference_layout":
+                        entry["kernel_reference_layout"] = pkg.last_kernel()
+                    entry[label] = {"us": round(ms * 1e3, 2), "gbs": round(alg / ms / 1e6, 0),
+                                    "frac_hbm": round(alg / ms / 1e6 / HBM_PEAK_GBS, 3)}
+                out.append(entry)
+                del a, c
+            del op, copies
+    return out
+
+
+def run_fine(torch, pkg):
+    """Config 5: the n:32 patterns and 2:4 with 4-column vectors at 4096 cubed, with the device
+    preprocessing time of each (one launch for 32-column vectors, the re-blocking launch for
+    shorter ones)."""
+    out = []
+    for (n, m, vl) in ((4, 32, 32), (8, 32, 32), (16, 32, 32), (2, 4, 4)):
+        op = GpuOperands(torch, pkg, M, N, K, n, m, vec_len=vl, normal=False)
+        ms, _ = time_launches(torch, lambda: pkg.spmm(op.A, op.B, op.D, op.cinfo, op.C, M, N, K, op.W, op.window,
+                                                      op.kept, vl, NS, 1, None), 20, 3, 0.3)
+        fam = pkg.last_kernel()
+        if vl == 32:
+            pre = lambda: pkg.preprocess_device(op.DT, n, m, op.W, op.Q, N, NS, op.D, op.cinfo)
+        else:
+            pre = lambda: pkg.preprocess_low_device(op.DT, op.D, op.W, op.Q, NS, vl)
+        pre_ms, _ = time_launches(torch, pre, 20, 3, 0.05)
+        useful = op.flops() / ms / 1e9
+        out.append({"pattern": "%d:%d" % (n, m), "vec_len": vl, "kernel": fam, "ms": round(ms, 4),
+                    "useful_tflops": round(useful, 1), "frac_fp32_mfma_peak": round(useful / FP32_MFMA_PEAK_TFLOPS, 3),
+                    "preprocess_device_ms": round(pre_ms, 4), "index_bytes": int(op.D.numel() * 4)})
+        del op
+    return out
+
+
+def run_preprocess(torch, pkg, datagen):
+    """Index preprocessing of the 4096 cubed patterns four ways: (i) the one-kernel device entry,
+    (ii) the reference's call sequence (transIndex x t, then PreProcessing_*) on device-resident
+    indices, (iii) the same sequence through the host-pointer drop-in calls (wall time: each call
+    stages the indices through the GPU, PCIe both ways), (iv) on the CPU: the restatement, and the
+    reference's own host code where oracle/_ref is built."""
+    from oracle.nm_oracle import Oracle, Reference
+    orc = Oracle()
+    ref = Reference() if Reference.available() else None
+    out = []
+    for (n, m, vl) in ((2, 4, 32), (1, 8, 32), (8, 32, 32), (2, 4, 4)):
+        d = datagen.init_data(4, N, K, n, m, vec_len=vl, seed=77 + n + vl)
+        W, Q = d["W"], d["Q"]
+        if vl == 32:
+            window, kept, times = geometry(n, m)
+        else:
+            window, kept, times = m, n, 0
+        high = window == 64
+        DT0 = torch.from_numpy(d["DT"].reshape(-1).copy()).cuda()
+        DT, D = torch.empty_like(DT0), torch.empty_like(DT0)
+        cinfo = torch.empty(max(pkg.column_info_ints(W, kept, window, N, NS), 1), dtype=torch.int32, device="cuda")
+        entry = {"pattern": "%d:%d" % (n, m), "vec_len": vl, "index_bytes": int(DT0.numel() * 4)}
+
+        def sequence_device():
+            DT.copy_(DT0)
+            pn, pm = n, m
+            for _ in range(times):
+                pn, pm = pkg.trans_index_device(DT, W, N, Q, pn, pm)
+            if high:
+                pkg.preprocess_high_device(cinfo, pm, pn, DT, D, W, Q, N, NS, vl)
+            else:
+                pkg.preprocess_low_device(DT, D, W, Q, NS, vl)
+
+        if vl == 32:
+            ms, _ = time_launches(torch, lambda: pkg.preprocess_device(DT0, n, m, W, Q, N, NS, D, cinfo if high else None),
+                                  20, 3, 0.05)
+            entry["device_one_kernel_ms"] = round(ms, 4)
+        ms, _ = time_launches(torch, sequence_device, 10, 2, 0.05)
+        entry["device_reference_sequence_ms"] = round(ms, 4)
+
+        def sequence(tr, low, hi):
+            host = d["DT"].reshape(-1).copy()
+            ci = np.empty(max(pkg.column_info_ints(W, kept, window, N, NS), 1) + window, np.int32)
+            t0 = time.perf_counter()
+            pn, pm = n, m
+            for _ in range(times):
+                pn, pm = tr(host, pn, pm)
+            if high:
+                hi(ci, pm, pn, host)
+            else:
+                low(host)
+            return (time.perf_counter() - t0) * 1e3
+
+        host_ms = min(sequence(lambda h, pn, pm: pkg.trans_index_host(h, W, N, Q, pn, pm),
+                               lambda h: pkg.preprocess_low_host(h, W, Q, NS, vl),
+                               lambda ci, pm, pn, h: pkg.preprocess_high_host(ci, pm, pn, h, W, Q, N, NS, vl))
+                      for _ in range(3))
+        entry["host_pointer_dropin_wall_ms"] = round(host_ms, 3)
+        cpu_ms = min(sequence(lambda h, pn, pm: orc.trans_index(h, W, Q, pn, pm),
+                              lambda h: orc.preprocess_low(h, W, Q, NS, vl),
+                              lambda ci, pm, pn, h: orc.preprocess_high(pm, pn, h, W, Q, NS, vl))
+                     for _ in range(2))
+        entry["cpu_restatement_wall_ms"] = round(cpu_ms, 3)
+        if ref is not None and vl == 32:
+            with stdout_to_stderr():
+                ref_ms = min(sequence(lambda h, pn, pm: ref.trans_index(h, W, N, Q, pn, pm),
+                                      lambda h: ref.preprocess_low(h, W, Q, NS),
+                                      lambda ci, pm, pn, h: ref.preprocess_high(pm, pn, h, W, Q, N, NS))
+                             for _ in range(2))
+            entry["cpu_reference_wall_ms"] = round(ref_ms, 3)
+        out.append(entry)
+        del DT0, DT, D, cinfo
+    return out
+
+
+def run_dispatch(torch, pkg):
+    """The library's own choice (nmspmm_gemm_auto: split from its run-time model, kernel from the
+    shape) against the best of the splits 1, 2, 4, 8 of nmspmm_spmm, on shapes from the reference's
+    search grid (benchmark/different_kernel/search_shape/search_shape.sh:16-43) and LLM layers."""
+    shapes = [(128, 4096, 4096, 2, 4), (256, 2048, 2048, 2, 8), (256, 4096, 4096, 1, 8), (512, 4096, 4096, 2, 8),
+              (512, 1024, 1024, 2, 4), (1024, 4096, 4096, 3, 8), (1024, 5120, 5120, 2, 4), (2048, 4096, 11008, 2, 8),
+              (160, 4096, 11008, 3, 8), (768, 4096, 14336, 2, 8), (4096, 4096, 4096, 1, 8), (2048, 11008, 4096, 2, 8)]
+    rows, ratios = [], []
+    for (m_rows, n_cols, k, n, m) in shapes:
+        op = GpuOperands(torch, pkg, m_rows, n_cols, k, n, m, normal=False)
+        best = (1e9, 0)
+        for split in (1, 2, 4, 8):
+            if split > op.W // op.kept:
+                continue
+            ws = None if split == 1 else torch.empty(pkg.workspace_bytes(m_rows, n_cols, split) // 4,
+                                                     dtype=torch.float32, device="cuda")
+            ms, _ = time_launches(torch, lambda: pkg.spmm(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k, op.W,
+                                                          op.window, op.kept, 32, NS, split, ws), 20, 3, 0.1)
+            best = min(best, (ms, split))
+            del ws
+        sparsity = 1.0 - n / m
+        ms, _ = time_launches(torch, lambda: pkg.gemm_auto(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k, op.W,
+                                                           sparsity), 20, 3, 0.1)
+        ratio = ms / best[0]
+        ratios.append(ratio)
+        rows.append({"M": m_rows, "Ncols": n_cols, "K": k, "pattern": "%d:%d" % (n, m),
+                     "library_split": pkg.suggest_split_k(m_rows, n_cols, op.W, op.kept), "library_ms": round(ms, 4),
+                     "best_split": best[1], "best_ms": round(best[0], 4), "ratio": round(ratio, 3)})
+        del op
+    return {"shapes": rows, "mean_ratio": round(float(np.mean(ratios)), 3), "worst_ratio": round(float(np.max(ratios)), 3)}
 
 
 def main():
@@ -160,13 +446,25 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the CPU baseline sample (0 = skip)")
-    ap.add_argument("--headline-only", action="store_true", help="time only the 2:4 kernel (for profiling runs)")
+    ap.add_argument("--only", default="", help="comma list of parts to run beside the headline kernel: " +
+                    ", ".join(PARTS) + " (default: all; 'none' times the headline kernel alone)")
+    ap.add_argument("--headline-only", action="store_true", help="same as --only none --cpu-rows 0")
+    ap.add_argument("--decode-rows", default="1,8,16,32", help="row counts of the decode part")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy 5 times (known traffic, to scale rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this library is a single-GPU kernel library; run with --gpus 1", file=sys.stderr)
+        return 2
+    parts = set(PARTS) if not args.only else set(p for p in args.only.split(",") if p and p != "none")
+    if args.headline_only:
+        parts = set()
+    if args.cpu_rows <= 0:
+        parts.discard("cpu")
+    unknown = parts - set(PARTS)
+    if unknown:
+        print("bench.py: unknown part(s) %s" % ", ".join(sorted(unknown)), file=sys.stderr)
         return 2
 
     import torch
@@ -177,36 +475,35 @@ def main():
     pkg.lib()  # fails loudly if the HIP library is still missing: there is no fallback
     torch.cuda.set_device(0)
     torch.backends.cuda.matmul.allow_tf32 = False
+    torch.manual_seed(20240)
 
-    sweep = {}
-    head = None
-    dense_ms = None
-    for idx, (n, m) in enumerate(PATTERNS):
-        if args.headline_only and idx > 0:
-            break
-        case = Case(torch, pkg, datagen, n, m, seed=2000 + 10 * n + m)
-        ms, wall_ms = time_launches(torch, lambda: case.launch(pkg), args.steps, args.warmup)
-        assert pkg.last_kernel() == "mfma"
-        if idx == 0:
-            head = (case, ms, wall_ms)
-            if not args.headline_only:
-                Amk = case.A.t().contiguous()
-                Bd = torch.randn((K, N), dtype=torch.float32, device="cuda")
-                Cd = torch.empty((M, N), dtype=torch.float32, device="cuda")
-                dense_ms, _ = time_launches(torch, lambda: torch.mm(Amk, Bd, out=Cd), args.steps, args.warmup)
-                del Amk, Bd, Cd
-        useful = case.useful_flops() / (ms * 1e-3) / 1e12
-        entry = {"ms": round(ms, 4), "useful_tflops": round(useful, 2),
-                 "dense_equiv_tflops": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 2),
-                 "frac_fp32_mfma_peak": round(useful / FP32_MFMA_PEAK_TFLOPS, 4),
-                 "preprocess_ms": round(case.preprocess_ms, 4),
-                 "preprocess_one_kernel_ms": round(case.preprocess_one_kernel_ms, 4)}
-        if dense_ms is not None:
-            entry["speedup_vs_dense"] = round(dense_ms / ms, 3)
-            entry["speedup_over_ideal"] = round(dense_ms / ms / (m / n), 3)
-        sweep["%d:%d" % (n, m)] = entry
-        if idx > 0:
-            del case
+    # ---- headline: 2:4 at 4096 cubed -------------------------------------------------------------
+    head = Case(torch, pkg, datagen, 2, 4, seed=2024)
+    ms, wall_ms = time_launches(torch, lambda: head.launch(pkg), args.steps, args.warmup)
+    assert pkg.last_kernel() == "mfma"
+    achieved = head.useful_flops() / (ms * 1e-3) / 1e12
+    kernel_name = tile_kernel_name(pkg, head)
+
+    sweep, dense = {}, None
+    if "sweep" in parts:
+        a = head.A.t().contiguous()
+        b = torch.randn((K, N), dtype=torch.float32, device="cuda")
+        c = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        dense_ms, _ = time_launches(torch, lambda: torch.mm(a, b, out=c), args.steps, args.warmup)
+        del a, b, c
+        dense = {"ms": round(dense_ms, 4), "tflops": round(2.0 * M * N * K / (dense_ms * 1e-3) / 1e12, 2),
+                 "library": "torch.mm fp32 (rocBLAS/hipBLASLt)"}
+        for idx, (n, m) in enumerate(PATTERNS):
+            case = head if idx == 0 else Case(torch, pkg, datagen, n, m, seed=2000 + 10 * n + m)
+            cms = ms if idx == 0 else time_launches(torch, lambda: case.launch(pkg), args.steps, args.warmup, 0.5)[0]
+            useful = case.useful_flops() / (cms * 1e-3) / 1e12
+            sweep["%d:%d" % (n, m)] = {
+                "ms": round(cms, 4), "useful_tflops": round(useful, 2),
+                "dense_equiv_tflops": round(2.0 * M * N * K / (cms * 1e-3) / 1e12, 2),
+                "frac_fp32_mfma_peak": round(useful / FP32_MFMA_PEAK_TFLOPS, 4), "kernel": tile_kernel_name(pkg, case),
+                "speedup_vs_dense": round(dense_ms / cms, 3), "speedup_over_ideal": round(dense_ms / cms / (m / n), 3)}
+            if idx > 0:
+                del case
 
     if args.calibrate_copy:
         src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
@@ -216,18 +513,28 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    case, ms, wall_ms = head
-    achieved = case.useful_flops() / (ms * 1e-3) / 1e12
     cpu = None
-    if args.cpu_rows > 0:
-        case.launch(pkg)
+    if "cpu" in parts:
+        head.launch(pkg)
         torch.cuda.synchronize()
-        got = case.C[:args.cpu_rows].cpu().numpy().astype(np.float64)
-        want, cpu = cpu_baseline(case, args.cpu_rows)
+        got = head.C[:args.cpu_rows].cpu().numpy().astype(np.float64)
+        want, cpu = cpu_baseline(head, args.cpu_rows)
         want = want.astype(np.float64)
         rms = np.sqrt(np.mean(want * want))
         cpu["gpu_vs_cpu_scaled_max_error"] = float(np.max(np.abs(got - want) / np.maximum(np.abs(want), rms)))
 
+    configs = {}
+    if "llm" in parts:
+        configs["llm"] = run_llm(torch, pkg)
+    if "decode" in parts:
+        configs["decode"] = run_decode(torch, pkg, tuple(int(x) for x in args.decode_rows.split(",")))
+    if "fine" in parts:
+        configs["fine"] = run_fine(torch, pkg)
+    preprocess = run_preprocess(torch, pkg, datagen) if "preprocess" in parts else None
+    dispatch = run_dispatch(torch, pkg) if "dispatch" in parts else None
+
+    alg_bytes = 4.0 * (M * K + head.W * N + head.W * N / 32 + M * N)
+    traffic, traffic_source = profiled_traffic()
     out = {
         "metric": "useful fp32 TFLOP/s, M=Ncols=K=4096, 2:4 (vector length 32)",
         "value": round(achieved, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -237,17 +544,18 @@ def main():
                                "vector; value at 2:4, others under sweep", "tile": "Ns=128", "split_k": 1},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
-                     # bytes behind L2 per launch: rocprofv3 FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the
-                     # factors coming from a plain 256 MiB copy in the same runs
-                     # (profiles/spmm_direct_kernel_4096cubed_2of4.md)
-                     "traffic": 411.2e6, "traffic_unit": "bytes per launch", "algorithmic_bytes": 168.8e6,
-                     "kernel": "spmm_direct_kernel<32,16,4,1,8,false>", "flops_per_launch": case.useful_flops(),
+                     # HBM-side bytes per launch are a counter measurement (rocprofv3 FETCH_SIZE and
+                     # WRITE_SIZE, scaled by a plain copy), taken in its own runs and read from the
+                     # tracked summary; everything else in this object is computed in this run
+                     "traffic": traffic, "traffic_unit": "bytes per launch", "traffic_source": traffic_source,
+                     "algorithmic_bytes": alg_bytes, "kernel": kernel_name, "flops_per_launch": head.useful_flops(),
                      "launch_ms_events": round(ms, 5), "launch_ms_wall": round(wall_ms, 5)},
         "cpu_baseline": cpu,
-        "dense_fp32_gemm": None if dense_ms is None else {
-            "ms": round(dense_ms, 4), "tflops": round(2.0 * M * N * K / (dense_ms * 1e-3) / 1e12, 2),
-            "library": "torch.mm fp32 (rocBLAS/hipBLASLt)"},
+        "dense_fp32_gemm": dense,
         "sweep": sweep,
+        "configs": configs,
+        "preprocess": preprocess,
+        "dispatch": dispatch,
     }
     print(json.dumps(out))
     return 0

@@ -255,6 +255,12 @@ int nmspmm_suggest_split_k(int M, int N, int W, int kept);
  * workspace, one launch), 0 when it is computed tile by tile or the arguments are invalid.
  * Informational: the choice is the library's. */
 int nmspmm_waves_along_k_rows(int M, int N, int W, int kept);
+/* No counterpart in the reference.  Rows of C one wave of the matrix-core tile kernel covers for
+ * this shape, column-block width and split (256, 128 or 64; a workgroup is four waves: 1 x 4,
+ * 2 x 2 or 4 x 1 rows x column vectors for Ns = 128, 64, 32), 0 when the call takes the launch
+ * with waves along K (nmspmm_waves_along_k_rows) or the arguments are invalid.  Informational,
+ * for profiles and benchmarks that want to name the kernel instance that ran. */
+int nmspmm_tile_wave_rows(int M, int N, int W, int kept, int Ns, int split_k);
 int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int32_t* column_info,
                      float* C, int M, int N, int K, int W, float sparsity, void* stream);
 

@@ -75,6 +75,7 @@ def lib():
         L.nmspmm_spmm_rowmajor.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, c_void_p]
         L.nmspmm_suggest_split_k.argtypes = [c_int] * 4
         L.nmspmm_waves_along_k_rows.argtypes = [c_int] * 4
+        L.nmspmm_tile_wave_rows.argtypes = [c_int] * 6
         L.nmspmm_gemm_auto.argtypes = [c_void_p] * 5 + [c_int] * 4 + [c_float, c_void_p]
         L.nmspmm_release.restype = c_int
         _lib = L
@@ -231,6 +232,11 @@ def waves_along_k_rows(M, N, W, kept):
     """128 or 64 when an unsplit multiplication of this shape shares the reduction between the
     waves of a workgroup, 0 otherwise."""
     return lib().nmspmm_waves_along_k_rows(M, N, W, kept)
+
+
+def tile_wave_rows(M, N, W, kept, Ns=128, split_k=1):
+    """Rows per wave of the tile kernel for this call (256, 128, 64), 0 for the launch with waves along K."""
+    return lib().nmspmm_tile_wave_rows(M, N, W, kept, Ns, split_k)
 
 
 def gemm_auto(A, B, D, cinfo, C, M, N, K, W, sparsity):

@@ -690,6 +690,19 @@ int nmspmm_waves_along_k_rows(int M, int N, int W, int kept)
     return inner_split_pays(M, N, W / kept, kept) ? plan_inner(M, N, W / kept, kept).rows : 0;
 }
 
+int nmspmm_tile_wave_rows(int M, int N, int W, int kept, int Ns, int split_k)
+{
+    if (M <= 0 || N <= 0 || W <= 0 || kept <= 0 || W % kept != 0 || split_k < 1 || (Ns != 32 && Ns != 64 && Ns != 128))
+        return 0;
+    const int nwin = W / kept;
+    if (split_k == 1 && nwin >= 4 && inner_split_pays(M, N, nwin, kept))
+        return 0;  // the launch with waves along K: nmspmm_waves_along_k_rows() describes it
+    const int blocks = choose_wave_blocks(M, N, nwin, kept, split_k);
+    if (blocks == 4 && Ns == 128 && short_waves_pay(M))
+        return 64;
+    return 32 * blocks;
+}
+
 int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C,
                      int M, int N, int K, int W, float sparsity, void* stream)
 {

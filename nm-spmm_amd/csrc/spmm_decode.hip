@@ -15,9 +15,9 @@
 // four k-steps; no lane exchange, no second table, and the layout no longer depends on the window
 // geometry or on Ns.
 //
-// Kernel: one workgroup per 32-column vector, 16 waves; wave w takes the groups w, w + 16, ... (so
-// the waves of a workgroup, and with them the whole GPU, read one band of adjacent rows of B at a
-// time).  A k-step is four kept rows on v_mfma_f32_16x16x4_f32: lane (kq, jl) = (l / 16, l % 16)
+// Kernel: one workgroup per 32-column vector, 16 or 8 waves; wave w takes the groups w, w + 16,
+// ... (so the waves of a workgroup, and with them the whole GPU, read one band of adjacent rows of
+// B at a time).  A k-step is four kept rows on v_mfma_f32_16x16x4_f32: lane (kq, jl) = (l / 16, l % 16)
 // loads B[4 s + kq][2 jl .. 2 jl + 1] with one 64-bit load (four 128-byte row segments per wave and
 // instruction, each byte of B read once) and A[jl][row]; even and odd columns accumulate in two
 // MFMA tiles.  17 to 32 rows take a second pair of tiles for the other 16 rows with the same B
@@ -25,14 +25,20 @@
 // no workspace).  Measured on the MI355X: more than one group per wave in flight does not help (the
 // 16 waves of a CU keep 32 KB of B in flight, which covers the latency at the rate the fabric
 // delivers), so the loop is: load a group, multiply it.
+//
+// Every workgroup asks for the same rows of A in the same order, and the workgroups of an XCD share
+// its L2: in step, they all hit the same few cache lines (and L2 channels) at the same moment.  For
+// long reductions (W >= 2048) up to 16 rows the kernel therefore runs with 8 waves and lets
+// workgroup j of an XCD start its walk 5 j groups further on, wrapping around (measured at
+// K = Ncols = 8192, 2:8, M = 16, B resident in the Infinity Cache: 12.99 -> 12.22 us; shorter
+// reductions and the 17-to-32-row form are faster in step on 16 waves, and so is B streamed from
+// HBM, which the caller signals with the non-temporal hint).
 #include "internal.h"
 
 namespace nmspmm {
 
 typedef float dfloatx4 __attribute__((ext_vector_type(4)));
 typedef int dintx4 __attribute__((ext_vector_type(4)));
-
-constexpr int kDecodeWaves = 16;
 
 struct DecodeParams {
     const float* A;
@@ -43,6 +49,7 @@ struct DecodeParams {
     // element (i, k) of A lies i * a_row_stride + k * a_k_stride bytes into its a_bytes bytes
     uint32_t a_row_stride, a_k_stride, a_bytes, b_bytes;
     int accumulate;
+    int rotate;  // groups by which consecutive workgroups of an XCD stagger the start of their walk
 };
 
 __device__ inline __amdgpu_buffer_rsrc_t dc_rsrc(const void* base, uint32_t bytes)
@@ -53,7 +60,7 @@ __device__ inline __amdgpu_buffer_rsrc_t dc_rsrc(const void* base, uint32_t byte
 // HB: 16-row halves (1: M <= 16, 2: M <= 32).  PAIRS (HB == 2, column-major A with an even pitch):
 // one 64-bit load fetches rows 2 jl and 2 jl + 1 for the two halves, instead of two loads of rows
 // jl and jl + 16.  NT: B is loaded with the non-temporal hint (it is not kept in the caches).
-template <int HB, bool PAIRS, bool NT>
+template <int HB, bool PAIRS, bool NT, int kDecodeWaves>
 __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const DecodeParams p)
 {
     constexpr int kAux = NT ? 2 : 0;
@@ -96,17 +103,20 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
         return r;
     };
 
-    dintx4 rows = load_rows(wave);
-    for (int g = wave; g < p.G; g += kDecodeWaves) {
-        float2 b[4];
-        float a[4][HB];
-        const uint32_t b_group = b_lane + (uint32_t)g * 4u * b_step;
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            // rows at or beyond W (the tail of the last group) lie beyond the descriptor: 0
-            const auto x = __builtin_amdgcn_raw_buffer_load_b64(rb, b_group + t * b_step, 0, kAux);
-            b[t] = make_float2(__int_as_float(x[0]), __int_as_float(x[1]));
-        }
+    // this wave's groups are wave, wave + kDecodeWaves, ...: cnt of them, walked from position
+    // `first` on and around (consecutive workgroup ids go to different XCDs, so id / 8 counts the
+    // workgroups of one XCD).  Positions advance by one with a wrap: the scalar work between a
+    // group's MFMAs and the next group's loads is on every wave's critical path, so it is kept to
+    // a compare and a select.
+    const int cnt = (p.G - wave + kDecodeWaves - 1) / kDecodeWaves;
+    const int first = cnt > 0 ? (int)((blockIdx.x / 8u) * (unsigned)p.rotate % (unsigned)cnt) : 0;
+    auto after = [&](int x) { return x + 1 >= cnt ? 0 : x + 1; };
+    auto group_of = [&](int x) { return wave + x * kDecodeWaves; };
+    float2 b[4];
+    float a[4][HB];
+    // A first: its addresses come from the row list, which has landed; the four loads of B follow
+    // (measured against B first: 1 to 2 % faster)
+    auto load_operands = [&](int g, const dintx4& rows) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             if constexpr (PAIRS) {
@@ -120,7 +130,25 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
                         __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane[hb] + (uint32_t)rows[t] * a_stride, 0, 0));
             }
         }
-        rows = load_rows(g + kDecodeWaves);  // beyond the list: zeros, never used
+        __builtin_amdgcn_sched_barrier(0);
+        const uint32_t b_group = b_lane + (uint32_t)g * 4u * b_step;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            // rows at or beyond W (the tail of the last group) lie beyond the descriptor: 0
+            const auto x = __builtin_amdgcn_raw_buffer_load_b64(rb, b_group + t * b_step, 0, kAux);
+            b[t] = make_float2(__int_as_float(x[0]), __int_as_float(x[1]));
+        }
+    };
+    // Software pipeline of depth one: while a group is multiplied the next group's operands and
+    // the rows of the group after it are in flight.
+    dintx4 rows_next;
+    int x_next = after(first);  // position whose rows are in rows_next
+    if (cnt > 0) {
+        const dintx4 rows = load_rows(group_of(first));
+        rows_next = load_rows(group_of(x_next));
+        load_operands(group_of(first), rows);
+    }
+    for (int i = 0; i < cnt; ++i) {
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -128,6 +156,11 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
                 acc_e[hb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t][hb], b[t].x, acc_e[hb], 0, 0, 0);
                 acc_o[hb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t][hb], b[t].y, acc_o[hb], 0, 0, 0);
             }
+        if (i + 1 < cnt) {
+            load_operands(group_of(x_next), rows_next);
+            x_next = after(x_next);
+            rows_next = load_rows(group_of(x_next));  // after the last group: a group that is not used
+        }
     }
 
     // the waves' tiles are added in wave order.  Value x of a lane: register x % 4 of the even
@@ -187,23 +220,28 @@ hipError_t launch_decode(const SpmmArgs& a)
     p.a_bytes = (uint32_t)((size_t)(a.a_rowmajor ? a.M : a.K) * a.lda * sizeof(float));
     p.b_bytes = (uint32_t)(((size_t)(a.W - 1) * a.N + 32) * sizeof(float));
     p.accumulate = (a.accumulate && a.split_k > 1) ? 1 : 0;
-    const dim3 grid(a.N / 32), block(64 * kDecodeWaves);
+    p.rotate = 0;
+    const dim3 grid(a.N / 32), block16(64 * 16), block8(64 * 8);
     const bool pairs = a.M > 16 && !a.a_rowmajor && a.lda % 2 == 0 && a.M % 2 == 0;
     if (a.M <= 16) {
-        if (a.stream_b)
-            spmm_decode_kernel<1, false, true><<<grid, block, 0, a.stream>>>(p);
-        else
-            spmm_decode_kernel<1, false, false><<<grid, block, 0, a.stream>>>(p);
+        if (a.stream_b) {
+            spmm_decode_kernel<1, false, true, 16><<<grid, block16, 0, a.stream>>>(p);
+        } else if (a.W >= 2048) {
+            p.rotate = 5;
+            spmm_decode_kernel<1, false, false, 8><<<grid, block8, 0, a.stream>>>(p);
+        } else {
+            spmm_decode_kernel<1, false, false, 16><<<grid, block16, 0, a.stream>>>(p);
+        }
     } else if (pairs) {
         if (a.stream_b)
-            spmm_decode_kernel<2, true, true><<<grid, block, 0, a.stream>>>(p);
+            spmm_decode_kernel<2, true, true, 16><<<grid, block16, 0, a.stream>>>(p);
         else
-            spmm_decode_kernel<2, true, false><<<grid, block, 0, a.stream>>>(p);
+            spmm_decode_kernel<2, true, false, 16><<<grid, block16, 0, a.stream>>>(p);
     } else {
         if (a.stream_b)
-            spmm_decode_kernel<2, false, true><<<grid, block, 0, a.stream>>>(p);
+            spmm_decode_kernel<2, false, true, 16><<<grid, block16, 0, a.stream>>>(p);
         else
-            spmm_decode_kernel<2, false, false><<<grid, block, 0, a.stream>>>(p);
+            spmm_decode_kernel<2, false, false, 16><<<grid, block16, 0, a.stream>>>(p);
     }
     return hipGetLastError();
 }
