@@ -540,6 +540,7 @@ def main():
         "value": round(achieved, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic", "clock_prewarm_s": PREWARM_S,
+        "device": dict(zip(("compute_units", "dies", "clock_hz"), pkg.device_figures())),
         "config": {"workload": "square sweep M=Ncols=K=4096 fp32, uniform(-1,1), seeded n:m patterns per 32-column "
                                "vector; value at 2:4, others under sweep", "tile": "Ns=128", "split_k": 1},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",

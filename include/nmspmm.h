@@ -255,6 +255,12 @@ int nmspmm_suggest_split_k(int M, int N, int W, int kept);
  * workspace, one launch), 0 when it is computed tile by tile or the arguments are invalid.
  * Informational: the choice is the library's. */
 int nmspmm_waves_along_k_rows(int M, int N, int W, int kept);
+/* No counterpart in the reference.  What the library's planning (split choice, wave height, tile
+ * walk) assumes about the current device: compute units, accelerator dies (each with its own L2)
+ * and shader clock, read from the HIP runtime once per device; the figures of an MI355X
+ * (256, 8, 2.4e9) when there is no device.  Any pointer may be NULL. */
+int nmspmm_device_figures(int* compute_units, int* dies, double* clock_hz);
+
 /* No counterpart in the reference.  Rows of C one wave of the matrix-core tile kernel covers for
  * this shape, column-block width and split (256, 128 or 64; a workgroup is four waves: 1 x 4,
  * 2 x 2 or 4 x 1 rows x column vectors for Ns = 128, 64, 32), 0 when the call takes the launch

@@ -76,6 +76,7 @@ def lib():
         L.nmspmm_suggest_split_k.argtypes = [c_int] * 4
         L.nmspmm_waves_along_k_rows.argtypes = [c_int] * 4
         L.nmspmm_tile_wave_rows.argtypes = [c_int] * 6
+        L.nmspmm_device_figures.argtypes = [ip, ip, ctypes.POINTER(ctypes.c_double)]
         L.nmspmm_gemm_auto.argtypes = [c_void_p] * 5 + [c_int] * 4 + [c_float, c_void_p]
         L.nmspmm_release.restype = c_int
         _lib = L
@@ -232,6 +233,13 @@ def waves_along_k_rows(M, N, W, kept):
     """128 or 64 when an unsplit multiplication of this shape shares the reduction between the
     waves of a workgroup, 0 otherwise."""
     return lib().nmspmm_waves_along_k_rows(M, N, W, kept)
+
+
+def device_figures():
+    """(compute units, dies, clock in Hz) the library's planning assumes for the current device."""
+    cus, dies, clock = ctypes.c_int(), ctypes.c_int(), ctypes.c_double()
+    _check("nmspmm_device_figures", lib().nmspmm_device_figures(ctypes.byref(cus), ctypes.byref(dies), ctypes.byref(clock)))
+    return cus.value, dies.value, clock.value
 
 
 def tile_wave_rows(M, N, W, kept, Ns=128, split_k=1):

@@ -48,6 +48,12 @@ void* noalloc_scratch()
     return g_scratch_ptr[dev];
 }
 
+// The GPU's figures, asked once per device; without a device, an MI355X in single-partition mode.
+Machine g_machine[kMaxDevices];
+bool g_machine_known[kMaxDevices] = {};
+const Machine kDefaultMachine = {256, 8, 2.4e9};
+std::mutex g_machine_mutex;
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 size_t slice_stride(int M, int N) { return (((size_t)M * N + 3) / 4) * 4; }
@@ -101,6 +107,36 @@ struct DeviceBuf {
 };
 
 } // namespace
+
+namespace nmspmm {
+
+const Machine& machine()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return kDefaultMachine;
+    }
+    std::lock_guard<std::mutex> lock(g_machine_mutex);
+    if (!g_machine_known[dev]) {
+        Machine m = kDefaultMachine;
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+            m.cus = v;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeNumberOfXccs, dev) == hipSuccess && v > 0)
+            m.xcds = v;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeClockRate, dev) == hipSuccess && v > 0)
+            m.clock = 1e3 * v;  // reported in kHz
+        (void)hipGetLastError();
+        if (m.cus % m.xcds != 0)
+            m.xcds = 1;  // an odd partition: the walk then treats the GPU as one die
+        g_machine[dev] = m;
+        g_machine_known[dev] = true;
+    }
+    return g_machine[dev];
+}
+
+} // namespace nmspmm
 
 extern "C" {
 
@@ -455,11 +491,7 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     }
     // up to 32 rows the decode kernel always wins; up to 128 it competes with the tile kernel at
     // the caller's split
-#ifdef NMSPMM_FORCE_DECODE  // tuning builds: the decode kernel wherever it applies
-    const bool decode_wins = true;
-#else
     const bool decode_wins = model_decode_seconds(M, N, W / kept, kept) < model_tile_seconds(M, N, W / kept, kept, split_k);
-#endif
     if (skinny_supported(a) && (M <= 32 || decode_wins || !mfma_supported(a))) {
         // one launch, reduction inside the workgroup: split_k and the workspace are not needed
         e = launch_skinny(a);
@@ -688,6 +720,18 @@ int nmspmm_waves_along_k_rows(int M, int N, int W, int kept)
     if (M <= 0 || N <= 0 || W <= 0 || kept <= 0 || W % kept != 0)
         return 0;
     return inner_split_pays(M, N, W / kept, kept) ? plan_inner(M, N, W / kept, kept).rows : 0;
+}
+
+int nmspmm_device_figures(int* compute_units, int* dies, double* clock_hz)
+{
+    const Machine& m = machine();
+    if (compute_units)
+        *compute_units = m.cus;
+    if (dies)
+        *dies = m.xcds;
+    if (clock_hz)
+        *clock_hz = m.clock;
+    return NMSPMM_OK;
 }
 
 int nmspmm_tile_wave_rows(int M, int N, int W, int kept, int Ns, int split_k)

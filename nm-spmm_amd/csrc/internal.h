@@ -33,6 +33,20 @@ struct SpmmArgs {
     hipStream_t stream;
 };
 
+// What the run-time models and the tile walks need to know about the GPU: read once per device
+// from the HIP runtime (capi.hip); the figures of an MI355X in its single-partition mode when
+// there is no device to ask (the planning entry points also work without a GPU).
+struct Machine {
+    int cus;        // compute units (hipDeviceAttributeMultiprocessorCount)
+    int xcds;       // accelerator dies, each with its own L2 (hipDeviceAttributeNumberOfXccs)
+    double clock;   // shader clock in Hz (hipDeviceAttributeClockRate)
+};
+const Machine& machine();
+
+// Matrix-pipe time of one kept row of one 128-row x 128-column workgroup: 128.4 shader cycles
+// (fitted on one MI355X at 2.39 GHz: 53.5 ns), i.e. kept/2 k-steps x 4 MFMAs x 64 cycles per window.
+inline double kept_row_seconds() { return 128.4 / machine().clock; }
+
 // Windows [begin, begin + count) of reduction slice `z` out of `split_k`: an even split when it
 // divides, otherwise the first (nwin % split_k) slices take one extra window — the partition
 // rule of the reference kernels (src/kernel_64x128_8x8.cu:20-37).
@@ -50,9 +64,6 @@ __host__ __device__ inline void split_windows(int nwin, int split_k, int z, int*
 // layout is used.
 inline double tall_wave_cost(int kept) { return kept <= 8 ? 2.0 / 1.03 : 2.0 / 1.05; }
 
-#ifndef NMSPMM_TAIL_ALONG_K
-#define NMSPMM_TAIL_ALONG_K 1
-#endif
 // Whether the last layer of a launch of fewer tiles than the GPU holds at once is computed by
 // workgroups whose four waves share the reduction (four per tile, each a quarter of a tile's time
 // and alone on its CU) rather than as two 64-row pieces per tile (0.55 of a tile's time each).
@@ -63,7 +74,8 @@ inline double tall_wave_cost(int kept) { return kept <= 8 ? 2.0 / 1.03 : 2.0 / 1
 // the whole problem takes the launch with waves along K, plan_inner.)
 inline bool tail_along_k(long long tiles, int nwin)
 {
-    return NMSPMM_TAIL_ALONG_K != 0 && tiles > 256 && tiles <= 320 && nwin >= 8;
+    const long long cus = machine().cus;
+    return tiles > cus && tiles <= cus + cus / 4 && nwin >= 8;
 }
 
 // Leftover tiles of 256-row waves (two workgroups per CU) after at least one full round: `rest`
@@ -80,10 +92,11 @@ inline bool tail_along_k(long long tiles, int nwin)
 inline double tall_tail_seconds(long long rest, double unit, int* pieces, int max_pieces = 4)
 {
     static const double piece_cost[3] = {1.0, 1.04, 1.2};
+    const long long cus = machine().cus;
     double best = 2.0 * unit;
     int best_sub = 0;
     for (int i = 0, sub = 1; i < 3 && sub <= max_pieces; ++i, sub *= 2) {
-        const long long busiest = (rest * sub + 255) / 256;
+        const long long busiest = (rest * sub + cus - 1) / cus;
         const double s = busiest * unit / sub * piece_cost[i] / (busiest == 1 ? 0.9 : 1.0) + 12e-6;
         if (s < best) {
             best = s;
@@ -108,26 +121,27 @@ inline double tall_tail_seconds(long long rest, double unit, int* pieces, int ma
 // below for 128-row ones.  Constants fitted to sweeps on one MI355X (mean error 6 %).
 inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks, int split)
 {
-    const double per_window = kept * 53.5e-9 * (blocks == 8 ? tall_wave_cost(kept) : blocks == 2 ? 0.5 * 1.25 : 1.0);
+    const long long cus = machine().cus;
+    const double per_window = kept * kept_row_seconds() * (blocks == 8 ? tall_wave_cost(kept) : blocks == 2 ? 0.5 * 1.25 : 1.0);
     const double unit = per_window * ((nwin + split - 1) / split);
     const long long groups = (long long)((M + 32 * blocks - 1) / (32 * blocks)) * ((N + 127) / 128) * split;
     const int slots = blocks == 8 ? 2 : blocks == 2 ? 6 : 4;
-    const long long full = groups / (256 * slots), rest = groups % (256 * slots);
-    const long long busiest = (rest + 255) / 256;
+    const long long full = groups / (cus * slots), rest = groups % (cus * slots);
+    const long long busiest = (rest + cus - 1) / cus;
     if (blocks == 4 && split == 1) {
         // plan_tail computes the last tiles of such a launch as two 64-row pieces each.  Next to
         // whole tiles a piece costs 0.55 of a tile; alone on its CU (one 64-row wave per SIMD) it
         // hides less latency: 0.65 of a tile, 0.7 on the 1:8 geometry (in its form that loads B two
         // windows ahead)
         const double lone = kept <= 8 ? 0.7 : 0.65;
-        const long long whole = rest / 256, layer = rest % 256;
-        if (full == 0 && layer > 0 && layer <= 128) {
+        const long long whole = rest / cus, layer = rest % cus;
+        if (full == 0 && layer > 0 && layer <= cus / 2) {
             if (tail_along_k(rest, nwin))  // a quarter of a tile each, one per CU at 0.9 of the rate
                 return (whole + 0.25 / 0.9) * unit + 1e-6;
             return whole == 0 ? lone * unit : (whole + 0.55) * unit;
         }
-        if (full >= 1 && rest > 0 && rest <= 128 * slots) {
-            const long long busiest_piece = (2 * rest + 255) / 256;
+        if (full >= 1 && rest > 0 && rest <= cus / 2 * slots) {
+            const long long busiest_piece = (2 * rest + cus - 1) / cus;
             return (double)full * slots * unit + (busiest_piece == 1 ? lone : 0.55 * busiest_piece) * unit + 10e-6;
         }
     }
@@ -142,7 +156,7 @@ inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks,
         const double spread = busiest * unit / (busiest == 1 ? lone_rate : 1.0);
         if (full < 2)
             t += spread;
-        else if (split == 1 && rest <= 128 * slots)
+        else if (split == 1 && rest <= cus / 2 * slots)
             t += spread + 6e-6;  // the leftovers get a launch of their own (plan_tail)
         else
             t += slots * unit;
@@ -162,9 +176,6 @@ inline int choose_wave_blocks(int M, int N, int nwin, int kept, int split)
 {
     if (M <= 128)
         return 4;
-#ifdef NMSPMM_FORCE_BLOCKS  // tuning builds: measure one wave height everywhere
-    return NMSPMM_FORCE_BLOCKS;
-#endif
     return model_kernel_seconds(M, N, nwin, kept, 8, split) < model_kernel_seconds(M, N, nwin, kept, 4, split) ? 8 : 4;
 }
 
@@ -195,7 +206,8 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
     t.blocks = choose_wave_blocks(M, N, nwin, kept, 1);
     const int tile_rows = 32 * t.blocks * wr, tile_cols = 128 / wr;
     const long long tiles = (long long)((M + tile_rows - 1) / tile_rows) * ((N + tile_cols - 1) / tile_cols);
-    const long long slots = 256LL * (t.blocks == 8 ? 2 : 4);
+    const long long cus = machine().cus;
+    const long long slots = cus * (t.blocks == 8 ? 2 : 4);
     t.head = tiles;
     t.tail = 0;
     t.slices = 1;
@@ -215,12 +227,12 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
         // as pieces in a launch of their own they spread (+12 to +33 % at 2:8, up to +13 % at 1:8,
         // +6 to +21 % at 2:4 except around a quarter round, where whole tiles are 2 % better).
         // More than half a round left over: only its last layer, as above (+2 to +5 %).
-        const long long rest = tiles % slots, layer = tiles % 256;
+        const long long rest = tiles % slots, layer = tiles % cus;
         t.separate = true;
         t.sub = 2;
         if (tiles >= slots && rest > 0 && rest <= slots / 2) {
             t.tail = rest;  // in a launch of their own: at the end of the first they would land packed too
-        } else if (layer > 0 && layer <= 128) {
+        } else if (layer > 0 && layer <= cus / 2) {
             t.tail = layer;
             t.fused = true;
             t.along_k = tail_along_k(tiles, nwin);
@@ -237,7 +249,7 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
         return t;
     if (t.blocks == 8) {
         int pieces = 0;
-        tall_tail_seconds(rest, kept * 53.5e-9 * tall_wave_cost(kept) * nwin, &pieces, max_pieces);
+        tall_tail_seconds(rest, kept * kept_row_seconds() * tall_wave_cost(kept) * nwin, &pieces, max_pieces);
         if (pieces == 0)
             return t;
         t.separate = true;
@@ -288,19 +300,20 @@ inline InnerPlan plan_inner(int M, int N, int nwin, int kept)
     r.pays = false;
     r.rows = 128;
     r.seconds = 0.0;
+    const long long cus = machine().cus;
     const long long tiles = (long long)((M + 127) / 128) * ((N + 127) / 128);
-    if (tiles > 256 || nwin < 8 || M <= 32)
+    if (tiles > cus || nwin < 8 || M <= 32)
         return r;
     const long long vecs = N / 32;
     const long long g4 = (long long)((M + 127) / 128) * vecs, g2 = (long long)((M + 63) / 64) * vecs;
-    const long long full = g4 / 512, rest = g4 % 512, b2 = (g2 + 255) / 256;
+    const long long full = g4 / (2 * cus), rest = g4 % (2 * cus), b2 = (g2 + cus - 1) / cus;
     double c4;
     if (full == 0)
-        c4 = rest <= 256 ? 1.0 / 0.9 : 2.0;
+        c4 = rest <= cus ? 1.0 / 0.9 : 2.0;
     else
-        c4 = 2.0 * full + (rest == 0 ? 0.0 : rest <= 128 ? 1.2 : 2.0);
+        c4 = 2.0 * full + (rest == 0 ? 0.0 : rest <= cus / 2 ? 1.2 : 2.0);
     const double c2 = 0.56 * (b2 == 1 ? 1.0 / 0.9 : (double)b2);
-    const double unit = kept * 53.5e-9 * ((nwin + 3) / 4);
+    const double unit = kept * kept_row_seconds() * ((nwin + 3) / 4);
     r.pays = true;
     r.rows = c2 < c4 ? 64 : 128;
     r.seconds = (c2 < c4 ? c2 : c4) * unit + 1e-6;
@@ -345,8 +358,9 @@ inline double model_tile_seconds(int M, int N, int nwin, int kept, int split)
 inline double model_decode_seconds(int M, int N, int nwin, int kept)
 {
     const int blocks = M <= 32 ? 1 : M <= 64 ? 2 : 4;
-    const long long rounds = ((N + 31) / 32 + 255) / 256;
-    return 5e-6 + (double)rounds * nwin * kept * blocks * 4.2e-9;
+    const long long cus = machine().cus;
+    const long long rounds = ((N + 31) / 32 + cus - 1) / cus;
+    return 5e-6 + (double)rounds * nwin * kept * blocks * (10.08 / machine().clock);
 }
 
 // Matrix-core path (spmm_direct.hip).  Returns false when the geometry has no instantiation.

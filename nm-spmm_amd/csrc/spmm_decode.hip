@@ -50,6 +50,7 @@ struct DecodeParams {
     uint32_t a_row_stride, a_k_stride, a_bytes, b_bytes;
     int accumulate;
     int rotate;  // groups by which consecutive workgroups of an XCD stagger the start of their walk
+    int xcds;    // accelerator dies: consecutive workgroup ids go to consecutive dies
 };
 
 __device__ inline __amdgpu_buffer_rsrc_t dc_rsrc(const void* base, uint32_t bytes)
@@ -104,12 +105,12 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
     };
 
     // this wave's groups are wave, wave + kDecodeWaves, ...: cnt of them, walked from position
-    // `first` on and around (consecutive workgroup ids go to different XCDs, so id / 8 counts the
+    // `first` on and around (consecutive workgroup ids go to different XCDs, so id / xcds counts the
     // workgroups of one XCD).  Positions advance by one with a wrap: the scalar work between a
     // group's MFMAs and the next group's loads is on every wave's critical path, so it is kept to
     // a compare and a select.
     const int cnt = (p.G - wave + kDecodeWaves - 1) / kDecodeWaves;
-    const int first = cnt > 0 ? (int)((blockIdx.x / 8u) * (unsigned)p.rotate % (unsigned)cnt) : 0;
+    const int first = cnt > 0 ? (int)((blockIdx.x / (unsigned)p.xcds) * (unsigned)p.rotate % (unsigned)cnt) : 0;
     auto after = [&](int x) { return x + 1 >= cnt ? 0 : x + 1; };
     auto group_of = [&](int x) { return wave + x * kDecodeWaves; };
     float2 b[4];
@@ -221,6 +222,7 @@ hipError_t launch_decode(const SpmmArgs& a)
     p.b_bytes = (uint32_t)(((size_t)(a.W - 1) * a.N + 32) * sizeof(float));
     p.accumulate = (a.accumulate && a.split_k > 1) ? 1 : 0;
     p.rotate = 0;
+    p.xcds = machine().xcds;
     const dim3 grid(a.N / 32), block16(64 * 16), block8(64 * 8);
     const bool pairs = a.M > 16 && !a.a_rowmajor && a.lda % 2 == 0 && a.M % 2 == 0;
     if (a.M <= 16) {

@@ -35,9 +35,6 @@ namespace nmspmm {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int kXcds = 8;
-constexpr int kCus = 256;
-
 struct DirectParams {
     const float* A;
     const float* B;
@@ -57,6 +54,7 @@ struct DirectParams {
     int tail_offset;     // first logical tile computed in pieces along M by the workgroups after them
     int sub_tiles;       // > 1: every workgroup of this launch is one of sub_tiles pieces, along M, of a
                          // tile of sub_tiles * MS rows (the tile walk and tiles_m are those taller tiles')
+    int xcds;            // accelerator dies of the GPU: consecutive workgroup ids go to consecutive dies
 };
 
 struct float8 { float4 lo, hi; };
@@ -90,20 +88,13 @@ __device__ inline float buffer_load_f1(__amdgpu_buffer_rsrc_t r, uint32_t byte_o
     return __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, byte_off, s_off, 0));
 }
 
-// Tuning knobs (compile-time): waves per SIMD the register allocation must allow for 128-row
-// waves (256-row waves get two), and the tile-walk band height.  The 2:8 geometry (64-row windows,
-// 16 kept) would take 134 registers at three waves per SIMD, six too many for the four workgroups
-// per CU the run-time model counts on: it is compiled for four (128 registers, nothing spills;
-// the dense geometry would spill, the others are below 128 anyway).
-#ifndef NMSPMM_OCC
-#define NMSPMM_OCC 3
-#endif
-#ifndef NMSPMM_GROUP
-#define NMSPMM_GROUP 2
-#endif
-#ifndef NMSPMM_RM_TALL
-#define NMSPMM_RM_TALL 8
-#endif
+// Waves per SIMD the register allocation must allow for 128-row waves (256-row waves get two), and
+// the tile-walk band height in row tiles.  The 2:8 geometry (64-row windows, 16 kept) would take
+// 134 registers at three waves per SIMD, six too many for the four workgroups per CU the run-time
+// model counts on: it is compiled for four (128 registers, nothing spills; the dense geometry
+// would spill, the others are below 128 anyway).
+constexpr int kWavesPerSimd = 3;
+constexpr int kBandTiles = 2;
 
 // Tile shapes that exist in a second form for launches of at most one workgroup per CU, where
 // each wave has its SIMD to itself (direct_unit's DEEP).
@@ -139,7 +130,7 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
 
     // logical tile -> (tile_m, tile_n): bands of GROUP row tiles across all column blocks; with
     // sub_tiles > 1 the walk and tiles_m are those of tiles sub_tiles times as tall as MS
-    constexpr int GROUP = NMSPMM_GROUP;
+    constexpr int GROUP = kBandTiles;
     int tile_m, tile_n;
     {
         const int band = logical / (GROUP * p.tiles_n);
@@ -415,14 +406,14 @@ __device__ __forceinline__ void direct_uniform_launch(const DirectParams& p, con
         logical = p.tile_offset + id / p.tail_slices;
     } else {
         const int total = p.head_units;
-        const int q = total / kXcds, r = total % kXcds;
-        const int xcd = id % kXcds, loc = id / kXcds;
+        const int q = total / p.xcds, r = total % p.xcds;
+        const int xcd = id % p.xcds, loc = id / p.xcds;
         logical = p.tile_offset + (xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc);
     }
     direct_unit<KS, WS, QS, WR, RM, HIGH, DEEP, KW>(p, logical, sub, p.sub_tiles, tail_unit, id);
 }
 
-#define NMSPMM_DIRECT_BOUNDS __launch_bounds__(64 * QS * WR, RM == 8 ? 2 : (HIGH && WS == 16) ? 4 : NMSPMM_OCC)
+#define NMSPMM_DIRECT_BOUNDS __launch_bounds__(64 * QS * WR, RM == 8 ? 2 : (HIGH && WS == 16) ? 4 : kWavesPerSimd)
 
 template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
 __global__ void NMSPMM_DIRECT_BOUNDS spmm_direct_kernel(const DirectParams p)
@@ -485,7 +476,7 @@ __global__ void __launch_bounds__(256)
 tail_reduce_kernel(const float* __restrict__ ws, float* __restrict__ C, int M, int N, int tiles_m, int tiles_n,
                    int head_tiles, int slices)
 {
-    constexpr int GROUP = NMSPMM_GROUP;
+    constexpr int GROUP = kBandTiles;
     const int logical = head_tiles + blockIdx.x;
     const int band = logical / (GROUP * tiles_n);
     const int first_m = band * GROUP;
@@ -519,7 +510,7 @@ static hipError_t launch_uniform(const dim3 grid, const dim3 block, hipStream_t 
 {
     bool lone = false;
     if constexpr (has_lone_form<WS, RM, HIGH>())
-        lone = (long long)grid.x * grid.y <= kCus;
+        lone = (long long)grid.x * grid.y <= machine().cus;
     if (lone) {
         if constexpr (has_lone_form<WS, RM, HIGH>())
             spmm_direct_lone_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, stream>>>(p);
@@ -554,6 +545,7 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     p.tail_ws = nullptr;
     p.tail_offset = 0;
     p.sub_tiles = 1;
+    p.xcds = machine().xcds;
     // the plan counts tiles of RM blocks per wave; it applies when that is this tile shape
     const bool own_tail = plan.separate && RM == plan.blocks;
     const dim3 block(64 * QS * WR);
@@ -574,7 +566,7 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
         }
         grid.x = (unsigned)(plan.head + plan.tail * plan.sub);
         if constexpr (RM == 4) {
-            if (has_lone_form<WS, RM, HIGH>() && grid.x <= (unsigned)kCus)
+            if (has_lone_form<WS, RM, HIGH>() && grid.x <= (unsigned)machine().cus)
                 spmm_direct_mixed_kernel<KS, WS, QS, WR, RM, HIGH, has_lone_form<WS, RM, HIGH>()><<<grid, block, 0, a.stream>>>(p);
             else
                 spmm_direct_mixed_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, a.stream>>>(p);
@@ -616,23 +608,13 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     return e;
 }
 
-// Tuning builds: NMSPMM_INNER 0 never takes the launch with waves along K, 2 takes it for every
-// unsplit call (1: where the run-time model expects it to win); NMSPMM_INNER_RM 2 or 4 fixes its
-// wave height (0: the model's choice).
-#ifndef NMSPMM_INNER
-#define NMSPMM_INNER 1
-#endif
-#ifndef NMSPMM_INNER_RM
-#define NMSPMM_INNER_RM 0
-#endif
-
 // The launch with four waves along K (spmm_direct_inner_kernel), on 128- or 64-row tiles as
 // plan_inner chooses.
 template <int KS, int WS, int QS, bool HIGH>
 static hipError_t launch_inner(const SpmmArgs& a)
 {
     const long long vecs = a.N / 32;
-    const int rows = NMSPMM_INNER_RM != 0 ? NMSPMM_INNER_RM * 32 : plan_inner(a.M, a.N, a.W / WS, WS).rows;
+    const int rows = plan_inner(a.M, a.N, a.W / WS, WS).rows;
     const bool tall = rows == 128;
     DirectParams p;
     p.A = a.A;
@@ -654,12 +636,13 @@ static hipError_t launch_inner(const SpmmArgs& a)
     p.tail_ws = nullptr;
     p.tail_offset = 0;
     p.sub_tiles = 1;
+    p.xcds = machine().xcds;
     const long long groups = (long long)p.tiles_m * p.tiles_n;
     if (groups > 0x7fffffffLL)
         return hipErrorInvalidValue;
     p.head_units = (int)groups;
     const dim3 grid((unsigned)groups), block(256);
-    const bool lone = groups <= kCus;
+    const bool lone = groups <= machine().cus;
     if (tall) {
         if (lone && has_lone_form<WS, 4, HIGH>())
             spmm_direct_inner_kernel<KS, WS, QS, 4, HIGH, has_lone_form<WS, 4, HIGH>()><<<grid, block, 0, a.stream>>>(p);
@@ -691,7 +674,7 @@ static TailPlan tail_plan_for(const SpmmArgs& a, bool have_scratch)
     none.sub = 1;
     none.fused = false;
     none.along_k = false;
-    if (a.split_k != 1 || NMSPMM_RM_TALL != 8)
+    if (a.split_k != 1)
         return none;
     TailPlan t = plan_tail(a.M, a.N, a.W / a.kept, a.kept, 128 / a.Ns);
     if (t.head + t.tail * t.slices * t.sub > 0x7fffffffLL)
@@ -706,7 +689,7 @@ static TailPlan tail_plan_for(const SpmmArgs& a, bool have_scratch)
 template <int KS, int WS, bool HIGH>
 static hipError_t launch_ns(const SpmmArgs& a)
 {
-    if (a.split_k == 1 && a.W / WS >= 4 && (NMSPMM_INNER == 2 || (NMSPMM_INNER == 1 && inner_split_pays(a.M, a.N, a.W / WS, WS)))) {
+    if (a.split_k == 1 && a.W / WS >= 4 && inner_split_pays(a.M, a.N, a.W / WS, WS)) {
         switch (a.Ns) {
         case 128: return launch_inner<KS, WS, 4, HIGH>(a);
         case 64: return launch_inner<KS, WS, 2, HIGH>(a);
@@ -714,16 +697,16 @@ static hipError_t launch_ns(const SpmmArgs& a)
         }
     }
     const TailPlan plan = tail_plan_for(a, true);
-    const bool tall = NMSPMM_RM_TALL == 8 && plan.blocks == 8;
+    const bool tall = plan.blocks == 8;
     if (!tall && a.Ns == 128 && short_waves_pay(a.M))
         return launch_cfg<KS, WS, 4, 1, 2, HIGH>(a, plan);
     switch (a.Ns) {
     case 128:
-        return tall ? launch_cfg<KS, WS, 4, 1, NMSPMM_RM_TALL, HIGH>(a, plan) : launch_cfg<KS, WS, 4, 1, 4, HIGH>(a, plan);
+        return tall ? launch_cfg<KS, WS, 4, 1, 8, HIGH>(a, plan) : launch_cfg<KS, WS, 4, 1, 4, HIGH>(a, plan);
     case 64:
-        return tall ? launch_cfg<KS, WS, 2, 2, NMSPMM_RM_TALL, HIGH>(a, plan) : launch_cfg<KS, WS, 2, 2, 4, HIGH>(a, plan);
+        return tall ? launch_cfg<KS, WS, 2, 2, 8, HIGH>(a, plan) : launch_cfg<KS, WS, 2, 2, 4, HIGH>(a, plan);
     case 32:
-        return tall ? launch_cfg<KS, WS, 1, 4, NMSPMM_RM_TALL, HIGH>(a, plan) : launch_cfg<KS, WS, 1, 4, 4, HIGH>(a, plan);
+        return tall ? launch_cfg<KS, WS, 1, 4, 8, HIGH>(a, plan) : launch_cfg<KS, WS, 1, 4, 4, HIGH>(a, plan);
     }
     return hipErrorInvalidValue;
 }

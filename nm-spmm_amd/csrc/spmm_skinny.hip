@@ -74,13 +74,8 @@ template <> __device__ inline SkFrag<4> sk_load_frag<4>(__amdgpu_buffer_rsrc_t r
     return f;
 }
 
-#ifndef NMSPMM_SK_MAX_M
-#define NMSPMM_SK_MAX_M 128
-#endif
-#ifndef NMSPMM_SK_WAVES
-#define NMSPMM_SK_WAVES 8
-#endif
-constexpr int kSkinnyWaves = NMSPMM_SK_WAVES;
+constexpr int kSkinnyMaxRows = 128;
+constexpr int kSkinnyWaves = 8;
 constexpr uint32_t kSkNoLoad = 0x80000000u;
 
 // KS: dense rows per window, WS: kept rows per window, QS: column vectors per preprocessed column
@@ -455,7 +450,7 @@ static int skinny_blocks(int M) { return M <= 32 ? 1 : M <= 64 ? 2 : 4; }
 
 bool skinny_supported(const SpmmArgs& a)
 {
-    if (a.M > NMSPMM_SK_MAX_M || a.vec_len != 32 || (a.Ns != 32 && a.Ns != 64 && a.Ns != 128))
+    if (a.M > kSkinnyMaxRows || a.vec_len != 32 || (a.Ns != 32 && a.Ns != 64 && a.Ns != 128))
         return false;
     if (a.a_rowmajor) {
         // a lane then loads one float of A per k-step, whatever the pitch: the one-block forms only

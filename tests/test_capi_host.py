@@ -54,6 +54,13 @@ def test_split_suggestion():
     assert L.nmspmm_gemm_auto(FAKE, FAKE, FAKE, None, FAKE, 64, 128, 128, 64, 0.3, None) == 3
 
 
+def test_device_figures_without_a_gpu_are_those_of_an_mi355x():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present: the figures are the device's")
+    assert nmspmm.device_figures() == (256, 8, 2.4e9)
+
+
 def test_pattern_table():
     assert nmspmm.pattern_from_sparsity(0.0) == (32, 32, False)
     assert nmspmm.pattern_from_sparsity(0.5) == (32, 16, False)
