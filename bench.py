@@ -15,6 +15,8 @@ Prints ONE JSON line:
                              algorithmic GB/s against the 8 TB/s HBM bound, with B re-read from the
                              caches ("hot") and streamed from HBM ("cold"), row list on and off
                      fine    4:32, 8:32, 16:32 and 2:4 with 4-column vectors at 4096 cubed
+                     launch_constant, compress, rowmajor: the part of a launch that does not scale
+                             with K; dense <-> compressed conversion; row-major activations
   preprocess       index preprocessing: one-kernel device call, the reference's call sequence on
                    the device, the host-pointer drop-in calls (wall time, PCIe included), and the
                    CPU restatement / the reference's own host code
@@ -43,7 +45,7 @@ M = N = K = 4096
 PATTERNS = [(2, 4), (3, 8), (2, 8), (1, 8)]  # first one is the headline
 NS = 128
 GEOMETRY = {(1, 1): (32, 32), (1, 2): (32, 16), (3, 8): (32, 12), (1, 4): (64, 16), (1, 8): (64, 8)}
-PARTS = ("sweep", "llm", "decode", "fine", "preprocess", "dispatch", "cpu")
+PARTS = ("sweep", "llm", "decode", "fine", "ksweep", "compress", "rowmajor", "preprocess", "dispatch", "cpu")
 
 
 def geometry(n, m):
@@ -268,15 +270,20 @@ def run_llm(torch, pkg):
     return rows
 
 
-def run_decode(torch, pkg, rows_list=(1, 8, 16, 32)):
+DECODE_MODES = (("hot", 0, True, False), ("cold", 0, True, True), ("cold_stream_hint", 2, True, True),
+                ("hot_reference_layout", 0, False, False), ("cold_reference_layout", 0, False, True))
+
+
+def run_decode(torch, pkg, rows_list=(1, 8, 16, 32), shapes=((8192, 8192), (4096, 14336)), patterns=((1, 8), (2, 8)),
+               modes=tuple(m[0] for m in DECODE_MODES)):
     """Config 4.  Per case: the decode kernel on the row list and the kernel on the reference-layout
     indices, with one B re-read by every launch (it then sits in the 256 MB Infinity Cache: "hot")
     and with launches that walk through copies of B adding up to more than 600 MB ("cold": every
     byte of B comes from HBM, as in a model whose layers do not fit the cache), the latter also
     with the non-temporal hint."""
     out = []
-    for (k, n_cols) in ((8192, 8192), (4096, 14336)):
-        for (n, m) in ((1, 8), (2, 8)):
+    for (k, n_cols) in shapes:
+        for (n, m) in patterns:
             op = GpuOperands(torch, pkg, 32, n_cols, k, n, m, row_list=True)
             b_bytes = op.B.numel() * 4
             copies = [op.B] + [op.B.clone() for _ in range(int(640e6 // b_bytes))]
@@ -292,10 +299,9 @@ def run_decode(torch, pkg, rows_list=(1, 8, 16, 32)):
                 alg = op.algorithmic_bytes()
                 entry = {"M": m_rows, "K": k, "Ncols": n_cols, "pattern": "%d:%d" % (n, m),
                          "algorithmic_bytes": int(alg)}
-                for label, flags, rl, cold in (("hot", 0, True, False), ("cold", 0, True, True),
-                                               ("cold_stream_hint", pkg.STREAM_B, True, True),
-                                               ("hot_reference_layout", 0, False, False),
-                                               ("cold_reference_layout", 0, False, True)):
+                for label, flags, rl, cold in DECODE_MODES:
+                    if label not in modes:
+                        continue
                     calls = [call(b, flags, rl) for b in (copies if cold else [op.B] * 20)]
                     ms = time_graph(torch, calls)
                     if label == "hot":
@@ -330,6 +336,75 @@ def run_fine(torch, pkg):
                     "useful_tflops": round(useful, 1), "frac_fp32_mfma_peak": round(useful / FP32_MFMA_PEAK_TFLOPS, 3),
                     "preprocess_device_ms": round(pre_ms, 4), "index_bytes": int(op.D.numel() * 4)})
         del op
+    return out
+
+
+def run_ksweep(torch, pkg, ks=(64, 1024, 4096), patterns=((2, 4), (1, 8), (4, 32))):
+    """M = Ncols = 4096 at three reduction lengths: separates the part of a launch that does not
+    scale with K (the gap between launches, the first loads, the 64 MiB store of C) from the rate."""
+    out = []
+    for (n, m) in patterns:
+        pts = []
+        for k in ks:
+            op = GpuOperands(torch, pkg, M, N, k, n, m, normal=False)
+            ms, _ = time_launches(torch, lambda: pkg.spmm(op.A, op.B, op.D, op.cinfo, op.C, M, N, k, op.W, op.window,
+                                                          op.kept, 32, NS, 1, None), 50, 5, 0.3)
+            pts.append((k, ms, op.flops()))
+            del op
+        row = {"pattern": "%d:%d" % (n, m), "ms_at_K": {str(k): round(ms, 4) for (k, ms, _) in pts}}
+        if len(pts) >= 2:
+            (k1, t1, f1), (k2, t2, f2) = pts[-2], pts[-1]
+            rate = (f2 - f1) / ((t2 - t1) * 1e-3) / 1e12        # TFLOP/s between the two longest reductions
+            row["rate_tflops"] = round(rate, 1)
+            row["constant_us"] = round((t2 * 1e-3 - f2 / (rate * 1e12)) * 1e6, 1)  # what is left at K -> 0
+        out.append(row)
+    return out
+
+
+def run_compress(torch, pkg):
+    """Dense B -> (values, indices) and back (nmspmm_compress_device / nmspmm_decompress_device):
+    microseconds and algorithmic GB/s, 4*(K*Ncols + W*Ncols + W*Ncols/32) bytes either way."""
+    out = []
+    for (k, n_cols) in ((4096, 4096), (11008, 4096), (8192, 8192)):
+        dense = torch.randn((k, n_cols), dtype=torch.float32, device="cuda")
+        for (n, m) in ((2, 4), (2, 8), (1, 8), (8, 32)):
+            w, q = k // m * n, n_cols // 32
+            bt = torch.empty((w, n_cols), dtype=torch.float32, device="cuda")
+            dt = torch.empty((w, q), dtype=torch.int32, device="cuda")
+            back = torch.empty_like(dense)
+            nbytes = 4.0 * (k * n_cols + w * n_cols + w * q)
+            row = {"K": k, "Ncols": n_cols, "pattern": "%d:%d" % (n, m)}
+            for name, fn in (("compress", lambda: pkg.compress_device(dense, k, n_cols, n, m, bt, dt)),
+                             ("decompress", lambda: pkg.decompress_device(bt, dt, k, n_cols, n, m, back))):
+                ms, _ = time_launches(torch, fn, 30, 5, 0.05)
+                row[name] = {"us": round(ms * 1e3, 1), "gbs": round(nbytes / ms / 1e6, 0),
+                             "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 3)}
+            out.append(row)
+            del bt, dt, back
+        del dense
+    return out
+
+
+def run_rowmajor(torch, pkg):
+    """Row-major activations (nmspmm_spmm_rowmajor): the transpose into the workspace, the
+    multiplication alone, and both, on the LLM-layer shapes at 2:8 and at decode sizes."""
+    out = []
+    for (m_rows, k, n_cols) in ((512, 4096, 4096), (2048, 4096, 11008), (8192, 11008, 4096), (8, 8192, 8192),
+                                (32, 8192, 8192)):
+        op = GpuOperands(torch, pkg, m_rows, n_cols, k, 2, 8)
+        a_rm = op.A.t().contiguous()
+        split = pkg.suggest_split_k(m_rows, n_cols, op.W, op.kept)
+        ws = torch.empty(max(pkg.workspace_bytes_rowmajor(m_rows, n_cols, k, split) // 4, 4), dtype=torch.float32,
+                         device="cuda")
+        ws_cm = torch.empty(max(pkg.workspace_bytes(m_rows, n_cols, split) // 4, 4), dtype=torch.float32, device="cuda")
+        t_mm = time_graph(torch, [lambda: pkg.spmm(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k, op.W, op.window,
+                                                  op.kept, 32, NS, split, ws_cm if split > 1 else None)] * 10, 4, 0.1)
+        t_both = time_graph(torch, [lambda: pkg.spmm_rowmajor(a_rm, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k, op.W,
+                                                              op.window, op.kept, ws, 32, NS, split)] * 10, 4, 0.1)
+        out.append({"M": m_rows, "K": k, "Ncols": n_cols, "pattern": "2:8", "split_k": split,
+                    "column_major_ms": round(t_mm, 4), "row_major_ms": round(t_both, 4),
+                    "overhead": round(t_both / t_mm - 1.0, 3)})
+        del op, a_rm, ws, ws_cm
     return out
 
 
@@ -411,7 +486,9 @@ def run_preprocess(torch, pkg, datagen):
 def run_dispatch(torch, pkg):
     """The library's own choice (nmspmm_gemm_auto: split from its run-time model, kernel from the
     shape) against the best of the splits 1, 2, 4, 8 of nmspmm_spmm, on shapes from the reference's
-    search grid (benchmark/different_kernel/search_shape/search_shape.sh:16-43) and LLM layers."""
+    search grid (benchmark/different_kernel/search_shape/search_shape.sh:16-43) and LLM layers.
+    Both sides are replayed from a HIP graph of ten launches: several of these problems last about
+    ten microseconds, less than a launch from Python."""
     shapes = [(128, 4096, 4096, 2, 4), (256, 2048, 2048, 2, 8), (256, 4096, 4096, 1, 8), (512, 4096, 4096, 2, 8),
               (512, 1024, 1024, 2, 4), (1024, 4096, 4096, 3, 8), (1024, 5120, 5120, 2, 4), (2048, 4096, 11008, 2, 8),
               (160, 4096, 11008, 3, 8), (768, 4096, 14336, 2, 8), (4096, 4096, 4096, 1, 8), (2048, 11008, 4096, 2, 8)]
@@ -424,13 +501,13 @@ def run_dispatch(torch, pkg):
                 continue
             ws = None if split == 1 else torch.empty(pkg.workspace_bytes(m_rows, n_cols, split) // 4,
                                                      dtype=torch.float32, device="cuda")
-            ms, _ = time_launches(torch, lambda: pkg.spmm(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k, op.W,
-                                                          op.window, op.kept, 32, NS, split, ws), 20, 3, 0.1)
+            ms = time_graph(torch, [lambda: pkg.spmm(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k, op.W,
+                                                     op.window, op.kept, 32, NS, split, ws)] * 10, 4, 0.1)
             best = min(best, (ms, split))
             del ws
         sparsity = 1.0 - n / m
-        ms, _ = time_launches(torch, lambda: pkg.gemm_auto(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k, op.W,
-                                                           sparsity), 20, 3, 0.1)
+        ms = time_graph(torch, [lambda: pkg.gemm_auto(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k, op.W,
+                                                      sparsity)] * 10, 4, 0.1)
         ratio = ms / best[0]
         ratios.append(ratio)
         rows.append({"M": m_rows, "Ncols": n_cols, "K": k, "pattern": "%d:%d" % (n, m),
@@ -450,6 +527,12 @@ def main():
                     ", ".join(PARTS) + " (default: all; 'none' times the headline kernel alone)")
     ap.add_argument("--headline-only", action="store_true", help="same as --only none --cpu-rows 0")
     ap.add_argument("--decode-rows", default="1,8,16,32", help="row counts of the decode part")
+    ap.add_argument("--decode-shapes", default="8192x8192,4096x14336", help="K x Ncols of the decode part")
+    ap.add_argument("--decode-patterns", default="1:8,2:8", help="patterns of the decode part")
+    ap.add_argument("--decode-modes", default=",".join(m[0] for m in DECODE_MODES),
+                    help="which of hot, cold, cold_stream_hint, hot_reference_layout, cold_reference_layout to time")
+    ap.add_argument("--ksweep-ks", default="64,1024,4096", help="reduction lengths of the ksweep part")
+    ap.add_argument("--ksweep-patterns", default="2:4,1:8,4:32", help="patterns of the ksweep part")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy 5 times (known traffic, to scale rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters)")
@@ -527,9 +610,21 @@ def main():
     if "llm" in parts:
         configs["llm"] = run_llm(torch, pkg)
     if "decode" in parts:
-        configs["decode"] = run_decode(torch, pkg, tuple(int(x) for x in args.decode_rows.split(",")))
+        configs["decode"] = run_decode(
+            torch, pkg, tuple(int(x) for x in args.decode_rows.split(",")),
+            tuple(tuple(int(v) for v in x.split("x")) for x in args.decode_shapes.split(",")),
+            tuple(tuple(int(v) for v in x.split(":")) for x in args.decode_patterns.split(",")),
+            tuple(args.decode_modes.split(",")))
     if "fine" in parts:
         configs["fine"] = run_fine(torch, pkg)
+    if "ksweep" in parts:
+        configs["launch_constant"] = run_ksweep(
+            torch, pkg, tuple(int(x) for x in args.ksweep_ks.split(",")),
+            tuple(tuple(int(v) for v in x.split(":")) for x in args.ksweep_patterns.split(",")))
+    if "compress" in parts:
+        configs["compress"] = run_compress(torch, pkg)
+    if "rowmajor" in parts:
+        configs["rowmajor"] = run_rowmajor(torch, pkg)
     preprocess = run_preprocess(torch, pkg, datagen) if "preprocess" in parts else None
     dispatch = run_dispatch(torch, pkg) if "dispatch" in parts else None
 
