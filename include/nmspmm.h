@@ -220,6 +220,13 @@ int nmspmm_spmm_rowmajor(const float* A_rowmajor, const float* B, const int32_t*
                          const int32_t* column_info, float* C, int M, int N, int K, int W, int window,
                          int kept, int vec_len, int Ns, int split_k, void* workspace,
                          size_t workspace_bytes, void* stream);
+/* The same with the optional row list and the flags of nmspmm_spmm_ex (up to 8 rows the decode
+ * kernel on the row list reads the row-major A in place, like the kernel it replaces). */
+int nmspmm_spmm_rowmajor_ex(const float* A_rowmajor, const float* B, const int32_t* D,
+                            const int32_t* column_info, const int32_t* row_index, float* C, int M,
+                            int N, int K, int W, int window, int kept, int vec_len, int Ns,
+                            int split_k, void* workspace, size_t workspace_bytes, unsigned flags,
+                            void* stream);
 
 /* Replace the reference launchers nmGEMM_{small,medium,large,huge}_matrices_low_sparsity
  * (reference include/NM-SpMM.h:14,17,20,23) and ..._high_sparsity (:15,18,21,24): `tile` is the

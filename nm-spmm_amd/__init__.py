@@ -73,6 +73,7 @@ def lib():
         L.nmspmm_workspace_bytes_rowmajor.restype = c_size_t
         L.nmspmm_workspace_bytes_rowmajor.argtypes = [c_int] * 4
         L.nmspmm_spmm_rowmajor.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, c_void_p]
+        L.nmspmm_spmm_rowmajor_ex.argtypes = [c_void_p] * 6 + [c_int] * 9 + [c_void_p, c_size_t, ctypes.c_uint, c_void_p]
         L.nmspmm_suggest_split_k.argtypes = [c_int] * 4
         L.nmspmm_waves_along_k_rows.argtypes = [c_int] * 4
         L.nmspmm_tile_wave_rows.argtypes = [c_int] * 6
@@ -217,12 +218,13 @@ def workspace_bytes_rowmajor(M, N, K, split_k):
     return lib().nmspmm_workspace_bytes_rowmajor(M, N, K, split_k)
 
 
-def spmm_rowmajor(A_rm, B, D, cinfo, C, M, N, K, W, window, kept, workspace, vec_len=32, Ns=128, split_k=1):
+def spmm_rowmajor(A_rm, B, D, cinfo, C, M, N, K, W, window, kept, workspace, vec_len=32, Ns=128, split_k=1,
+                  row_index=None, flags=0):
     """A_rm is row-major M x K; `workspace` (float32 tensor) holds workspace_bytes_rowmajor() bytes."""
-    _check("nmspmm_spmm_rowmajor",
-           lib().nmspmm_spmm_rowmajor(_ptr(A_rm), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(C), M, N, K, W, window, kept,
-                                      vec_len, Ns, split_k, _ptr(workspace), workspace.numel() * workspace.element_size(),
-                                      _stream()))
+    _check("nmspmm_spmm_rowmajor_ex",
+           lib().nmspmm_spmm_rowmajor_ex(_ptr(A_rm), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(row_index), _ptr(C), M, N, K, W,
+                                         window, kept, vec_len, Ns, split_k, _ptr(workspace),
+                                         workspace.numel() * workspace.element_size(), flags, _stream()))
 
 
 def suggest_split_k(M, N, W, kept):

@@ -541,10 +541,13 @@ size_t nmspmm_workspace_bytes_rowmajor(int M, int N, int K, int split_k)
     return sizeof(float) * rowmajor_copy_floats(M, K) + nmspmm_workspace_bytes(M, N, split_k);
 }
 
-int nmspmm_spmm_rowmajor(const float* A_rowmajor, const float* B, const int32_t* D, const int32_t* column_info,
-                         float* C, int M, int N, int K, int W, int window, int kept, int vec_len, int Ns,
-                         int split_k, void* workspace, size_t workspace_bytes, void* stream)
+int nmspmm_spmm_rowmajor_ex(const float* A_rowmajor, const float* B, const int32_t* D, const int32_t* column_info,
+                            const int32_t* row_index, float* C, int M, int N, int K, int W, int window, int kept,
+                            int vec_len, int Ns, int split_k, void* workspace, size_t workspace_bytes, unsigned flags,
+                            void* stream)
 {
+    if (row_index && ((uintptr_t)row_index & 15u))
+        return NMSPMM_ERR_ALIGNMENT;
     if (!A_rowmajor)
         return NMSPMM_ERR_NULL_POINTER;
     if (M <= 0 || N <= 0 || K <= 0 || (M + 63) / 64 > 65535)
@@ -561,20 +564,28 @@ int nmspmm_spmm_rowmajor(const float* A_rowmajor, const float* B, const int32_t*
     // costs 2.5 to 4 us at these sizes: level up to 8 rows, 0.4 to 2 times slower from 16 on.)
     if (M <= 8 && aligned16(A_rowmajor)) {
         const int st = spmm_impl(A_rowmajor, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k,
-                                 slices, slice_bytes, stream, K, false, nullptr, true);
+                                 slices, slice_bytes, stream, K, false, nullptr, true, flags, row_index);
         if (st != kNotTaken)
             return st;
     }
     // check every argument and settle the row pitch of the copy before anything is launched
     int lda = M;
     const int st = spmm_impl(At, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k, slices,
-                             slice_bytes, stream, 0, true, &lda);
+                             slice_bytes, stream, 0, true, &lda, false, flags, row_index);
     if (st != NMSPMM_OK)
         return st;
     if (launch_transpose(A_rowmajor, At, M, K, lda, (hipStream_t)stream) != hipSuccess)
         return NMSPMM_ERR_HIP;
     return spmm_impl(At, B, D, column_info, C, M, N, K, W, window, kept, vec_len, Ns, split_k, slices, slice_bytes,
-                     stream, lda, false, nullptr);
+                     stream, lda, false, nullptr, false, flags, row_index);
+}
+
+int nmspmm_spmm_rowmajor(const float* A_rowmajor, const float* B, const int32_t* D, const int32_t* column_info,
+                         float* C, int M, int N, int K, int W, int window, int kept, int vec_len, int Ns,
+                         int split_k, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return nmspmm_spmm_rowmajor_ex(A_rowmajor, B, D, column_info, nullptr, C, M, N, K, W, window, kept, vec_len, Ns,
+                                   split_k, workspace, workspace_bytes, 0, stream);
 }
 
 int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C, int M,

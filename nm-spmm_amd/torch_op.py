@@ -59,9 +59,13 @@ class NMSparseLinear(torch.nn.Module):
                                 device=weight.device)
         got = _nm.preprocess_device(DT, n, m, self.W, self.Q, N, self.Ns, D, cinfo)
         assert got == (self.window, self.kept)
+        # the row list: the index form the decode kernel (up to 32 rows) reads
+        rows = torch.empty(_nm.row_index_ints(self.W, N), dtype=torch.int32, device=weight.device)
+        _nm.row_index_device(D, cinfo, self.W, N, self.window, self.kept, self.Ns, rows)
         self.register_buffer("values", BT)
         self.register_buffer("indices", D.reshape(-1))
         self.register_buffer("column_info", cinfo)
+        self.register_buffer("row_index", rows)
         self.register_buffer("bias", None if bias is None else bias.detach().to(torch.float32))
         self._workspace = None
         self._plans = {}
@@ -89,7 +93,7 @@ class NMSparseLinear(torch.nn.Module):
         if self._workspace is None or self._workspace.numel() < need or self._workspace.device != x.device:
             self._workspace = torch.empty(need, dtype=torch.float32, device=x.device)
         _nm.spmm_rowmajor(x2, self.values, self.indices, self.column_info, y, M, N, K, self.W, self.window, self.kept,
-                          self._workspace, 32, self.Ns, split)
+                          self._workspace, 32, self.Ns, split, self.row_index)
         if add_bias and self.bias is not None:
             y += self.bias
         return y.reshape(*lead, N)

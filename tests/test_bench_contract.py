@@ -39,3 +39,31 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert c["kind"] in ("reference", "port") and c["cores"] >= 1 and c["value"] > 0
     assert c["gpu_vs_cpu_scaled_max_error"] <= 1e-4
     assert set(d["sweep"]) == {"2:4", "3:8", "2:8", "1:8"}
+    # every baseline workload is timed in the same run
+    assert r["traffic_source"].startswith("profiles/") and r["traffic"] > r["algorithmic_bytes"] > 0
+    assert r["kernel"].startswith("spmm_direct_kernel<32,16,4,1,")
+    cfg = d["configs"]
+    assert len(cfg["llm"]) == 9 and all(x["kernel"] == "mfma" and x["speedup_vs_dense"] > 1 for x in cfg["llm"])
+    assert len(cfg["decode"]) == 16
+    for x in cfg["decode"]:
+        assert x["kernel"] == "decode" and x["kernel_reference_layout"] == "skinny"
+        for mode in ("hot", "cold", "cold_stream_hint", "hot_reference_layout", "cold_reference_layout"):
+            assert 0 < x[mode]["frac_hbm"] < 1.5 and x[mode]["us"] > 0
+    assert [x["pattern"] for x in cfg["fine"]] == ["4:32", "8:32", "16:32", "2:4"] and cfg["fine"][3]["vec_len"] == 4
+    assert len(cfg["launch_constant"]) == 3 and len(cfg["compress"]) == 12 and len(cfg["rowmajor"]) == 5
+    for x in d["preprocess"]:
+        assert x["host_pointer_dropin_wall_ms"] > 0 and x["cpu_restatement_wall_ms"] > 0
+        assert x["device_reference_sequence_ms"] > 0
+    assert len(d["dispatch"]["shapes"]) == 12 and d["dispatch"]["mean_ratio"] < 1.1
+    assert d["device"]["compute_units"] > 0 and d["device"]["dies"] > 0
+
+
+@pytest.mark.gpu
+def test_parts_can_be_selected():
+    out = subprocess.run([sys.executable, BENCH, "--steps", "5", "--warmup", "1", "--only", "fine", "--cpu-rows", "0"],
+                         capture_output=True, text=True, timeout=600)
+    assert out.returncode == 0, out.stderr
+    d = json.loads(out.stdout.strip())
+    assert list(d["configs"]) == ["fine"] and d["cpu_baseline"] is None and d["sweep"] == {} and d["dispatch"] is None
+    bad = subprocess.run([sys.executable, BENCH, "--only", "nonsense"], capture_output=True, text=True, timeout=120)
+    assert bad.returncode != 0 and "unknown part" in bad.stderr

@@ -169,3 +169,24 @@ def test_graph_replays_of_the_decode_kernel_equal_eager_calls(oracle, M, n, m):
         call(C_e)
         torch.cuda.synchronize()
         assert torch.isfinite(C_g).all().item() and torch.equal(C_g, C_e), "replay %d" % rep
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 9, 16, 21, 32])
+@pytest.mark.parametrize("n,m", [(1, 8), (2, 4)])
+def test_row_major_activations_on_the_row_list(oracle, M, n, m):
+    """nmspmm_spmm_rowmajor_ex with the row list: up to 8 rows the decode kernel reads the
+    row-major A in place, above that the column-major copy in the workspace (pitch padded to four
+    floats for odd row counts)."""
+    N, K = 256, 1024
+    d = datagen.init_data(M, N, K, n, m, seed=M + n, dist="normal", b_scale=0.02)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    R = gpu_row_list(D, cinfo, d["W"], N, window, kept, 128)
+    A_rm = dev(d["A_km"].T)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    ws = torch.full((nmspmm.workspace_bytes_rowmajor(M, N, K, 1) // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    nmspmm.spmm_rowmajor(A_rm, dev(d["BT"]), dev(D), None if cinfo is None else dev(cinfo), C, M, N, K, d["W"], window,
+                         kept, ws, 32, 128, 1, R)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == "decode"
+    got = C.cpu().numpy()
+    assert np.isfinite(got).all() and scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
