@@ -707,7 +707,7 @@ int nmspmm_suggest_split_k(int M, int N, int W, int kept)
     if (M <= 32)
         return 1;  // the decode kernel reduces inside its workgroups
     // The split with the smallest modelled time of the tile kernel (model_tile_seconds); a finer
-    // split has to win by 3 %.  Fitted to sweeps of M in 48..4096, N and K in 512..14336 at 2:4,
+    // split has to win by 5 %.  Fitted to sweeps of M in 48..4096, N and K in 512..14336 at 2:4,
     // 3:8, 2:8 and 1:8 on one MI355X: the choice is within 1 % of the best split on average, where
     // never splitting loses 32 %.  Up to 128 rows the one-launch decode kernel is the alternative;
     // where its model is faster no split is needed.
@@ -716,7 +716,7 @@ int nmspmm_suggest_split_k(int M, int N, int W, int kept)
     double best_t = 0.0;
     for (int split = 1; split <= 16 && split <= nwin; split *= 2) {
         const double t = model_tile_seconds(M, N, nwin, kept, split);
-        if (split == 1 || t < 0.97 * best_t) {
+        if (split == 1 || t < 0.95 * best_t) {
             best = split;
             best_t = t;
         }

@@ -283,12 +283,12 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
 // added in LDS.  It cuts the reduction without scratch or a second pass, for problems of at most
 // 256 tiles of 128 x 128 (measured on 96 shapes, M = 192 ... 1024, against the best of the splits
 // 1, 2, 4, 8 of the tile kernel: 2 to 56 % faster up to 256 tiles, 0 to 16 % slower at 512).
-// Two workgroups of 128-row waves fit a CU (64 KB of LDS each), so they retire in rounds of 512:
-// up to 256 run one per CU (at 0.9 of the rate, one wave per SIMD), up to 512 two per CU, and the
-// leftovers of full rounds land two per CU on the CUs that free up first (768 workgroups take as
-// long as 1024, measured) unless they are at most 128 (then 1.2 of a workgroup's time, measured).
-// Workgroups of 64-row waves (32 KB) spread evenly, a layer per 256, and cost 0.56 of the taller
-// ones each.
+// Two workgroups of 128-row waves fit a CU (64 KB of LDS each): a layer of up to one per CU costs
+// 1.17 of a workgroup's time (one wave per SIMD; 1.3 behind full pairs of layers), two layers
+// together 2.16.  Workgroups of 64-row
+// waves (32 KB) cost 0.56 of a taller one per layer, 0.62 when there is only one layer.  Both
+// measured on 144 shapes (M = 160 ... 1024, four patterns, reductions of 2048 to 14336) with each
+// form forced; the choice between them then lands within 1 % of the better one on average.
 struct InnerPlan {
     bool pays;     // eligible at all
     int rows;      // 128 or 64 rows per workgroup
@@ -306,12 +306,8 @@ inline InnerPlan plan_inner(int M, int N, int nwin, int kept)
         return r;
     const long long vecs = N / 32;
     const long long g4 = (long long)((M + 127) / 128) * vecs, g2 = (long long)((M + 63) / 64) * vecs;
-    const long long full = g4 / (2 * cus), rest = g4 % (2 * cus), b2 = (g2 + cus - 1) / cus;
-    double c4;
-    if (full == 0)
-        c4 = rest <= cus ? 1.0 / 0.9 : 2.0;
-    else
-        c4 = 2.0 * full + (rest == 0 ? 0.0 : rest <= cus / 2 ? 1.2 : 2.0);
+    const long long b4 = (g4 + cus - 1) / cus, b2 = (g2 + cus - 1) / cus;
+    const double c4 = 2.16 * (double)(b4 / 2) + (b4 % 2 ? (b4 == 1 ? 1.17 : 1.3) : 0.0);
     const double c2 = 0.56 * (b2 == 1 ? 1.0 / 0.9 : (double)b2);
     const double unit = kept * kept_row_seconds() * ((nwin + 3) / 4);
     r.pays = true;
