@@ -28,11 +28,12 @@
 //
 // Every workgroup asks for the same rows of A in the same order, and the workgroups of an XCD share
 // its L2: in step, they all hit the same few cache lines (and L2 channels) at the same moment.  For
-// long reductions (W >= 2048) up to 16 rows the kernel therefore runs with 8 waves and lets
+// long reductions (W >= 2048) of 8 to 16 rows the kernel therefore runs with 8 waves and lets
 // workgroup j of an XCD start its walk 5 j groups further on, wrapping around (measured at
-// K = Ncols = 8192, 2:8, M = 16, B resident in the Infinity Cache: 12.99 -> 12.22 us; shorter
-// reductions and the 17-to-32-row form are faster in step on 16 waves, and so is B streamed from
-// HBM, which the caller signals with the non-temporal hint).
+// K = Ncols = 8192, 2:8, M = 16, B resident in the Infinity Cache: 12.99 -> 12.22 us; with B
+// streamed from HBM the 16 waves in step are 3 to 5 % ahead, which the caller can ask for with the
+// non-temporal hint).  Fewer rows gather little of A and run faster on 16 waves either way, and so
+// do shorter reductions and the 17-to-32-row form.
 #include "internal.h"
 
 namespace nmspmm {
@@ -78,16 +79,20 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
     const __amdgpu_buffer_rsrc_t rr = dc_rsrc(p.R + (size_t)v * p.G * 16, (uint32_t)p.G * 64u);
     const __amdgpu_buffer_rsrc_t ra = dc_rsrc(p.A, p.a_bytes);
     const uint32_t a_stride = p.a_k_stride;
-    // the list holds row + 1: entry 0 (no such kept row, or a read beyond the list) puts the offset
-    // below zero, which is out of range and loads 0; so does a lane whose row of C does not exist
+    // Lanes whose row of C does not exist read the last row that does (their tile rows are never
+    // stored): out-of-range lanes would be dropped by the descriptor as well, but loads with most
+    // lanes out of range are slow (M = 1, B streamed from HBM: 17.3 -> 13.6 us at K = Ncols = 8192,
+    // 2:8).  The list holds row + 1; entry 0 (no such kept row, or a read beyond the list) selects
+    // an offset beyond the descriptor, which loads 0.
     uint32_t a_lane[HB];
     if (PAIRS) {
-        a_lane[0] = (2 * jl < M ? (uint32_t)jl * 8u : 0x80000000u) - a_stride;
+        a_lane[0] = (uint32_t)min(jl, M / 2 - 1) * 8u - a_stride;
     } else {
 #pragma unroll
         for (int hb = 0; hb < HB; ++hb)
-            a_lane[hb] = (jl + 16 * hb < M ? (uint32_t)(jl + 16 * hb) * p.a_row_stride : 0x80000000u) - a_stride;
+            a_lane[hb] = (uint32_t)min(jl + 16 * hb, M - 1) * p.a_row_stride - a_stride;
     }
+    auto a_offset = [&](uint32_t lane_part, int row) { return row > 0 ? lane_part + (uint32_t)row * a_stride : 0x80000000u; };
     const uint32_t b_lane = (uint32_t)(((size_t)kq * N + 2 * jl) * sizeof(float));
     const uint32_t b_step = (uint32_t)((size_t)4 * N * sizeof(float));
 
@@ -121,14 +126,14 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             if constexpr (PAIRS) {
-                const auto x = __builtin_amdgcn_raw_buffer_load_b64(ra, a_lane[0] + (uint32_t)rows[t] * a_stride, 0, 0);
+                const auto x = __builtin_amdgcn_raw_buffer_load_b64(ra, a_offset(a_lane[0], rows[t]), 0, 0);
                 a[t][0] = __int_as_float(x[0]);
                 a[t][1] = __int_as_float(x[1]);
             } else {
 #pragma unroll
                 for (int hb = 0; hb < HB; ++hb)
                     a[t][hb] = __int_as_float(
-                        __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane[hb] + (uint32_t)rows[t] * a_stride, 0, 0));
+                        __builtin_amdgcn_raw_buffer_load_b32(ra, a_offset(a_lane[hb], rows[t]), 0, 0));
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -228,7 +233,7 @@ hipError_t launch_decode(const SpmmArgs& a)
     if (a.M <= 16) {
         if (a.stream_b) {
             spmm_decode_kernel<1, false, true, 16><<<grid, block16, 0, a.stream>>>(p);
-        } else if (a.W >= 2048) {
+        } else if (a.W >= 2048 && a.M >= 8) {
             p.rotate = 5;
             spmm_decode_kernel<1, false, false, 8><<<grid, block8, 0, a.stream>>>(p);
         } else {

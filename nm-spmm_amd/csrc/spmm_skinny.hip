@@ -76,7 +76,6 @@ template <> __device__ inline SkFrag<4> sk_load_frag<4>(__amdgpu_buffer_rsrc_t r
 
 constexpr int kSkinnyMaxRows = 128;
 constexpr int kSkinnyWaves = 8;
-constexpr uint32_t kSkNoLoad = 0x80000000u;
 
 // KS: dense rows per window, WS: kept rows per window, QS: column vectors per preprocessed column
 // block, HIGH: high-sparsity layout, RB: 32-row blocks per wave, U: windows per chunk (all loads
@@ -110,7 +109,9 @@ spmm_skinny_kernel(const SkinnyParams p)
     const int32_t* const Dblk = p.D + (size_t)jb * p.W * QS;
     const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)jb * p.nwin * KS : nullptr;
     const uint32_t a_bytes = p.a_bytes;
-    const uint32_t a_lane = RB * j < M ? (uint32_t)(RB * j) * p.a_row_stride : kSkNoLoad;
+    // lanes beyond the last row read the last fragment that exists (their tile rows are never stored):
+    // loads with most lanes out of range are slow
+    const uint32_t a_lane = (uint32_t)min(RB * j, (M - 1) / RB * RB) * p.a_row_stride;
     const uint32_t row_bytes = p.a_k_stride;
     const uint32_t b_lane = (uint32_t)(((size_t)h * N + j) * sizeof(float));
     const uint32_t b_step = (uint32_t)(2 * (size_t)N * sizeof(float));
@@ -275,7 +276,9 @@ spmm_skinny16_kernel(const SkinnyParams p)
     const int32_t* const Dblk = p.D + (size_t)jb * p.W * QS;
     const int32_t* const Cinfo = HIGH ? p.cinfo + (size_t)jb * p.nwin * KS : nullptr;
     const uint32_t a_bytes = p.a_bytes;
-    const uint32_t a_lane = jl < M ? (uint32_t)jl * p.a_row_stride : kSkNoLoad;
+    // lanes beyond the last row read the last row (their tile rows are never stored): loads with most
+    // lanes out of range are slow
+    const uint32_t a_lane = (uint32_t)min(jl, M - 1) * p.a_row_stride;
     const uint32_t row_bytes = p.a_k_stride;
     const uint32_t b_lane = (uint32_t)(((size_t)kq * N + 2 * jl) * sizeof(float));
     const uint32_t b_step = (uint32_t)(4 * (size_t)N * sizeof(float));
