@@ -74,6 +74,35 @@ def test_decode_kernel_every_row_count(oracle, M, n, m, K):
     assert np.isfinite(got).all() and scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
 
 
+@pytest.mark.parametrize("M", [1, 3, 9, 16, 19, 26])
+@pytest.mark.parametrize("n,m,K", [(2, 8, 1088), (3, 8, 96), (1, 8, 2048)])
+def test_nothing_outside_a_leaks_into_c(oracle, M, n, m, K):
+    """The lanes of a 16-row tile whose row of C does not exist read the last row that does, and
+    the last group of a reduction that is not whole groups has entries without a row: neither may
+    bring anything from outside A into C.  A lies in the middle of a buffer of NaNs."""
+    d = datagen.init_data(M, 128, K, n, m, seed=3 * M + K, dist="normal", b_scale=0.02)
+    N, W = d["N"], d["W"]
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    R = gpu_row_list(D, cinfo, W, N, window, kept, 128)
+    pad = 4096
+    buf = torch.full((2 * pad + K * M,), float("nan"), dtype=torch.float32, device="cuda")
+    buf[pad:pad + K * M] = dev(d["A_km"]).reshape(-1)
+    A = buf[pad:pad + K * M]
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    nmspmm.spmm_ex(A, dev(d["BT"]), dev(D), None if cinfo is None else dev(cinfo), C, M, N, K, W, window, kept, 32, 128,
+                   1, None, 0, R)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == "decode"
+    got = C.cpu().numpy()
+    assert np.isfinite(got).all() and scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
+    # and on the reference layout (no list)
+    C.fill_(float("nan"))
+    nmspmm.spmm(A, dev(d["BT"]), dev(D), None if cinfo is None else dev(cinfo), C, M, N, K, W, window, kept, 32, 128, 1, None)
+    torch.cuda.synchronize()
+    got = C.cpu().numpy()
+    assert np.isfinite(got).all() and scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
+
+
 @pytest.mark.parametrize("Ns", [64, 32])
 @pytest.mark.parametrize("M,n,m", [(5, 1, 8), (32, 2, 8), (16, 2, 4)])
 def test_decode_kernel_with_lists_from_other_block_widths(oracle, Ns, M, n, m):
