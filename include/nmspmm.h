@@ -95,7 +95,9 @@ int nmspmm_preprocess_high_device(int32_t* d_column_info, int pruning_M, int pru
  * after the other) are folded into the re-blocking / ranking pass.  dD_out and, for the
  * high-sparsity geometries, d_column_info receive exactly what the separate calls produce;
  * *window and *kept are what nmspmm_spmm then takes.  dDT_in is not modified.  n/m must reduce to
- * 1/1, 1/2, 3/8, 1/4 or 1/8 with m a power-of-two fraction of the kernel window. */
+ * 1/1, 1/2, 3/8, 1/4 or 1/8 with m a power-of-two fraction of the kernel window.  With vectors
+ * of 4, 8 or 16 columns (N / Q below 32) the kernels take the window as generated: the call
+ * re-blocks, *window = m, *kept = n, d_column_info is not used. */
 int nmspmm_preprocess_device(const int32_t* dDT_in, int n, int m, int W, int Q, int N, int Ns,
                              int32_t* dD_out, int32_t* d_column_info, int* window, int* kept,
                              void* stream);
@@ -281,7 +283,7 @@ int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int
 int nmspmm_release(void);
 
 /* Name of the kernel family the last successful nmspmm_spmm call on this thread dispatched to
- * ("mfma", "short", "skinny", "decode", "simt"), for tests and profiles.  Never NULL. */
+ * ("mfma", "short", "gather", "skinny", "decode", "simt"), for tests and profiles.  Never NULL. */
 const char* nmspmm_last_kernel(void);
 
 #ifdef __cplusplus

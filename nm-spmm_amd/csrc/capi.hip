@@ -334,6 +334,23 @@ int nmspmm_preprocess_device(const int32_t* dDT_in, int n, int m, int W, int Q, 
         return NMSPMM_ERR_NULL_POINTER;
     if (n <= 0 || m <= 0 || n > m)
         return NMSPMM_ERR_BAD_PATTERN;
+    if (Q > 0 && N > 0 && N % Q == 0 && N / Q < 32) {
+        // vectors of 4, 8 or 16 columns: the kernels take the window as generated, so the whole
+        // preprocessing is the re-blocking
+        const int vec_len = N / Q;
+        if (!valid_vec_len(vec_len))
+            return NMSPMM_ERR_BAD_PATTERN;
+        const int st = check_reblock(dDT_in, dD_out, W, Q, Ns, vec_len);
+        if (st != NMSPMM_OK)
+            return st;
+        if (dDT_in == dD_out || W % n != 0)
+            return NMSPMM_ERR_BAD_SHAPE;
+        if (launch_reblock(dDT_in, dD_out, W, Q, Ns / vec_len, n, m, 0, (hipStream_t)stream) != hipSuccess)
+            return NMSPMM_ERR_HIP;
+        *window = m;
+        *kept = n;
+        return NMSPMM_OK;
+    }
     // the kernel geometry of the pattern's sparsity, reached by doubling the generated window
     int win = 0, kp = 0, high = 0;
     const int st0 = nmspmm_pattern_from_sparsity(1.0f - (float)n / (float)m, &win, &kp, &high);
@@ -472,7 +489,7 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     if (lda == 0 && M > 32 && M % 4 != 0) {
         // a padded copy of A is only worth making if it reaches the matrix-core kernel
         a.lda = (M + 3) / 4 * 4;
-        if (!mfma_supported(a) && !short_supported(a))
+        if (!mfma_supported(a) && !short_supported(a) && !gather_supported(a))
             a.lda = M;
     }
     if (lda_out)
@@ -501,6 +518,10 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     if (mfma_supported(a)) {
         e = launch_mfma(a);
         g_last_kernel = "mfma";
+    } else if (gather_supported(a)) {
+        // short vectors at densities up to one half: multiply the kept rows only
+        e = launch_gather(a);
+        g_last_kernel = "gather";
     } else if (short_supported(a)) {
         e = launch_short(a);
         g_last_kernel = "short";

@@ -370,6 +370,12 @@ size_t mfma_tail_workspace_bytes(const SpmmArgs& a);
 bool short_supported(const SpmmArgs& a);
 hipError_t launch_short(const SpmmArgs& a);
 
+// Gathering matrix-core path for the same vector lengths at densities up to one half
+// (spmm_gather.hip): multiplies kept rows only; K a multiple of 64 (32 for windows of 4 rows),
+// N a multiple of 64, any M.
+bool gather_supported(const SpmmArgs& a);
+hipError_t launch_gather(const SpmmArgs& a);
+
 // Decode-sized path (spmm_skinny.hip): M <= 32, the reference geometries, no workspace needed.
 bool skinny_supported(const SpmmArgs& a);
 hipError_t launch_skinny(const SpmmArgs& a);

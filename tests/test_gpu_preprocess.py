@@ -76,6 +76,23 @@ def test_full_size_index_buffers_bit_exact_vs_checker(oracle, N, K, n, m, vl, ti
         assert np.array_equal(ci.cpu().numpy(), want_ci)
 
 
+@pytest.mark.parametrize("vl,n,m,Ns", [(4, 2, 4, 128), (4, 1, 8, 32), (8, 2, 8, 64), (16, 3, 8, 128), (8, 4, 16, 128)])
+def test_one_kernel_preprocessing_of_short_vectors(oracle, vl, n, m, Ns):
+    """With vectors of 4, 8 or 16 columns the window stays as generated: the one-kernel entry point
+    re-blocks, reports (m, n) as the geometry and needs no column_info."""
+    N, K = 512, 256
+    d = datagen.init_data(4, N, K, n, m, vec_len=vl, seed=vl + n)
+    W, Q = d["W"], d["Q"]
+    src = torch.from_numpy(d["DT"].reshape(-1).copy()).cuda()
+    out = torch.full_like(src, -5)
+    assert nmspmm.preprocess_device(src, n, m, W, Q, N, Ns, out, None) == (m, n)
+    torch.cuda.synchronize()
+    want = d["DT"].reshape(-1).copy()
+    oracle.preprocess_low(want, W, Q, Ns, vl)
+    assert np.array_equal(out.cpu().numpy(), want)
+    assert np.array_equal(src.cpu().numpy(), d["DT"].reshape(-1))
+
+
 @pytest.mark.parametrize("n,m", [(2, 4), (3, 8), (2, 8), (1, 8), (16, 32), (12, 32), (8, 32), (4, 32), (32, 32), (1, 2), (4, 16)])
 @pytest.mark.parametrize("Ns", [128, 64, 32])
 def test_one_kernel_preprocessing_equals_the_separate_calls(oracle, n, m, Ns):

@@ -193,10 +193,11 @@ def test_decode_shapes_at_full_size(oracle, M, n, m, K, N):
     check(oracle, d, got)
 
 
-@pytest.mark.parametrize("vl,n,m", [(4, 2, 4), (8, 1, 8), (16, 3, 8)])
+@pytest.mark.parametrize("vl,n,m", [(4, 3, 4), (8, 5, 8), (16, 7, 8)])
 def test_short_vectors_on_the_generic_kernel(oracle, vl, n, m):
-    """Per-vector length below 32 on a shape the matrix-core kernels do not take (64 columns):
-    indices are used as generated (no widening), any window."""
+    """Per-vector length below 32 on shapes and patterns the matrix-core kernels do not take (64
+    columns are too few for the expanding kernel, densities above one half are not for the gathering
+    one): indices are used as generated (no widening), any window."""
     M, N, K = 64, 64, 256
     d = datagen.init_data(M, N, K, n, m, vec_len=vl, seed=vl)
     W, Q = d["W"], d["Q"]
@@ -213,7 +214,8 @@ def test_short_vectors_on_the_generic_kernel(oracle, vl, n, m):
                                        (4, 4, 8, 128), (8, 2, 16, 32), (16, 4, 16, 64), (4, 8, 16, 128)])
 @pytest.mark.parametrize("M,split_k", [(64, 1), (256, 1), (300, 2), (132, 3)])
 def test_short_vectors_on_the_matrix_cores(oracle, vl, n, m, Ns, M, split_k):
-    """Vector lengths 4, 8 and 16 with windows of 4, 8 and 16 rows: the expanding MFMA kernel."""
+    """Vector lengths 4, 8 and 16 with windows of 4, 8 and 16 rows: the gathering MFMA kernel up to a
+    density of one half, the expanding one above."""
     N, K = 256, 512
     d = datagen.init_data(M, N, K, n, m, vec_len=vl, seed=vl + n + M)
     W, Q = d["W"], d["Q"]
@@ -224,7 +226,49 @@ def test_short_vectors_on_the_matrix_cores(oracle, vl, n, m, Ns, M, split_k):
     nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), None, C, M, N, K, W, m, n, vl, Ns, split_k,
                 ws if split_k > 1 else None)
     torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == ("gather" if 2 * n <= m else "short")
+    check(oracle, d, C.cpu().numpy())
+
+
+@pytest.mark.parametrize("vl,n,m,Ns", [(4, 2, 4, 128), (8, 1, 8, 64), (16, 4, 16, 32), (4, 3, 4, 128)])
+@pytest.mark.parametrize("M,split_k", [(64, 1), (300, 2)])
+def test_short_vectors_on_the_expanding_kernel(oracle, vl, n, m, Ns, M, split_k):
+    """A reduction that is whole 16-row chunks but not whole 64-row (32-row) chunks stays on the
+    expanding kernel at any density."""
+    N, K = 256, 528
+    d = datagen.init_data(M, N, K, n, m, vec_len=vl, seed=vl + n + M)
+    W, Q = d["W"], d["Q"]
+    D = d["DT"].reshape(-1).copy()
+    oracle.preprocess_low(D, W, Q, Ns, vl)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    ws = torch.empty(max(nmspmm.workspace_bytes(M, N, split_k) // 4, 1), dtype=torch.float32, device="cuda")
+    nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), None, C, M, N, K, W, m, n, vl, Ns, split_k,
+                ws if split_k > 1 else None)
+    torch.cuda.synchronize()
     assert nmspmm.last_kernel() == "short"
+    check(oracle, d, C.cpu().numpy())
+
+
+@pytest.mark.parametrize("vl", [4, 8, 16])
+@pytest.mark.parametrize("n,m", [(1, 4), (2, 4), (1, 8), (2, 8), (3, 8), (4, 8), (2, 16), (4, 16), (8, 16)])
+@pytest.mark.parametrize("M,N,K,split_k", [(4, 64, 64, 1), (36, 192, 256, 1), (64, 256, 512, 4), (200, 320, 384, 3), (260, 1088, 128, 2)])
+def test_gathering_kernel_every_pattern_and_vector_length(oracle, vl, n, m, M, N, K, split_k):
+    """The gathering kernel on every pattern it is built for: row counts that are not whole 64-row
+    tiles (from four rows; like every matrix-core kernel it wants a row count that is a multiple of
+    four), column counts that are not whole 256-column workgroups, reductions of one chunk, splits
+    that leave slices unequal."""
+    Ns = 64 if N % 128 else 128
+    d = datagen.init_data(M, N, K, n, m, vec_len=vl, seed=vl + 3 * n + M)
+    W, Q = d["W"], d["Q"]
+    D = d["DT"].reshape(-1).copy()
+    oracle.preprocess_low(D, W, Q, Ns, vl)
+    chunk = 32 if m == 4 else 64
+    split_k = min(split_k, K // chunk)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    ws = torch.empty(max(nmspmm.workspace_bytes(M, N, split_k) // 4, 1), dtype=torch.float32, device="cuda")
+    nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), None, C, M, N, K, W, m, n, vl, Ns, split_k, ws if split_k > 1 else None)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == "gather"
     check(oracle, d, C.cpu().numpy())
 
 
@@ -429,12 +473,13 @@ def test_full_size_4096_cubed_remaining_patterns(oracle, n, m):
     check_every_tile_once(oracle, 4096, 4096, 4096, n, m, 128)
 
 
-def test_full_size_4096_cubed_2of4_with_vectors_of_four_columns(oracle):
-    """2:4 with index vectors of 4 columns at M = Ncols = K = 4096: 2048 x 1024 indices (8 MiB), the
-    expanding matrix-core kernel.  Column sums in fp64 over all of C; sampled rows against the
-    checker."""
+@pytest.mark.parametrize("n,m", [(2, 4), (2, 8), (1, 8)])
+def test_full_size_4096_cubed_with_vectors_of_four_columns(oracle, n, m):
+    """2:4, 2:8 and 1:8 with index vectors of 4 columns at M = Ncols = K = 4096 (2:4: 2048 x 1024
+    indices, 8 MiB), the gathering matrix-core kernel.  Column sums in fp64 over all of C; sampled
+    rows against the checker."""
     M = N = K = 4096
-    vl, n, m = 4, 2, 4
+    vl = 4
     d = datagen.init_data(M, N, K, n, m, vec_len=vl, seed=5004)
     W, Q = d["W"], d["Q"]
     DT = dev(d["DT"].reshape(-1))
@@ -446,7 +491,7 @@ def test_full_size_4096_cubed_2of4_with_vectors_of_four_columns(oracle):
     C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
     nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), D, None, C, M, N, K, W, m, n, vl, 128)
     torch.cuda.synchronize()
-    assert nmspmm.last_kernel() == "short" and bool(torch.isfinite(C).all())
+    assert nmspmm.last_kernel() == "gather" and bool(torch.isfinite(C).all())
     dense = torch.zeros((K, N), dtype=torch.float64, device="cuda")
     rows = (torch.arange(W, device="cuda") // n * m)[:, None] + dev(d["DT"]).long()
     dense[rows.repeat_interleave(vl, dim=1), torch.arange(N, device="cuda")[None, :].expand(W, -1)] = dev(d["BT"]).double()
@@ -566,7 +611,7 @@ def test_row_counts_either_side_of_the_tile_kernels_limit(oracle, M, family):
     assert not torch.isnan(C).any().item()
 
 
-@pytest.mark.parametrize("M,N,K,vl,n,m", [(2048, 11008, 256, 4, 2, 4), (4096, 5120, 512, 8, 1, 8), (1000, 24576, 256, 16, 3, 8)])
+@pytest.mark.parametrize("M,N,K,vl,n,m", [(2048, 11008, 256, 4, 3, 4), (4096, 5120, 528, 8, 1, 8), (1000, 24576, 272, 16, 3, 8)])
 def test_short_vector_kernel_with_leftover_tiles(oracle, M, N, K, vl, n, m):
     """The short-vector kernel on more tiles than the GPU holds at once with a ragged last round:
     the leftovers run as a second launch, whole or as two 128-row pieces each.  Column sums in fp64
