@@ -316,13 +316,13 @@ def run_decode(torch, pkg, rows_list=(1, 8, 16, 32), shapes=((8192, 8192), (4096
     return out
 
 
-def run_fine(torch, pkg):
+def run_fine(torch, pkg, cases):
     """Config 5: the n:32 patterns and 2:4 with 4-column vectors at 4096 cubed, with the device
     preprocessing time of each (one launch for 32-column vectors, the re-blocking launch for
     shorter ones); beyond the baseline's list, 2:8 and 1:8 with 4-column vectors and 1:8 with
     8-column ones."""
     out = []
-    for (n, m, vl) in ((4, 32, 32), (8, 32, 32), (16, 32, 32), (2, 4, 4), (2, 8, 4), (1, 8, 4), (1, 8, 8)):
+    for (n, m, vl) in cases:
         op = GpuOperands(torch, pkg, M, N, K, n, m, vec_len=vl, normal=False)
         ms, _ = time_launches(torch, lambda: pkg.spmm(op.A, op.B, op.D, op.cinfo, op.C, M, N, K, op.W, op.window,
                                                       op.kept, vl, NS, 1, None), 20, 3, 0.3)
@@ -531,6 +531,8 @@ def main():
     ap.add_argument("--decode-patterns", default="1:8,2:8", help="patterns of the decode part")
     ap.add_argument("--decode-modes", default=",".join(m[0] for m in DECODE_MODES),
                     help="which of hot, cold, cold_stream_hint, hot_reference_layout, cold_reference_layout to time")
+    ap.add_argument("--fine-cases", default="4:32x32,8:32x32,16:32x32,2:4x4,2:8x4,1:8x4,1:8x8",
+                    help="cases of the fine part, n:m x vector length")
     ap.add_argument("--ksweep-ks", default="64,1024,4096", help="reduction lengths of the ksweep part")
     ap.add_argument("--ksweep-patterns", default="2:4,1:8,4:32", help="patterns of the ksweep part")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -616,7 +618,8 @@ def main():
             tuple(tuple(int(v) for v in x.split(":")) for x in args.decode_patterns.split(",")),
             tuple(args.decode_modes.split(",")))
     if "fine" in parts:
-        configs["fine"] = run_fine(torch, pkg)
+        configs["fine"] = run_fine(torch, pkg, tuple(
+            (int(x.split(":")[0]), int(x.split(":")[1].split("x")[0]), int(x.split("x")[1])) for x in args.fine_cases.split(",")))
     if "ksweep" in parts:
         configs["launch_constant"] = run_ksweep(
             torch, pkg, tuple(int(x) for x in args.ksweep_ks.split(",")),
