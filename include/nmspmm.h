@@ -279,7 +279,8 @@ int nmspmm_tile_wave_rows(int M, int N, int W, int kept, int Ns, int split_k);
 int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int32_t* column_info,
                      float* C, int M, int N, int K, int W, float sparsity, void* stream);
 
-/* Frees the cached split-K workspaces of every device. */
+/* Frees what the library keeps per device: the cached split-K workspaces and the staging buffer
+ * of the host-pointer preprocessing forms. */
 int nmspmm_release(void);
 
 /* Name of the kernel family the last successful nmspmm_spmm call on this thread dispatched to

@@ -95,15 +95,56 @@ int cached_workspace(size_t bytes, void** out)
     return NMSPMM_OK;
 }
 
-// RAII device buffer for the host-pointer preprocessing forms.
-struct DeviceBuf {
-    void* p = nullptr;
-    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes); }
-    ~DeviceBuf()
+// Device staging for the host-pointer preprocessing forms: one buffer per device, grown on demand
+// and kept until nmspmm_release(), instead of an allocation per call.  Those calls are synchronous
+// (they end with a copy back to the host), so a lease simply holds the lock for the duration of
+// the call; an outgrown buffer has no work pending and is freed at once.
+struct Staging {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
+Staging g_staging[kMaxDevices];
+std::mutex g_staging_mutex;
+
+class StagingLease {
+public:
+    // `parts` regions of the given sizes, each on a 256-byte boundary
+    StagingLease(const size_t* sizes, int parts) : lock_(g_staging_mutex)
     {
-        if (p)
-            (void)hipFree(p);
+        int dev = 0;
+        if (parts > kMaxParts || hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+            return;
+        size_t total = 0;
+        size_t offset[kMaxParts];
+        for (int i = 0; i < parts; ++i) {
+            offset[i] = total;
+            total += (sizes[i] + 255) / 256 * 256;
+        }
+        Staging& st = g_staging[dev];
+        if (st.bytes < total) {
+            if (st.ptr)
+                (void)hipFree(st.ptr);
+            st.ptr = nullptr;
+            st.bytes = 0;
+            if (hipMalloc(&st.ptr, total) != hipSuccess) {
+                (void)hipGetLastError();
+                st.ptr = nullptr;
+                return;
+            }
+            st.bytes = total;
+        }
+        for (int i = 0; i < parts; ++i)
+            part_[i] = (char*)st.ptr + offset[i];
+        ok_ = true;
     }
+    bool ok() const { return ok_; }
+    void* part(int i) const { return part_[i]; }
+
+private:
+    static constexpr int kMaxParts = 3;
+    std::lock_guard<std::mutex> lock_;
+    void* part_[kMaxParts] = {nullptr, nullptr, nullptr};
+    bool ok_ = false;
 };
 
 } // namespace
@@ -212,15 +253,15 @@ int nmspmm_trans_index_host(int32_t* DT, int W, int N, int Q, int* pruning_N, in
     if (st != NMSPMM_OK)
         return st;
     const size_t bytes = sizeof(int32_t) * (size_t)W * Q;
-    DeviceBuf d;
-    if (d.alloc(bytes) != hipSuccess)
+    const StagingLease d(&bytes, 1);
+    if (!d.ok())
         return NMSPMM_ERR_HIP;
-    if (hipMemcpy(d.p, DT, bytes, hipMemcpyHostToDevice) != hipSuccess)
+    if (hipMemcpy(d.part(0), DT, bytes, hipMemcpyHostToDevice) != hipSuccess)
         return NMSPMM_ERR_HIP;
-    const int rc = nmspmm_trans_index_device((int32_t*)d.p, W, N, Q, pruning_N, pruning_M, nullptr);
+    const int rc = nmspmm_trans_index_device((int32_t*)d.part(0), W, N, Q, pruning_N, pruning_M, nullptr);
     if (rc != NMSPMM_OK)
         return rc;
-    if (hipMemcpy(DT, d.p, bytes, hipMemcpyDeviceToHost) != hipSuccess)
+    if (hipMemcpy(DT, d.part(0), bytes, hipMemcpyDeviceToHost) != hipSuccess)
         return NMSPMM_ERR_HIP;
     return NMSPMM_OK;
 }
@@ -255,15 +296,17 @@ int nmspmm_preprocess_low_host(int32_t* DT, int W, int Q, int Ns, int vec_len)
     if (st != NMSPMM_OK)
         return st;
     const size_t bytes = sizeof(int32_t) * (size_t)W * Q;
-    DeviceBuf in, out;
-    if (in.alloc(bytes) != hipSuccess || out.alloc(bytes) != hipSuccess)
+    const size_t sizes[2] = {bytes, bytes};
+    const StagingLease d(sizes, 2);
+    if (!d.ok())
         return NMSPMM_ERR_HIP;
-    if (hipMemcpy(in.p, DT, bytes, hipMemcpyHostToDevice) != hipSuccess)
+    if (hipMemcpy(d.part(0), DT, bytes, hipMemcpyHostToDevice) != hipSuccess)
         return NMSPMM_ERR_HIP;
-    const int rc = nmspmm_preprocess_low_device((const int32_t*)in.p, (int32_t*)out.p, W, Q, Ns, vec_len, nullptr);
+    const int rc =
+        nmspmm_preprocess_low_device((const int32_t*)d.part(0), (int32_t*)d.part(1), W, Q, Ns, vec_len, nullptr);
     if (rc != NMSPMM_OK)
         return rc;
-    if (hipMemcpy(DT, out.p, bytes, hipMemcpyDeviceToHost) != hipSuccess)
+    if (hipMemcpy(DT, d.part(1), bytes, hipMemcpyDeviceToHost) != hipSuccess)
         return NMSPMM_ERR_HIP;
     return NMSPMM_OK;
 }
@@ -312,17 +355,18 @@ int nmspmm_preprocess_high_host(int32_t* column_info, int pruning_M, int pruning
         return st;
     const size_t bytes = sizeof(int32_t) * (size_t)W * Q;
     const size_t ci_bytes = sizeof(int32_t) * nmspmm_column_info_ints(W, pruning_N, pruning_M, N, Ns);
-    DeviceBuf in, out, ci;
-    if (in.alloc(bytes) != hipSuccess || out.alloc(bytes) != hipSuccess || ci.alloc(ci_bytes) != hipSuccess)
+    const size_t sizes[3] = {bytes, bytes, ci_bytes};
+    const StagingLease d(sizes, 3);
+    if (!d.ok())
         return NMSPMM_ERR_HIP;
-    if (hipMemcpy(in.p, DT, bytes, hipMemcpyHostToDevice) != hipSuccess)
+    if (hipMemcpy(d.part(0), DT, bytes, hipMemcpyHostToDevice) != hipSuccess)
         return NMSPMM_ERR_HIP;
-    const int rc = nmspmm_preprocess_high_device((int32_t*)ci.p, pruning_M, pruning_N, (const int32_t*)in.p,
-                                                 (int32_t*)out.p, W, Q, N, Ns, vec_len, nullptr);
+    const int rc = nmspmm_preprocess_high_device((int32_t*)d.part(2), pruning_M, pruning_N, (const int32_t*)d.part(0),
+                                                 (int32_t*)d.part(1), W, Q, N, Ns, vec_len, nullptr);
     if (rc != NMSPMM_OK)
         return rc;
-    if (hipMemcpy(DT, out.p, bytes, hipMemcpyDeviceToHost) != hipSuccess ||
-        hipMemcpy(column_info, ci.p, ci_bytes, hipMemcpyDeviceToHost) != hipSuccess)
+    if (hipMemcpy(DT, d.part(1), bytes, hipMemcpyDeviceToHost) != hipSuccess ||
+        hipMemcpy(column_info, d.part(2), ci_bytes, hipMemcpyDeviceToHost) != hipSuccess)
         return NMSPMM_ERR_HIP;
     return NMSPMM_OK;
 }
@@ -815,6 +859,18 @@ int nmspmm_release(void)
         ws.retired.clear();
         ws.ptr = nullptr;
         ws.bytes = 0;
+    }
+    {
+        std::lock_guard<std::mutex> staging_lock(g_staging_mutex);
+        for (int d = 0; d < kMaxDevices; ++d) {
+            Staging& st = g_staging[d];
+            if (!st.ptr)
+                continue;
+            if (hipSetDevice(d) != hipSuccess || hipFree(st.ptr) != hipSuccess)
+                rc = NMSPMM_ERR_HIP;
+            st.ptr = nullptr;
+            st.bytes = 0;
+        }
     }
     if (have_dev)
         (void)hipSetDevice(prev);
