@@ -17,7 +17,7 @@
 // MFMAs, and the value of B it needs (one 32-bit load per kept row) is reused by all sixteen MFMAs of
 // the step.  Index and B value are loaded eight steps ahead, the next chunk of A is fetched into
 // registers while the current one is multiplied.  Measured at 4096 cubed with vectors of 4 columns:
-// 1:8 70, 2:8 82, 2:4 95 useful TFLOP/s, where the expanding kernel reaches 18, 36 and 71.
+// 1:8 85, 2:8 93, 2:4 93 useful TFLOP/s, where the expanding kernel reaches 18, 36 and 71.
 #include "internal.h"
 
 namespace nmspmm {
@@ -74,19 +74,22 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
     const int M = p.M, N = p.N, W = p.W, lda = p.lda;
     // a wave beyond the last column repeats the last 64 columns (it has to reach the barriers)
     const int col0 = min(tile_n * kGatherCols + wave * 64, N - 64);
+    // this slice's chunks: everything below counts chunks and steps from the slice's first one
     int c_begin, c_count;
     split_windows(p.nchunk, p.split_k, blockIdx.y, &c_begin, &c_count);
-    const int s_begin = c_begin * STEPS, s_end = (c_begin + c_count) * STEPS;
+    const int s_begin = c_begin * STEPS, s_count = c_count * STEPS;
 
     const size_t K = (size_t)p.nchunk * KC;
     const __amdgpu_buffer_rsrc_t ra = gather_rsrc(p.A, (uint32_t)(K * lda * sizeof(float)));
-    const __amdgpu_buffer_rsrc_t rb = gather_rsrc(p.B + col0, (uint32_t)(((size_t)(W - 1) * N + 64) * sizeof(float)));
+    const __amdgpu_buffer_rsrc_t rb = gather_rsrc(p.B + (size_t)s_begin * N + col0,
+                                                  (uint32_t)(((size_t)(W - 1 - s_begin) * N + 64) * sizeof(float)));
     const __amdgpu_buffer_rsrc_t rd = gather_rsrc(p.D, (uint32_t)((size_t)W * (N >> (2 + p.lshift)) * sizeof(int32_t)));
     const uint32_t b_row = (uint32_t)N * 4u, d_row = (uint32_t)p.Qs * 4u;
     // D is blocked [N / Ns][W][Qs]: this block's vector is (col0 + 4b) / L
     const int Ns = p.Qs << (2 + p.lshift);
     const int col = col0 + 4 * b;
-    const uint32_t d_lane = (uint32_t)(((size_t)(col / Ns) * W * p.Qs + ((col % Ns) >> (2 + p.lshift))) * sizeof(int32_t));
+    const uint32_t d_lane = (uint32_t)(((size_t)(col / Ns) * W * p.Qs + (size_t)s_begin * p.Qs + ((col % Ns) >> (2 + p.lshift))) *
+                                       sizeof(int32_t));
     const uint32_t b_lane = (uint32_t)lane * 4u;
 
     // chunk copy: segment tid + 256 j is 16 bytes (4 rows) of dense row seg / 16 of the chunk
@@ -94,7 +97,7 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
 #pragma unroll
     for (int j = 0; j < SPT; ++j) {
         const int seg = tid + 256 * j, kk = seg / (4 * RB), part = seg % (4 * RB);
-        cp_src[j] = (uint32_t)(((size_t)kk * lda + row0 + part * 4) * sizeof(float));
+        cp_src[j] = (uint32_t)((((size_t)c_begin * KC + kk) * lda + row0 + part * 4) * sizeof(float));
         cp_dst[j] = (uint32_t)(kk * STRIDE + part * 16);
     }
     const uint32_t chunk_bytes = (uint32_t)((size_t)KC * lda * sizeof(float));
@@ -104,7 +107,7 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
 #pragma unroll
         for (int j = 0; j < SPT; ++j) {
             const auto x = __builtin_amdgcn_raw_buffer_load_b128(
-                ra, c < c_begin + c_count ? cp_src[j] + (uint32_t)c * chunk_bytes : kGatherNoLoad, 0, 0);
+                ra, c < c_count ? cp_src[j] + (uint32_t)c * chunk_bytes : kGatherNoLoad, 0, 0);
             stage[j] = gfloatx4{__int_as_float(x[0]), __int_as_float(x[1]), __int_as_float(x[2]), __int_as_float(x[3])};
         }
     };
@@ -119,13 +122,13 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
     for (int r = 0; r < 4 * RB; ++r)
         acc[r] = {0.0f, 0.0f, 0.0f, 0.0f};
 
-    // step s = kept row s of the reduction.  The uniform part of both addresses is a scalar offset
+    // step s = kept row s of the slice.  The uniform part of both addresses is a scalar offset
     // (not covered by the descriptor's range check: steps outside the slice take the vector offset
     // that is out of range instead).
     int idx[PF];
     float bv[PF];
     auto load_meta = [&](int s, int slot) {
-        const bool ok = s < s_end;
+        const bool ok = s < s_count;
         idx[slot] = __builtin_amdgcn_raw_buffer_load_b32(rd, ok ? d_lane : kGatherNoLoad, ok ? (uint32_t)s * d_row : 0u, 0);
         bv[slot] = __int_as_float(
             __builtin_amdgcn_raw_buffer_load_b32(rb, ok ? b_lane : kGatherNoLoad, ok ? (uint32_t)s * b_row : 0u, 0));
@@ -146,11 +149,11 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
 
 #pragma unroll
     for (int t = 0; t < PF; ++t)
-        load_meta(s_begin + t, t);
-    fetch_chunk(c_begin);
+        load_meta(t, t);
+    fetch_chunk(0);
     store_chunk();
     __syncthreads();
-    for (int c = c_begin; c < c_begin + c_count; ++c) {
+    for (int c = 0; c < c_count; ++c) {
         fetch_chunk(c + 1);
         const int s_base = c * STEPS;
         read_a(0, idx[0], a[0]);
