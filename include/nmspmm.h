@@ -212,8 +212,8 @@ int nmspmm_spmm_noalloc(const float* A, const float* B, const int32_t* D, const 
  * row-major A into the layout nmspmm_spmm takes; one such copy serves every weight matrix that
  * multiplies the same activations).  nmspmm_spmm_rowmajor does both steps: the workspace holds the
  * column-major copy followed by the split-K slices, nmspmm_workspace_bytes_rowmajor() bytes, never
- * optional.  The copy's row pitch is M rounded up to 4 floats, so any M above 32 runs on the
- * matrix-core kernel (nmspmm_spmm itself needs M % 4 == 0 for that).  Up to 8 rows (decoding) the
+ * optional.  The copy's row pitch is M rounded up to 4 floats (the matrix-core kernels take any
+ * pitch; this one keeps their 128-bit loads on 16-byte boundaries).  Up to 8 rows (decoding) the
  * kernel reads the row-major A in place and nothing is copied; the workspace is still required,
  * so that a caller sizes it once for every M.  Other arguments and requirements as nmspmm_spmm. */
 int nmspmm_transpose_device(const float* src, int rows, int cols, float* dst, void* stream);

@@ -722,7 +722,10 @@ bool mfma_supported(const SpmmArgs& a)
         return false;
     if (a.vec_len != 32 || (a.Ns != 32 && a.Ns != 64 && a.Ns != 128))
         return false;
-    if (a.lda % 4 != 0 || a.lda < a.M || a.M < 32)
+    // any pitch: 128-bit buffer loads only need their address on a 4-byte boundary, and their range
+    // check is per 32-bit word (a pitch that is a multiple of four floats keeps them on 16-byte
+    // boundaries, which is faster)
+    if (a.lda < a.M || a.M < 32)
         return false;
     // 32-bit buffer offsets: one window of A and one window of B must stay below 2 GiB; the row
     // offset of A is formed with a 24-bit multiply

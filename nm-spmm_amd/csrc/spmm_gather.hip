@@ -198,8 +198,7 @@ bool gather_supported(const SpmmArgs& a)
     if (a.vec_len != 4 && a.vec_len != 8 && a.vec_len != 16)
         return false;
     const int chunk = a.window == 4 ? 32 : 64;
-    if (a.N % 64 != 0 || a.Ns % a.vec_len != 0 || a.N % a.Ns != 0 || a.K % chunk != 0 || a.M < 1 || a.lda % 4 != 0 ||
-        a.lda < a.M)
+    if (a.N % 64 != 0 || a.Ns % a.vec_len != 0 || a.N % a.Ns != 0 || a.K % chunk != 0 || a.M < 1 || a.lda < a.M)
         return false;
     if (a.split_k < 1 || a.split_k > a.K / chunk)
         return false;

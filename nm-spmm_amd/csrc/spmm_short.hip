@@ -247,7 +247,7 @@ bool short_supported(const SpmmArgs& a)
         return false;
     if (a.cinfo != nullptr || a.vec_len >= 32 || (a.vec_len != 4 && a.vec_len != 8 && a.vec_len != 16))
         return false;
-    if (a.N % 128 != 0 || a.Ns % 32 != 0 || a.K % kChunk != 0 || a.M <= 32 || a.lda % 4 != 0 || a.lda < a.M)
+    if (a.N % 128 != 0 || a.Ns % 32 != 0 || a.K % kChunk != 0 || a.M <= 32 || a.lda < a.M)
         return false;
     if (a.split_k > a.K / kChunk)
         return false;

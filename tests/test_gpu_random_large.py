@@ -53,7 +53,7 @@ def test_random_large_shape(case):
         cinfo = torch.empty(nmspmm.column_info_ints(W, kept, window, N, Ns), dtype=torch.int32, device="cuda")
     assert nmspmm.preprocess_device(DT, n, m, W, Q, N, Ns, D, cinfo) == (window, kept)
     C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
-    if row_major or M % 4 != 0:  # (a column-major A with such a row count would take the generic kernel)
+    if row_major:
         ws = torch.empty(nmspmm.workspace_bytes_rowmajor(M, N, K, split_k) // 4, dtype=torch.float32, device="cuda")
         nmspmm.spmm_rowmajor(X, BT, D, cinfo, C, M, N, K, W, window, kept, ws, 32, Ns, split_k)
     else:

@@ -62,9 +62,11 @@ def test_config1_512_cubed_2of4(oracle):
     assert scaled_max_error(got, want) <= REL_TOL
 
 
-@pytest.mark.parametrize("M", [36, 64, 100, 132, 192, 328, 448])
+@pytest.mark.parametrize("M", [33, 36, 37, 64, 100, 101, 131, 132, 192, 257, 328, 333, 448, 1001])
 @pytest.mark.parametrize("n,m,Ns", [(2, 4, 128), (1, 8, 128), (2, 8, 64), (3, 8, 32)])
 def test_ragged_row_counts(oracle, M, n, m, Ns):
+    """Row counts that are not whole tiles, odd ones included: with a pitch of A that is not a multiple
+    of four floats the 128-bit loads of the matrix-core kernels sit on 4-byte boundaries only."""
     d = datagen.init_data(M, 256, 256, n, m, seed=M + n)
     got, fam = run_gpu(oracle, d, Ns)
     assert fam == "mfma" if M > 128 else fam in ("mfma", "skinny")   # up to 128 rows the two kernels compete
@@ -212,7 +214,7 @@ def test_short_vectors_on_the_generic_kernel(oracle, vl, n, m):
 
 @pytest.mark.parametrize("vl,n,m,Ns", [(4, 2, 4, 128), (4, 1, 4, 32), (4, 3, 4, 64), (8, 1, 8, 128), (8, 2, 8, 64), (16, 3, 8, 128),
                                        (4, 4, 8, 128), (8, 2, 16, 32), (16, 4, 16, 64), (4, 8, 16, 128)])
-@pytest.mark.parametrize("M,split_k", [(64, 1), (256, 1), (300, 2), (132, 3)])
+@pytest.mark.parametrize("M,split_k", [(64, 1), (256, 1), (301, 2), (132, 3)])
 def test_short_vectors_on_the_matrix_cores(oracle, vl, n, m, Ns, M, split_k):
     """Vector lengths 4, 8 and 16 with windows of 4, 8 and 16 rows: the gathering MFMA kernel up to a
     density of one half, the expanding one above."""
@@ -231,7 +233,7 @@ def test_short_vectors_on_the_matrix_cores(oracle, vl, n, m, Ns, M, split_k):
 
 
 @pytest.mark.parametrize("vl,n,m,Ns", [(4, 2, 4, 128), (8, 1, 8, 64), (16, 4, 16, 32), (4, 3, 4, 128)])
-@pytest.mark.parametrize("M,split_k", [(64, 1), (300, 2)])
+@pytest.mark.parametrize("M,split_k", [(64, 1), (301, 2)])
 def test_short_vectors_on_the_expanding_kernel(oracle, vl, n, m, Ns, M, split_k):
     """A reduction that is whole 16-row chunks but not whole 64-row (32-row) chunks stays on the
     expanding kernel at any density."""
@@ -251,12 +253,11 @@ def test_short_vectors_on_the_expanding_kernel(oracle, vl, n, m, Ns, M, split_k)
 
 @pytest.mark.parametrize("vl", [4, 8, 16])
 @pytest.mark.parametrize("n,m", [(1, 4), (2, 4), (1, 8), (2, 8), (3, 8), (4, 8), (2, 16), (4, 16), (8, 16)])
-@pytest.mark.parametrize("M,N,K,split_k", [(4, 64, 64, 1), (36, 192, 256, 1), (64, 256, 512, 4), (200, 320, 384, 3), (260, 1088, 128, 2)])
+@pytest.mark.parametrize("M,N,K,split_k", [(1, 64, 64, 1), (4, 64, 64, 1), (37, 192, 256, 1), (64, 256, 512, 4), (201, 320, 384, 3), (260, 1088, 128, 2)])
 def test_gathering_kernel_every_pattern_and_vector_length(oracle, vl, n, m, M, N, K, split_k):
     """The gathering kernel on every pattern it is built for: row counts that are not whole 64-row
-    tiles (from four rows; like every matrix-core kernel it wants a row count that is a multiple of
-    four), column counts that are not whole 256-column workgroups, reductions of one chunk, splits
-    that leave slices unequal."""
+    tiles (from a single row, odd ones included), column counts that are not whole 256-column
+    workgroups, reductions of one chunk, splits that leave slices unequal."""
     Ns = 64 if N % 128 else 128
     d = datagen.init_data(M, N, K, n, m, vec_len=vl, seed=vl + 3 * n + M)
     W, Q = d["W"], d["Q"]
