@@ -64,7 +64,9 @@ int nmspmm_pattern_from_sparsity(float sparsity, int* window, int* kept, int* is
  * pair of adjacent windows of the row-major int32 DT[W][Q] by adding *pruning_M to the indices
  * of every odd window, then doubles *pruning_N and *pruning_M.  N is accepted for signature
  * parity and only checked against Q * vec_len.  Host-pointer form: DT is host memory, updated
- * in place (staged through the device, the work is done by the HIP kernel). */
+ * in place (staged through the device, the work is done by the HIP kernel).  The three
+ * host-pointer forms are synchronous and share one staging buffer per device, grown on demand and
+ * kept until nmspmm_release(): concurrent calls from several threads are safe and take turns. */
 int nmspmm_trans_index_host(int32_t* DT, int W, int N, int Q, int* pruning_N, int* pruning_M);
 /* Device-pointer form of the same operation, in place on device memory, asynchronous. */
 int nmspmm_trans_index_device(int32_t* dDT, int W, int N, int Q, int* pruning_N, int* pruning_M,
