@@ -22,9 +22,10 @@
 // instruction, each byte of B read once) and A[jl][row]; even and odd columns accumulate in two
 // MFMA tiles.  17 to 32 rows take a second pair of tiles for the other 16 rows with the same B
 // operands.  The waves add their tiles up through LDS in wave order (deterministic, one launch,
-// no workspace).  Measured on the MI355X: more than one group per wave in flight does not help (the
-// 16 waves of a CU keep 32 KB of B in flight, which covers the latency at the rate the fabric
-// delivers), so the loop is: load a group, multiply it.
+// no workspace).  Measured on the MI355X: more than one group per wave in flight does not help.
+// The counters show a CU with about 64 requests outstanding whatever the kernel does, which looks
+// like what its vector L1 keeps in flight: the 16 waves' one group each (256 lines of B plus their
+// rows of A) already fill it, so the loop is: load a group, multiply it.
 //
 // Every workgroup asks for the same rows of A in the same order, and the workgroups of an XCD share
 // its L2: in step, they all hit the same few cache lines (and L2 channels) at the same moment.  For
