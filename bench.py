@@ -45,7 +45,7 @@ M = N = K = 4096
 PATTERNS = [(2, 4), (3, 8), (2, 8), (1, 8)]  # first one is the headline
 NS = 128
 GEOMETRY = {(1, 1): (32, 32), (1, 2): (32, 16), (3, 8): (32, 12), (1, 4): (64, 16), (1, 8): (64, 8)}
-PARTS = ("sweep", "llm", "decode", "fine", "ksweep", "compress", "rowmajor", "preprocess", "dispatch", "cpu")
+PARTS = ("sweep", "llm", "decode", "decode_llm", "fine", "ksweep", "compress", "rowmajor", "preprocess", "dispatch", "cpu")
 
 
 def geometry(n, m):
@@ -271,11 +271,17 @@ def run_llm(torch, pkg):
 
 
 DECODE_MODES = (("hot", 0, True, False), ("cold", 0, True, True), ("cold_stream_hint", 2, True, True),
-                ("hot_reference_layout", 0, False, False), ("cold_reference_layout", 0, False, True))
+                ("hot_reference_layout", 0, False, False), ("cold_reference_layout", 0, False, True),
+                ("hot_split", 4, True, False), ("cold_split", 4, True, True))
+DECODE_DEFAULT_MODES = tuple(m[0] for m in DECODE_MODES[:5])
+# the decode sizes of the LLM-layer shapes (config 3's K x Ncols): fewer column vectors than compute
+# units, where NMSPMM_DECODE_SPLIT lets the kernel cut the reductions across workgroups
+DECODE_LLM_SHAPES = ((4096, 4096), (11008, 4096), (4096, 11008))
+DECODE_LLM_MODES = ("hot", "cold", "hot_split", "cold_split")
 
 
 def run_decode(torch, pkg, rows_list=(1, 8, 16, 32), shapes=((8192, 8192), (4096, 14336)), patterns=((1, 8), (2, 8)),
-               modes=tuple(m[0] for m in DECODE_MODES)):
+               modes=DECODE_DEFAULT_MODES):
     """Config 4.  Per case: the decode kernel on the row list and the kernel on the reference-layout
     indices, with one B re-read by every launch (it then sits in the 256 MB Infinity Cache: "hot")
     and with launches that walk through copies of B adding up to more than 600 MB ("cold": every
@@ -529,8 +535,8 @@ def main():
     ap.add_argument("--decode-rows", default="1,8,16,32", help="row counts of the decode part")
     ap.add_argument("--decode-shapes", default="8192x8192,4096x14336", help="K x Ncols of the decode part")
     ap.add_argument("--decode-patterns", default="1:8,2:8", help="patterns of the decode part")
-    ap.add_argument("--decode-modes", default=",".join(m[0] for m in DECODE_MODES),
-                    help="which of hot, cold, cold_stream_hint, hot_reference_layout, cold_reference_layout to time")
+    ap.add_argument("--decode-modes", default=",".join(DECODE_DEFAULT_MODES),
+                    help="which of " + ", ".join(m[0] for m in DECODE_MODES) + " to time")
     ap.add_argument("--fine-cases", default="4:32x32,8:32x32,16:32x32,2:4x4,2:8x4,1:8x4,1:8x8",
                     help="cases of the fine part, n:m x vector length")
     ap.add_argument("--ksweep-ks", default="64,1024,4096", help="reduction lengths of the ksweep part")
@@ -617,6 +623,8 @@ def main():
             tuple(tuple(int(v) for v in x.split("x")) for x in args.decode_shapes.split(",")),
             tuple(tuple(int(v) for v in x.split(":")) for x in args.decode_patterns.split(",")),
             tuple(args.decode_modes.split(",")))
+    if "decode_llm" in parts:
+        configs["decode_llm"] = run_decode(torch, pkg, (1, 16, 32), DECODE_LLM_SHAPES, ((2, 8),), DECODE_LLM_MODES)
     if "fine" in parts:
         configs["fine"] = run_fine(torch, pkg, tuple(
             (int(x.split(":")[0]), int(x.split(":")[1].split("x")[0]), int(x.split("x")[1])) for x in args.fine_cases.split(",")))

@@ -165,12 +165,25 @@ int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t*
  * before they would have left the caches anyway (a decode step walks through every layer of a
  * model: gigabytes between two uses of one B).  Only the decode kernel on the row list honours
  * it; measured there: faster when B comes from HBM, slower when a loop re-reads one B that fits
- * the 256 MB Infinity Cache.  Any other flag bit: NMSPMM_ERR_BAD_SHAPE.
+ * the 256 MB Infinity Cache.
+ * NMSPMM_DECODE_SPLIT: with fewer 32-column vectors than the GPU has compute units (Ncols below
+ * 8192 on an MI355X) the decode kernel on the row list leaves compute units idle; this flag lets it
+ * cut each vector's reduction across several workgroups, the last of which to finish adds the
+ * partial sums up in slice order (one launch, reproducible bit for bit).  The partial sums and the
+ * arrival counters live in a device-resident array of the library (the one nmspmm_spmm_noalloc
+ * uses), one copy per GPU: calls with this flag, and nmspmm_spmm_noalloc calls, that overlap on
+ * one GPU (two streams, two threads) race on it, so the flag is for callers that issue their
+ * multiplications on one stream.  Measured: K = 11008, Ncols = 4096 at 2:8, 1 / 16 / 32 rows
+ * 11.4 / 14.6 / 17.2 -> 10.1 / 11.3 / 12.6 us re-reading one B, 15.5 / 20.1 / 20.8 -> 11.4 / 13.5 /
+ * 14.6 us with B from HBM; the library splits only where the model expects a gain (long
+ * reductions, at most half as many vectors as compute units).
+ * Any other flag bit: NMSPMM_ERR_BAD_SHAPE.
  * row_index: NULL, or the row list nmspmm_row_index_device() made from these same D / column_info
  * (16-byte aligned).  With it, M <= 32 runs on the decode kernel that reads the list instead of
  * D and column_info; larger M ignore it. */
 #define NMSPMM_ACCUMULATE 1u
 #define NMSPMM_STREAM_B 2u
+#define NMSPMM_DECODE_SPLIT 4u
 int nmspmm_spmm_ex(const float* A, const float* B, const int32_t* D, const int32_t* column_info,
                    const int32_t* row_index, float* C, int M, int N, int K, int W, int window,
                    int kept, int vec_len, int Ns, int split_k, void* workspace,

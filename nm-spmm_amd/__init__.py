@@ -21,6 +21,7 @@ STATUS_NAMES = {
 TILE_SMALL, TILE_MEDIUM, TILE_LARGE, TILE_HUGE = 32, 64, 64, 128
 ACCUMULATE = 1  # flag of spmm_ex: with split_k > 1 the product is added to what C holds
 STREAM_B = 2    # flag of spmm_ex: B is loaded with the non-temporal hint (decode kernel on the row list)
+DECODE_SPLIT = 4  # flag of spmm_ex: the decode kernel may cut reductions across workgroups (library scratch)
 
 
 class NmSpmmError(RuntimeError):

@@ -48,6 +48,29 @@ void* noalloc_scratch()
     return g_scratch_ptr[dev];
 }
 
+// Arrival counters of the decode kernel's cut reductions (NMSPMM_DECODE_SPLIT): zero when the code
+// object is loaded, and every launch leaves them zero again.
+constexpr int kDecodeTickets = 1024;
+static __device__ unsigned int decode_tickets[kDecodeTickets];
+unsigned int* g_tickets_ptr[64] = {};
+
+unsigned int* decode_ticket_array()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        return nullptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_tickets_ptr[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(decode_tickets)) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        g_tickets_ptr[dev] = (unsigned int*)ptr;
+    }
+    return g_tickets_ptr[dev];
+}
+
 // The GPU's figures, asked once per device; without a device, an MI355X in single-partition mode.
 Machine g_machine[kMaxDevices];
 bool g_machine_known[kMaxDevices] = {};
@@ -481,7 +504,7 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
                      size_t workspace_bytes, void* stream, int lda, bool dry_run, int* lda_out, bool a_rowmajor = false,
                      unsigned flags = 0, const int32_t* row_index = nullptr)
 {
-    if (flags & ~(unsigned)(NMSPMM_ACCUMULATE | NMSPMM_STREAM_B))
+    if (flags & ~(unsigned)(NMSPMM_ACCUMULATE | NMSPMM_STREAM_B | NMSPMM_DECODE_SPLIT))
         return NMSPMM_ERR_BAD_SHAPE;
     if (!A || !B || !D || !C)
         return NMSPMM_ERR_NULL_POINTER;
@@ -509,6 +532,10 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     a.cinfo = column_info;
     a.row_index = row_index;
     a.stream_b = (flags & NMSPMM_STREAM_B) != 0;
+    a.decode_part = nullptr;
+    a.decode_part_bytes = 0;
+    a.decode_tickets = nullptr;
+    a.decode_ticket_count = 0;
     a.C = C;
     a.partial = split_k > 1 ? (float*)workspace : nullptr;
     a.slice_stride = slice_stride(M, N);
@@ -545,7 +572,19 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
         return kNotTaken;
     hipError_t e;
     if (decode_supported(a)) {
-        // decode sizes with the row list: one launch, reduction inside the workgroup
+        // decode sizes with the row list: one launch, reduction inside the workgroup (or, on request,
+        // across a few workgroups through the library's device-resident scratch)
+        if (flags & NMSPMM_DECODE_SPLIT) {
+            a.decode_part = (float*)noalloc_scratch();
+            a.decode_tickets = decode_ticket_array();
+            if (a.decode_part && a.decode_tickets) {
+                a.decode_part_bytes = NMSPMM_NOALLOC_MAX_BYTES;
+                a.decode_ticket_count = kDecodeTickets;
+            } else {
+                a.decode_part = nullptr;
+                a.decode_tickets = nullptr;
+            }
+        }
         e = launch_decode(a);
         g_last_kernel = "decode";
         return e == hipSuccess ? NMSPMM_OK : NMSPMM_ERR_HIP;

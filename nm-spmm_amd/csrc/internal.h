@@ -16,6 +16,10 @@ struct SpmmArgs {
     const int32_t* cinfo;  // [N/Ns][W/kept][window] or nullptr (low-sparsity layout)
     const int32_t* row_index;  // optional row list [N/32][ceil(W/16)][4][4] (spmm_decode.hip) or nullptr
     bool stream_b;         // B is loaded with the non-temporal hint (decode kernel on the row list)
+    float* decode_part;    // decode kernel on the row list: scratch for partial tiles when a vector's
+    size_t decode_part_bytes;  // reduction is cut across workgroups, and one arrival counter per vector
+    unsigned int* decode_tickets;  // (zero between launches); all three 0 / nullptr: never cut
+    int decode_ticket_count;
     float* C;              // row-major M x N
     float* partial;        // split_k slices of slice_stride floats when split_k > 1, else nullptr
     size_t slice_stride;   // M * N rounded up to a multiple of 4

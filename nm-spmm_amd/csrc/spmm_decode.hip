@@ -53,6 +53,11 @@ struct DecodeParams {
     int accumulate;
     int rotate;  // groups by which consecutive workgroups of an XCD stagger the start of their walk
     int xcds;    // accelerator dies: consecutive workgroup ids go to consecutive dies
+    // cut reductions (SPLIT): workgroup id = slice * vectors + vector; each of the `slices` workgroups
+    // of a vector leaves its partial tile in `part`, takes a ticket, and the last one adds them up
+    float* part;
+    unsigned int* tickets;
+    int slices, vectors;
 };
 
 __device__ inline __amdgpu_buffer_rsrc_t dc_rsrc(const void* base, uint32_t bytes)
@@ -63,7 +68,9 @@ __device__ inline __amdgpu_buffer_rsrc_t dc_rsrc(const void* base, uint32_t byte
 // HB: 16-row halves (1: M <= 16, 2: M <= 32).  PAIRS (HB == 2, column-major A with an even pitch):
 // one 64-bit load fetches rows 2 jl and 2 jl + 1 for the two halves, instead of two loads of rows
 // jl and jl + 16.  NT: B is loaded with the non-temporal hint (it is not kept in the caches).
-template <int HB, bool PAIRS, bool NT, int kDecodeWaves>
+// SPLIT: the reduction of a vector is cut across p.slices workgroups (fewer vectors than compute
+// units would otherwise leave compute units idle).
+template <int HB, bool PAIRS, bool NT, int kDecodeWaves, bool SPLIT = false>
 __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const DecodeParams p)
 {
     constexpr int kAux = NT ? 2 : 0;
@@ -71,7 +78,8 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kq = lane >> 4, jl = lane & 15;
-    const int v = blockIdx.x;
+    const int v = SPLIT ? (int)(blockIdx.x % (unsigned)p.vectors) : (int)blockIdx.x;
+    const int slice = SPLIT ? (int)(blockIdx.x / (unsigned)p.vectors) : 0;
     const int M = p.M, N = p.N;
 
     // every offset that relies on the descriptor's range check is a vector offset: the scalar
@@ -115,10 +123,15 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
     // workgroups of one XCD).  Positions advance by one with a wrap: the scalar work between a
     // group's MFMAs and the next group's loads is on every wave's critical path, so it is kept to
     // a compare and a select.
-    const int cnt = (p.G - wave + kDecodeWaves - 1) / kDecodeWaves;
+    // (a cut reduction: this workgroup's groups are [g_first, g_first + g_count), the partition rule
+    // of every split here)
+    int g_first = 0, g_count = p.G;
+    if (SPLIT)
+        split_windows(p.G, p.slices, slice, &g_first, &g_count);
+    const int cnt = (g_count - wave + kDecodeWaves - 1) / kDecodeWaves;
     const int first = cnt > 0 ? (int)((blockIdx.x / (unsigned)p.xcds) * (unsigned)p.rotate % (unsigned)cnt) : 0;
     auto after = [&](int x) { return x + 1 >= cnt ? 0 : x + 1; };
-    auto group_of = [&](int x) { return wave + x * kDecodeWaves; };
+    auto group_of = [&](int x) { return g_first + wave + x * kDecodeWaves; };
     float2 b[4];
     float a[4][HB];
     // A first: its addresses come from the row list, which has landed; the four loads of B follow
@@ -180,6 +193,43 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
             red[wave][8 * hb + 4 + x][lane] = acc_o[hb][x];
         }
     __syncthreads();
+    if constexpr (SPLIT) {
+        // Partial tile to scratch with device-scope stores (they reach the point where the other
+        // dies see them), wait for their acknowledgement, take a ticket.  No workgroup ever waits for
+        // another: whoever draws the last ticket of its vector finds all partial tiles complete.
+        constexpr int kTile = 8 * HB * 64;
+        __shared__ unsigned int ticket;
+        float* const mine = p.part + ((size_t)v * p.slices + slice) * kTile;
+        for (int x = wave; x < 8 * HB; x += kDecodeWaves) {
+            float s = red[0][x][lane];
+#pragma unroll
+            for (int y = 1; y < kDecodeWaves; ++y)
+                s += red[y][x][lane];
+            __hip_atomic_store(&mine[x * 64 + lane], s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        if (tid == 0)
+            ticket = __hip_atomic_fetch_add(&p.tickets[v], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (ticket != (unsigned int)(p.slices - 1))
+            return;
+        for (int x = wave; x < 8 * HB; x += kDecodeWaves) {
+            float s = 0.0f;
+            for (int z = 0; z < p.slices; ++z)
+                s += __hip_atomic_load(&p.part[((size_t)v * p.slices + z) * kTile + x * 64 + lane], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+            const int tile_row = 4 * kq + (x % 4);
+            const int row = PAIRS ? 2 * tile_row + x / 8 : 16 * (x / 8) + tile_row;
+            if (row < M) {
+                float* const dst = p.C + (size_t)row * N + (size_t)v * 32 + 2 * jl + (x % 8) / 4;
+                *dst = p.accumulate ? *dst + s : s;
+            }
+        }
+        if (tid == 0)
+            __hip_atomic_store(&p.tickets[v], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+        return;
+    }
     for (int x = wave; x < 8 * HB; x += kDecodeWaves) {
         float s = red[0][x][lane];
 #pragma unroll
@@ -229,12 +279,58 @@ hipError_t launch_decode(const SpmmArgs& a)
     p.accumulate = (a.accumulate && a.split_k > 1) ? 1 : 0;
     p.rotate = 0;
     p.xcds = machine().xcds;
-    const dim3 grid(a.N / 32), block16(64 * 16), block8(64 * 8);
+    const int vectors = a.N / 32;
+    const int cus = machine().cus;
     const bool pairs = a.M > 16 && !a.a_rowmajor && a.lda % 2 == 0 && a.M % 2 == 0;
+    const dim3 block16(64 * 16), block8(64 * 8);
+
+    // Fewer vectors than compute units: with scratch from the caller's flag, cut each reduction
+    // across as many workgroups as fill the GPU once, as long as every wave of a slice keeps at
+    // least four groups (the partial tiles, the ticket and the final sum cost about 1.3 us; measured
+    // at 128 vectors: K = 11008 at 2:8 gains 11 to 27 % re-reading one B and 26 to 33 % with B from
+    // HBM, K = 4096 nothing).
+    int slices = 1;
+    if (a.decode_part != nullptr && a.decode_tickets != nullptr) {
+        int s = cus / vectors;
+        if (s > p.G / 64)
+            s = p.G / 64;
+        if (s > 8)
+            s = 8;
+        const size_t tile_bytes = (size_t)(a.M <= 16 ? 8 : 16) * 64 * sizeof(float);
+        if (s >= 2 && vectors <= a.decode_ticket_count && (size_t)vectors * s * tile_bytes <= a.decode_part_bytes)
+            slices = s;
+    }
+    p.part = a.decode_part;
+    p.tickets = a.decode_tickets;
+    p.slices = slices;
+    p.vectors = vectors;
+    if (slices > 1) {
+        const dim3 grid((unsigned)(vectors * slices));
+        if (a.M <= 16) {
+            if (a.stream_b)
+                spmm_decode_kernel<1, false, true, 16, true><<<grid, block16, 0, a.stream>>>(p);
+            else
+                spmm_decode_kernel<1, false, false, 16, true><<<grid, block16, 0, a.stream>>>(p);
+        } else if (pairs) {
+            if (a.stream_b)
+                spmm_decode_kernel<2, true, true, 16, true><<<grid, block16, 0, a.stream>>>(p);
+            else
+                spmm_decode_kernel<2, true, false, 16, true><<<grid, block16, 0, a.stream>>>(p);
+        } else {
+            if (a.stream_b)
+                spmm_decode_kernel<2, false, true, 16, true><<<grid, block16, 0, a.stream>>>(p);
+            else
+                spmm_decode_kernel<2, false, false, 16, true><<<grid, block16, 0, a.stream>>>(p);
+        }
+        return hipGetLastError();
+    }
+
+    const dim3 grid((unsigned)vectors);
     if (a.M <= 16) {
         if (a.stream_b) {
             spmm_decode_kernel<1, false, true, 16><<<grid, block16, 0, a.stream>>>(p);
-        } else if (a.W >= 2048 && a.M >= 8) {
+        } else if (a.W >= 2048 && a.M >= 8 && vectors >= cus) {
+            // (with fewer workgroups than compute units 8 waves per CU are too few: 16 then)
             p.rotate = 5;
             spmm_decode_kernel<1, false, false, 8><<<grid, block8, 0, a.stream>>>(p);
         } else {

@@ -33,11 +33,17 @@ class NMSparseLinear(torch.nn.Module):
     weight: float32 CUDA tensor [out_features, in_features]; in_features % window == 0 and
     out_features % 32 == 0.  Leading dimensions of x are flattened into rows; any row count runs on
     the matrix-core kernels (the copy of x the row-major entry point makes is padded to a row pitch
-    of a multiple of four floats).
+    of a multiple of four floats).  single_stream=True promises that all forwards of such modules
+    are issued on one stream at a time; up to 32 rows they may then use more of the GPU when
+    out_features is small (fewer than 256 groups of 32).
     """
 
-    def __init__(self, weight, n, m, bias=None):
+    def __init__(self, weight, n, m, bias=None, single_stream=False):
         super().__init__()
+        # single_stream: the caller issues every forward of every such module on one stream at a
+        # time, which lets decode-sized calls cut their reductions across workgroups through the
+        # library's device-resident scratch (nmspmm.h: NMSPMM_DECODE_SPLIT)
+        self.flags = _nm.DECODE_SPLIT if single_stream else 0
         if weight.dtype != torch.float32 or not weight.is_cuda or weight.dim() != 2:
             raise ValueError("weight must be a 2-D float32 CUDA tensor")
         self.out_features, self.in_features = weight.shape
@@ -93,7 +99,7 @@ class NMSparseLinear(torch.nn.Module):
         if self._workspace is None or self._workspace.numel() < need or self._workspace.device != x.device:
             self._workspace = torch.empty(need, dtype=torch.float32, device=x.device)
         _nm.spmm_rowmajor(x2, self.values, self.indices, self.column_info, y, M, N, K, self.W, self.window, self.kept,
-                          self._workspace, 32, self.Ns, split, self.row_index)
+                          self._workspace, 32, self.Ns, split, self.row_index, self.flags)
         if add_bias and self.bias is not None:
             y += self.bias
         return y.reshape(*lead, N)

@@ -49,6 +49,9 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
         assert x["kernel"] == "decode" and x["kernel_reference_layout"] == "skinny"
         for mode in ("hot", "cold", "cold_stream_hint", "hot_reference_layout", "cold_reference_layout"):
             assert 0 < x[mode]["frac_hbm"] < 1.5 and x[mode]["us"] > 0
+    assert len(cfg["decode_llm"]) == 9
+    for x in cfg["decode_llm"]:
+        assert x["kernel"] == "decode" and x["hot_split"]["us"] > 0 and x["cold_split"]["us"] > 0
     assert [x["pattern"] for x in cfg["fine"]][:4] == ["4:32", "8:32", "16:32", "2:4"] and cfg["fine"][3]["vec_len"] == 4
     assert len(cfg["launch_constant"]) == 3 and len(cfg["compress"]) == 12 and len(cfg["rowmajor"]) == 5
     for x in d["preprocess"]:

@@ -128,7 +128,7 @@ def test_noalloc_entry_rejects_bad_arguments_without_a_gpu():
 def test_spmm_ex_rejects_unknown_flags_without_a_gpu():
     L = nmspmm.lib()
     args = [FAKE, FAKE, FAKE, None, None, FAKE, 128, 128, 128, 64, 32, 16, 32, 128, 1, None, 0]
-    assert L.nmspmm_spmm_ex(*args, 4, None) == 2
+    assert L.nmspmm_spmm_ex(*args, 8, None) == 2
     assert L.nmspmm_spmm_ex(FAKE, FAKE, FAKE, None, None, None, 128, 128, 128, 64, 32, 16, 32, 128, 1, None, 0, 1, None) == 1
     args[4] = FAKE + 4   # a row list that is not 16-byte aligned
     assert L.nmspmm_spmm_ex(*args, 0, None) == 8

@@ -219,3 +219,59 @@ def test_row_major_activations_on_the_row_list(oracle, M, n, m):
     assert nmspmm.last_kernel() == "decode"
     got = C.cpu().numpy()
     assert np.isfinite(got).all() and scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
+
+
+@pytest.mark.parametrize("M", [1, 7, 16, 19, 32])
+@pytest.mark.parametrize("n,m,K,N", [(2, 8, 11008, 4096), (2, 8, 8192, 2048), (1, 8, 16384, 1024), (2, 4, 4096, 4096), (2, 4, 16384, 1024), (3, 8, 8192, 2048)])
+def test_reductions_cut_across_workgroups(oracle, M, n, m, K, N):
+    """NMSPMM_DECODE_SPLIT with fewer column vectors than compute units and a long reduction: two to
+    eight workgroups per vector, the last one to arrive adds the partial tiles up.  Against the
+    checker; then forty more launches, every one bit-identical to the first (the sum is taken in
+    slice order whoever arrives last, and the arrival counters are left at zero)."""
+    d = datagen.init_data(M, N, K, n, m, seed=M + K // 64, dist="normal", b_scale=0.02)
+    W = d["W"]
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    R = gpu_row_list(D, cinfo, W, N, window, kept, 128)
+    A, B, Dd = dev(d["A_km"]), dev(d["BT"]), dev(D)
+    ci = None if cinfo is None else dev(cinfo)
+    want = want_c(oracle, d)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    nmspmm.spmm_ex(A, B, Dd, ci, C, M, N, K, W, window, kept, 32, 128, 1, None, nmspmm.DECODE_SPLIT, R)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == "decode"
+    first = C.clone()
+    assert np.isfinite(first.cpu().numpy()).all() and scaled_max_error(first.cpu().numpy(), want) <= REL_TOL
+    for _ in range(40):
+        C.fill_(float("nan"))
+        nmspmm.spmm_ex(A, B, Dd, ci, C, M, N, K, W, window, kept, 32, 128, 1, None, nmspmm.DECODE_SPLIT, R)
+    torch.cuda.synchronize()
+    assert torch.equal(C, first)
+    # the same call without the flag (one workgroup per vector) agrees within the bound
+    nmspmm.spmm_ex(A, B, Dd, ci, C, M, N, K, W, window, kept, 32, 128, 1, None, 0, R)
+    torch.cuda.synchronize()
+    assert scaled_max_error(C.cpu().numpy(), want) <= REL_TOL
+    # with the hint for streamed weights, and adding to C like a split call of the reference
+    C0 = np.random.default_rng(M).standard_normal((M, N)).astype(np.float32)
+    Cd = dev(C0)
+    ws = torch.empty(nmspmm.workspace_bytes(M, N, 2) // 4, dtype=torch.float32, device="cuda")
+    nmspmm.spmm_ex(A, B, Dd, ci, Cd, M, N, K, W, window, kept, 32, 128, 2, ws,
+                   nmspmm.DECODE_SPLIT | nmspmm.STREAM_B | nmspmm.ACCUMULATE, R)
+    torch.cuda.synchronize()
+    assert scaled_max_error(Cd.cpu().numpy(), want_c(oracle, d, C0)) <= REL_TOL
+
+
+def test_the_split_flag_changes_nothing_where_every_compute_unit_has_a_vector(oracle):
+    """8192 columns are 256 vectors: nothing to gain, the flag is ignored and the result is the
+    unsplit kernel's bit for bit."""
+    M, N, K, n, m = 8, 8192, 2048, 2, 8
+    d = datagen.init_data(M, N, K, n, m, seed=11, dist="normal", b_scale=0.02)
+    W = d["W"]
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    R = gpu_row_list(D, cinfo, W, N, window, kept, 128)
+    A, B, Dd, ci = dev(d["A_km"]), dev(d["BT"]), dev(D), dev(cinfo)
+    C1 = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    C2 = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    nmspmm.spmm_ex(A, B, Dd, ci, C1, M, N, K, W, window, kept, 32, 128, 1, None, 0, R)
+    nmspmm.spmm_ex(A, B, Dd, ci, C2, M, N, K, W, window, kept, 32, 128, 1, None, nmspmm.DECODE_SPLIT, R)
+    torch.cuda.synchronize()
+    assert torch.equal(C1, C2)

@@ -151,7 +151,7 @@ def test_split_k_adds_to_c_like_the_reference(oracle, M, N, K, n, m, family, spl
 def test_unknown_flag_bits_are_rejected():
     with pytest.raises(nmspmm.NmSpmmError, match="BAD_SHAPE"):
         x = torch.zeros(64 * 64, dtype=torch.float32, device="cuda")
-        nmspmm.spmm_ex(x, x, x.int(), None, x, 32, 32, 32, 16, 32, 16, 32, 32, 1, None, 4)
+        nmspmm.spmm_ex(x, x, x.int(), None, x, 32, 32, 32, 16, 32, 16, 32, 32, 1, None, 8)
 
 
 @pytest.mark.parametrize("M", [1, 2, 8, 13, 16, 30, 32])

@@ -37,6 +37,24 @@ def test_linear_standin_matches_dense_layer_with_pruned_weight(oracle, out_f, in
     assert np.array_equal(layer.dense_weight().cpu().numpy(), pruned.T)
 
 
+def test_decode_sized_forward_of_a_layer_with_few_output_features_on_one_stream(oracle):
+    """single_stream=True: a decode-sized forward of a layer with fewer than 256 groups of 32 output
+    features and a long reduction cuts its reductions across workgroups; same result within the
+    bound, and row-major activations are read in place (8 rows) or copied (24 rows)."""
+    op = importlib.import_module("nm-spmm_amd.torch_op")
+    g = torch.Generator(device="cuda").manual_seed(5)
+    w = torch.randn((2048, 8192), generator=g, dtype=torch.float32, device="cuda") * 0.05
+    plain = op.NMSparseLinear(w, 2, 8)
+    split = op.NMSparseLinear(w, 2, 8, single_stream=True)
+    for rows in (1, 8, 24):
+        x = torch.randn((rows, 8192), generator=g, dtype=torch.float32, device="cuda")
+        y0, y1 = plain(x), split(x)
+        assert nmspmm.last_kernel() == "decode"
+        want = x.double() @ plain.dense_weight().double().t()
+        assert scaled_max_error(y1.cpu().numpy(), want.cpu().numpy()) <= REL_TOL
+        assert scaled_max_error(y0.cpu().numpy(), want.cpu().numpy()) <= REL_TOL
+
+
 def test_rejects_unsupported_layers():
     op = importlib.import_module("nm-spmm_amd.torch_op")
     w = torch.zeros((64, 80), dtype=torch.float32, device="cuda")
