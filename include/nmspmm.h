@@ -214,7 +214,8 @@ int nmspmm_row_index_device(const int32_t* dD, const int32_t* d_column_info, int
  * overwritten; results are bit-identical to nmspmm_spmm with a caller-owned workspace.  All calls
  * on a GPU share that GPU's array (the kernels overwrite every slice element they later read, so
  * nothing needs clearing between calls): split calls that overlap in time on one GPU, from
- * different streams or threads, race on it and must be serialised by the caller. */
+ * different streams or threads, race on it and must be serialised by the caller (so must they and
+ * nmspmm_spmm_ex calls with NMSPMM_DECODE_SPLIT, which keep their partial sums in the same array). */
 #define NMSPMM_NOALLOC_MAX_BYTES (32u << 20)
 int nmspmm_spmm_noalloc(const float* A, const float* B, const int32_t* D, const int32_t* column_info,
                         float* C, int M, int N, int K, int W, int window, int kept, int vec_len,
