@@ -79,3 +79,62 @@ def test_random_shape(oracle, case):
     got = C.cpu().numpy()
     assert np.isfinite(got).all()
     assert scaled_max_error(got, want) <= REL_TOL
+
+
+def draw_decode_case(rng):
+    """One random decode-sized problem on the row list: (M, N, K, n, m, Ns, flags, row_major, accumulate)."""
+    while True:
+        n, m = rng.choice([(2, 4), (3, 8), (2, 8), (1, 8), (8, 32), (4, 32)])
+        window, kept, _ = kernel_geometry(n, m)
+        Ns = rng.choice([128, 64, 32])
+        N = Ns * rng.randint(1, 2048 // Ns)
+        K = window * rng.choice([rng.randint(1, 24), rng.randint(24, 16384 // window)])
+        M = rng.randint(1, 32)
+        W = K // window * kept
+        if M * N * W > MAX_MACS:
+            continue
+        flags = rng.choice([0, 0, 2, 4, 4, 6])
+        return M, N, K, n, m, Ns, flags, rng.random() < 0.3, rng.random() < 0.3
+
+
+DECODE_CASES = [draw_decode_case(random.Random(9000 + i)) for i in range(120)]
+
+
+@pytest.mark.parametrize("case", DECODE_CASES,
+                         ids=lambda c: "M%d-N%d-K%d-%dof%d-Ns%d-f%d-%s-%s" % (c[:7] + ("rm" if c[7] else "cm", "acc" if c[8] else "st")))
+def test_random_decode_shape(oracle, case):
+    """Up to 32 rows on the row list, with the stream hint and the cut reductions drawn at random
+    (long reductions on few column vectors are among the cases, so the cut is taken), both storage
+    orders of A, storing and adding to C."""
+    M, N, K, n, m, Ns, flags, row_major, accumulate = case
+    d = datagen.init_data(M, N, K, n, m, seed=M * 17 + N + K + n, dist="normal", b_scale=0.05)
+    W = d["W"]
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, Ns)
+    dD, dcinfo = dev(D), None if cinfo is None else dev(cinfo)
+    R = torch.empty(nmspmm.row_index_ints(W, N), dtype=torch.int32, device="cuda")
+    nmspmm.row_index_device(dD, dcinfo, W, N, window, kept, Ns, R)
+    C0 = np.random.default_rng(M + N).standard_normal((M, N)).astype(np.float32) if accumulate else None
+    C = dev(C0) if accumulate else torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    split_k = 2 if accumulate and K // window >= 2 else 1
+    if accumulate and split_k == 1:
+        C0 = None
+        C.fill_(float("nan"))
+    if accumulate and split_k > 1:
+        flags |= nmspmm.ACCUMULATE
+    if row_major:
+        ws = torch.full((nmspmm.workspace_bytes_rowmajor(M, N, K, split_k) // 4,), float("nan"), dtype=torch.float32,
+                        device="cuda")
+        nmspmm.spmm_rowmajor(dev(d["A_km"].T), dev(d["BT"]), dD, dcinfo, C, M, N, K, W, window, kept, ws, 32, Ns, split_k,
+                             R, flags)
+    else:
+        ws = None
+        if split_k > 1:
+            ws = torch.full((nmspmm.workspace_bytes(M, N, split_k) // 4,), float("nan"), dtype=torch.float32, device="cuda")
+        nmspmm.spmm_ex(dev(d["A_km"]), dev(d["BT"]), dD, dcinfo, C, M, N, K, W, window, kept, 32, Ns, split_k, ws, flags, R)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() == "decode"
+    want = oracle.gemm_cpu(d["A_km"].reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), M, N, W, 32,
+                           C=None if C0 is None else C0.reshape(-1).copy()).reshape(M, N)
+    got = C.cpu().numpy()
+    assert np.isfinite(got).all()
+    assert scaled_max_error(got, want) <= REL_TOL
