@@ -18,6 +18,20 @@ namespace nmspmm {
 // remaining ones by lane exchange.
 constexpr int kColsPerBlock = 1024;
 
+typedef unsigned int cuintx4 __attribute__((ext_vector_type(4)));
+
+// The expanded operand is stored system-coherent (sc1, bit 4 of the cache-policy operand): written
+// through, the stores leave no dirty lines in L2 for the end of the launch to flush, which makes
+// the expansion 4 to 20 % shorter (4096 x 4096 at 2:8: 12.4 -> 10.0 us); the compression, which
+// writes less than it reads, gains nothing from it and keeps plain stores.  `base` is the same for
+// the whole workgroup: the rows of one window, `bytes` long.
+__device__ inline void store_segment(float* base, uint32_t bytes, uint32_t offset_bytes, float4 v)
+{
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(base, 0, (int)bytes, 0x00020000);
+    const cuintx4 x = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
+    __builtin_amdgcn_raw_buffer_store_b128(x, rs, (int)offset_bytes, 0, 16);
+}
+
 template <int MW>
 __global__ void __launch_bounds__(256)
 compress_kernel(const float* __restrict__ B, float* __restrict__ BT, int32_t* __restrict__ DT, int N, int Q,
@@ -101,7 +115,7 @@ decompress_kernel(const float* __restrict__ BT, const int32_t* __restrict__ DT, 
             const int p = __popc(keep & ((1u << r) - 1u));
             x = *reinterpret_cast<const float4*>(BT + ((size_t)w * n + p) * N + col);
         }
-        *reinterpret_cast<float4*>(B + ((size_t)w * MW + r) * N + col) = x;
+        store_segment(B + (size_t)w * MW * N, (uint32_t)MW * N * 4u, ((uint32_t)r * N + col) * 4u, x);
     }
 }
 
