@@ -14,6 +14,8 @@ Prints ONE JSON line:
                      decode  M in {1, 8, 16, 32} x two weight shapes x {1:8, 2:8}: microseconds and
                              algorithmic GB/s against the 8 TB/s HBM bound, with B re-read from the
                              caches ("hot") and streamed from HBM ("cold"), row list on and off
+                     decode_llm, decode_wide: decode sizes of the LLM-layer weight shapes with and
+                             without cut reductions; 48 and 64 rows on the row list
                      fine    4:32, 8:32, 16:32 and 2:4 with 4-column vectors at 4096 cubed
                      launch_constant, compress, rowmajor: the part of a launch that does not scale
                              with K; dense <-> compressed conversion; row-major activations
@@ -45,7 +47,7 @@ M = N = K = 4096
 PATTERNS = [(2, 4), (3, 8), (2, 8), (1, 8)]  # first one is the headline
 NS = 128
 GEOMETRY = {(1, 1): (32, 32), (1, 2): (32, 16), (3, 8): (32, 12), (1, 4): (64, 16), (1, 8): (64, 8)}
-PARTS = ("sweep", "llm", "decode", "decode_llm", "fine", "ksweep", "compress", "rowmajor", "preprocess", "dispatch", "cpu")
+PARTS = ("sweep", "llm", "decode", "decode_llm", "decode_wide", "fine", "ksweep", "compress", "rowmajor", "preprocess", "dispatch", "cpu")
 
 
 def geometry(n, m):
@@ -290,7 +292,7 @@ def run_decode(torch, pkg, rows_list=(1, 8, 16, 32), shapes=((8192, 8192), (4096
     out = []
     for (k, n_cols) in shapes:
         for (n, m) in patterns:
-            op = GpuOperands(torch, pkg, 32, n_cols, k, n, m, row_list=True)
+            op = GpuOperands(torch, pkg, max(rows_list), n_cols, k, n, m, row_list=True)
             b_bytes = op.B.numel() * 4
             copies = [op.B] + [op.B.clone() for _ in range(int(640e6 // b_bytes))]
             for m_rows in rows_list:
@@ -625,6 +627,10 @@ def main():
             tuple(args.decode_modes.split(",")))
     if "decode_llm" in parts:
         configs["decode_llm"] = run_decode(torch, pkg, (1, 16, 32), DECODE_LLM_SHAPES, ((2, 8),), DECODE_LLM_MODES)
+    if "decode_wide" in parts:
+        # beyond the baseline's row counts: 33 to 64 rows on the row list (serving batches)
+        configs["decode_wide"] = run_decode(torch, pkg, (48, 64), ((8192, 8192),), ((1, 8), (2, 8)),
+                                            ("hot", "cold", "hot_reference_layout", "cold_reference_layout"))
     if "fine" in parts:
         configs["fine"] = run_fine(torch, pkg, tuple(
             (int(x.split(":")[0]), int(x.split(":")[1].split("x")[0]), int(x.split("x")[1])) for x in args.fine_cases.split(",")))

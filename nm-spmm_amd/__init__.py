@@ -99,6 +99,27 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
+def _need(fn, **tensors):
+    """The C interface takes plain pointers and cannot see how much memory lies behind them; a
+    tensor smaller than the shape arguments imply would make a kernel read or write beyond it (a
+    GPU memory fault).  name=(tensor, elements): raises ValueError when the tensor holds fewer.
+    None and shapes the library rejects anyway (non-positive counts) are left to the library."""
+    for name, (t, count) in tensors.items():
+        if t is None or not isinstance(count, int) or count <= 0:
+            continue
+        if t.numel() < count:
+            raise ValueError("%s: %s holds %d elements, the shape arguments need %d" % (fn, name, t.numel(), count))
+
+
+def _spmm_need(fn, A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len, Ns, row_index=None, a_elems=None):
+    ok = all(isinstance(v, int) and v > 0 for v in (M, N, K, W, window, kept, vec_len, Ns))
+    if not ok:
+        return
+    _need(fn, A=(A, a_elems if a_elems is not None else K * M), B=(B, W * N), D=(D, W * (N // vec_len)),
+          C=(C, M * N), column_info=(cinfo, int(lib().nmspmm_column_info_ints(W, kept, window, N, Ns))),
+          row_index=(row_index, int(lib().nmspmm_row_index_ints(W, N))))
+
+
 def pattern_from_sparsity(sparsity):
     w, k, h = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
     _check("nmspmm_pattern_from_sparsity",
@@ -113,6 +134,7 @@ def last_kernel():
 # ---- device-pointer forms: arguments are torch tensors on the GPU -----------------------------------
 
 def trans_index_device(dDT, W, N, Q, pN, pM):
+    _need("trans_index_device", dDT=(dDT, W * Q))
     n, m = ctypes.c_int(pN), ctypes.c_int(pM)
     _check("nmspmm_trans_index_device",
            lib().nmspmm_trans_index_device(_ptr(dDT), W, N, Q, ctypes.byref(n), ctypes.byref(m), _stream()))
@@ -120,11 +142,14 @@ def trans_index_device(dDT, W, N, Q, pN, pM):
 
 
 def preprocess_low_device(dDT_in, dDT_out, W, Q, Ns, vec_len=32):
+    _need("preprocess_low_device", dDT_in=(dDT_in, W * Q), dDT_out=(dDT_out, W * Q))
     _check("nmspmm_preprocess_low_device",
            lib().nmspmm_preprocess_low_device(_ptr(dDT_in), _ptr(dDT_out), W, Q, Ns, vec_len, _stream()))
 
 
 def preprocess_high_device(d_cinfo, pM, pN, dDT_in, dDT_out, W, Q, N, Ns, vec_len=32):
+    _need("preprocess_high_device", dDT_in=(dDT_in, W * Q), dDT_out=(dDT_out, W * Q),
+          column_info=(d_cinfo, int(column_info_ints(W, pN, pM, N, Ns))))
     _check("nmspmm_preprocess_high_device",
            lib().nmspmm_preprocess_high_device(_ptr(d_cinfo), pM, pN, _ptr(dDT_in), _ptr(dDT_out), W, Q, N, Ns,
                                                vec_len, _stream()))
@@ -132,11 +157,15 @@ def preprocess_high_device(d_cinfo, pM, pN, dDT_in, dDT_out, W, Q, N, Ns, vec_le
 
 def compress_device(dB, K, N, n, m, dBT, dDT, vec_len=32):
     """Dense row-major float32[K][N] on the GPU -> BT float32[K*n/m][N], DT int32[K*n/m][N/vec_len]."""
+    if min(K, N, n, m, vec_len) > 0:
+        _need("compress_device", dB=(dB, K * N), dBT=(dBT, K // m * n * N), dDT=(dDT, K // m * n * (N // vec_len)))
     _check("nmspmm_compress_device",
            lib().nmspmm_compress_device(_ptr(dB), K, N, n, m, vec_len, _ptr(dBT), _ptr(dDT), _stream()))
 
 
 def decompress_device(dBT, dDT, K, N, n, m, dB, vec_len=32):
+    if min(K, N, n, m, vec_len) > 0:
+        _need("decompress_device", dB=(dB, K * N), dBT=(dBT, K // m * n * N), dDT=(dDT, K // m * n * (N // vec_len)))
     _check("nmspmm_decompress_device",
            lib().nmspmm_decompress_device(_ptr(dBT), _ptr(dDT), K, N, n, m, vec_len, _ptr(dB), _stream()))
 
@@ -144,6 +173,7 @@ def decompress_device(dBT, dDT, K, N, n, m, dB, vec_len=32):
 def preprocess_device(dDT_in, n, m, W, Q, N, Ns, dD_out, d_cinfo):
     """Widening + re-blocking (+ ranking) in one kernel; returns (window, kept)."""
     window, kept = ctypes.c_int(0), ctypes.c_int(0)
+    _need("preprocess_device", dDT_in=(dDT_in, W * Q), dD_out=(dD_out, W * Q))
     _check("nmspmm_preprocess_device",
            lib().nmspmm_preprocess_device(_ptr(dDT_in), n, m, W, Q, N, Ns, _ptr(dD_out), _ptr(d_cinfo),
                                           ctypes.byref(window), ctypes.byref(kept), _stream()))
@@ -164,6 +194,7 @@ def workspace_bytes(M, N, split_k):
 
 def spmm(A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len=32, Ns=128, split_k=1, workspace=None):
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _spmm_need("spmm", A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len, Ns)
     _check("nmspmm_spmm",
            lib().nmspmm_spmm(_ptr(A), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(C), M, N, K, W, window, kept, vec_len,
                              Ns, split_k, _ptr(workspace), ws_bytes, _stream()))
@@ -172,6 +203,7 @@ def spmm(A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len=32, Ns=128, split_
 def spmm_ex(A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len=32, Ns=128, split_k=1, workspace=None, flags=0,
             row_index=None):
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _spmm_need("spmm_ex", A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len, Ns, row_index)
     _check("nmspmm_spmm_ex",
            lib().nmspmm_spmm_ex(_ptr(A), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(row_index), _ptr(C), M, N, K, W, window,
                                 kept, vec_len, Ns, split_k, _ptr(workspace), ws_bytes, flags, _stream()))
@@ -183,6 +215,8 @@ def row_index_ints(W, N):
 
 def row_index_device(D, cinfo, W, N, window, kept, Ns, row_index):
     """Row list for the decode kernel from the preprocessed D (and column_info)."""
+    if min(W, N) > 0:
+        _need("row_index_device", D=(D, W * (N // 32)), row_index=(row_index, int(row_index_ints(W, N))))
     _check("nmspmm_row_index_device",
            lib().nmspmm_row_index_device(_ptr(D), _ptr(cinfo), W, N, window, kept, Ns, _ptr(row_index), _stream()))
 
@@ -192,18 +226,21 @@ NOALLOC_MAX_BYTES = 32 << 20  # NMSPMM_NOALLOC_MAX_BYTES
 
 def spmm_noalloc(A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len=32, Ns=128, split_k=1):
     """spmm with the split-K slices in the library's fixed device-resident scratch: allocates nothing."""
+    _spmm_need("spmm_noalloc", A, B, D, cinfo, C, M, N, K, W, window, kept, vec_len, Ns)
     _check("nmspmm_spmm_noalloc",
            lib().nmspmm_spmm_noalloc(_ptr(A), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(C), M, N, K, W, window, kept,
                                      vec_len, Ns, split_k, _stream()))
 
 
 def gemm_low_sparsity(tile, A, B, D, C, M, N, K, W, sparsity, split_k=1):
+    _need("gemm_low_sparsity", A=(A, K * M), B=(B, W * N), D=(D, W * (N // 32)), C=(C, M * N))
     _check("nmspmm_gemm_low_sparsity",
            lib().nmspmm_gemm_low_sparsity(tile, _ptr(A), _ptr(B), _ptr(D), _ptr(C), M, N, K, W, sparsity, split_k,
                                           _stream()))
 
 
 def gemm_high_sparsity(tile, A, B, D, cinfo, C, M, N, K, W, sparsity, split_k=1):
+    _need("gemm_high_sparsity", A=(A, K * M), B=(B, W * N), D=(D, W * (N // 32)), C=(C, M * N))
     _check("nmspmm_gemm_high_sparsity",
            lib().nmspmm_gemm_high_sparsity(tile, _ptr(A), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(C), M, N, K, W,
                                            sparsity, split_k, _stream()))
@@ -212,6 +249,7 @@ def gemm_high_sparsity(tile, A, B, D, cinfo, C, M, N, K, W, sparsity, split_k=1)
 # ---- host-pointer forms: arguments are C-contiguous numpy int32 arrays, updated in place ----------
 
 def transpose_device(src, rows, cols, dst):
+    _need("transpose_device", src=(src, rows * cols), dst=(dst, rows * cols))
     _check("nmspmm_transpose_device", lib().nmspmm_transpose_device(_ptr(src), rows, cols, _ptr(dst), _stream()))
 
 
@@ -222,6 +260,7 @@ def workspace_bytes_rowmajor(M, N, K, split_k):
 def spmm_rowmajor(A_rm, B, D, cinfo, C, M, N, K, W, window, kept, workspace, vec_len=32, Ns=128, split_k=1,
                   row_index=None, flags=0):
     """A_rm is row-major M x K; `workspace` (float32 tensor) holds workspace_bytes_rowmajor() bytes."""
+    _spmm_need("spmm_rowmajor", A_rm, B, D, cinfo, C, M, N, K, W, window, kept, vec_len, Ns, row_index)
     _check("nmspmm_spmm_rowmajor_ex",
            lib().nmspmm_spmm_rowmajor_ex(_ptr(A_rm), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(row_index), _ptr(C), M, N, K, W,
                                          window, kept, vec_len, Ns, split_k, _ptr(workspace),
@@ -252,6 +291,7 @@ def tile_wave_rows(M, N, W, kept, Ns=128, split_k=1):
 
 def gemm_auto(A, B, D, cinfo, C, M, N, K, W, sparsity):
     """Multiply with the library's own choice of split_k (indices preprocessed for Ns = 128)."""
+    _need("gemm_auto", A=(A, K * M), B=(B, W * N), D=(D, W * (N // 32)), C=(C, M * N))
     _check("nmspmm_gemm_auto",
            lib().nmspmm_gemm_auto(_ptr(A), _ptr(B), _ptr(D), _ptr(cinfo), _ptr(C), M, N, K, W, sparsity, _stream()))
 

@@ -571,7 +571,10 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     if (a_rowmajor && !(M <= 32 && (skinny_supported(a) || decode_supported(a))))
         return kNotTaken;
     hipError_t e;
-    if (decode_supported(a)) {
+    // up to 32 rows the kernels with one workgroup per vector always win; up to 128 they compete
+    // with the tile kernel at the caller's split
+    const bool decode_wins = model_decode_seconds(M, N, W / kept, kept) < model_tile_seconds(M, N, W / kept, kept, split_k);
+    if (decode_supported(a) && (M <= 32 || decode_wins || !mfma_supported(a))) {
         // decode sizes with the row list: one launch, reduction inside the workgroup (or, on request,
         // across a few workgroups through the library's device-resident scratch)
         if (flags & NMSPMM_DECODE_SPLIT) {
@@ -589,9 +592,6 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
         g_last_kernel = "decode";
         return e == hipSuccess ? NMSPMM_OK : NMSPMM_ERR_HIP;
     }
-    // up to 32 rows the decode kernel always wins; up to 128 it competes with the tile kernel at
-    // the caller's split
-    const bool decode_wins = model_decode_seconds(M, N, W / kept, kept) < model_tile_seconds(M, N, W / kept, kept, split_k);
     if (skinny_supported(a) && (M <= 32 || decode_wins || !mfma_supported(a))) {
         // one launch, reduction inside the workgroup: split_k and the workspace are not needed
         e = launch_skinny(a);

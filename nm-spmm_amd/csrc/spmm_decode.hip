@@ -1,4 +1,4 @@
-// Decode-sized multiplication (M <= 32) on the row list: the index format this library adds for
+// Decode-sized multiplication (M <= 32, and 33 to 64 rows of a column-major A) on the row list: the index format this library adds for
 // the memory-bound case, next to the reference's D / column_info buffers (which stay as they are).
 //
 // The reference layout makes a kernel chase two dependent loads before it can ask for a row of A:
@@ -21,7 +21,7 @@
 // loads B[4 s + kq][2 jl .. 2 jl + 1] with one 64-bit load (four 128-byte row segments per wave and
 // instruction, each byte of B read once) and A[jl][row]; even and odd columns accumulate in two
 // MFMA tiles.  17 to 32 rows take a second pair of tiles for the other 16 rows with the same B
-// operands.  The waves add their tiles up through LDS in wave order (deterministic, one launch,
+// operands, 33 to 64 rows four pairs.  The waves add their tiles up through LDS in wave order (deterministic, one launch,
 // no workspace).  Measured on the MI355X: more than one group per wave in flight does not help.
 // The counters show a CU with about 64 requests outstanding whatever the kernel does, which looks
 // like what its vector L1 keeps in flight: the 16 waves' one group each (256 lines of B plus their
@@ -65,16 +65,21 @@ __device__ inline __amdgpu_buffer_rsrc_t dc_rsrc(const void* base, uint32_t byte
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }
 
-// HB: 16-row halves (1: M <= 16, 2: M <= 32).  PAIRS (HB == 2, column-major A with an even pitch):
-// one 64-bit load fetches rows 2 jl and 2 jl + 1 for the two halves, instead of two loads of rows
-// jl and jl + 16.  NT: B is loaded with the non-temporal hint (it is not kept in the caches).
+// HB: 16-row halves (1: M <= 16, 2: M <= 32, 4: M <= 64).  WIDE (column-major A): one
+// load fetches the rows of several halves at once, instead of one 32-bit load per half: HB = 2 a
+// 64-bit load of rows 2 jl, 2 jl + 1; HB = 4 a 128-bit load of rows 4 jl .. 4 jl + 3 (half hb is then
+// the rows HB t + hb, t the tile row; written for any multiple of four halves, two such loads 64 rows
+// apart for eight, which was measured and lost to the tile kernel: 41 against 36 us at 128 rows).  NT: B is loaded with the non-temporal hint (it is not kept in the caches).
 // SPLIT: the reduction of a vector is cut across p.slices workgroups (fewer vectors than compute
 // units would otherwise leave compute units idle).
-template <int HB, bool PAIRS, bool NT, int kDecodeWaves, bool SPLIT = false>
+template <int HB, bool WIDE, bool NT, int kDecodeWaves, bool SPLIT = false>
 __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const DecodeParams p)
 {
+    constexpr int HBW = HB < 4 ? HB : 4;   // halves that one wide load serves
+    constexpr int NW = HB / HBW;           // wide loads per lane and kept row
+    constexpr int HBC = HB < 2 ? HB : 2;   // halves per pass of the reduction through LDS
     constexpr int kAux = NT ? 2 : 0;
-    __shared__ float red[kDecodeWaves][8 * HB][64];
+    __shared__ float red[kDecodeWaves][8 * HBC][64];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kq = lane >> 4, jl = lane & 15;
@@ -94,8 +99,13 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
     // 2:8).  The list holds row + 1; entry 0 (no such kept row, or a read beyond the list) selects
     // an offset beyond the descriptor, which loads 0.
     uint32_t a_lane[HB];
-    if (PAIRS) {
-        a_lane[0] = (uint32_t)min(jl, M / 2 - 1) * 8u - a_stride;
+    if (WIDE) {
+        // lane jl holds rows HBW jl .. HBW jl + HBW - 1 of each group of 16 HBW rows; a lane whose
+        // rows all lie beyond M reads the last run that holds a live row (what a run reads beyond
+        // row M - 1 is whatever follows it in A, or 0 beyond its end: those tile rows are never stored)
+#pragma unroll
+        for (int w = 0; w < NW; ++w)
+            a_lane[w] = (uint32_t)min(16 * HBW * w + HBW * jl, (M - 1) / HBW * HBW) * (uint32_t)sizeof(float) - a_stride;
     } else {
 #pragma unroll
         for (int hb = 0; hb < HB; ++hb)
@@ -134,29 +144,46 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
     auto group_of = [&](int x) { return g_first + wave + x * kDecodeWaves; };
     float2 b[4];
     float a[4][HB];
+    auto load_a_step = [&](int t, const dintx4& rows) {
+        if constexpr (WIDE && HBW == 2) {
+            const auto x = __builtin_amdgcn_raw_buffer_load_b64(ra, a_offset(a_lane[0], rows[t]), 0, 0);
+            a[t][0] = __int_as_float(x[0]);
+            a[t][1] = __int_as_float(x[1]);
+        } else if constexpr (WIDE) {
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                const auto x = __builtin_amdgcn_raw_buffer_load_b128(ra, a_offset(a_lane[w], rows[t]), 0, 0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    a[t][4 * w + e] = __int_as_float(x[e]);
+            }
+        } else {
+#pragma unroll
+            for (int hb = 0; hb < HB; ++hb)
+                a[t][hb] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(ra, a_offset(a_lane[hb], rows[t]), 0, 0));
+        }
+    };
+    auto load_b_step = [&](int t, int g) {
+        // rows at or beyond W (the tail of the last group) lie beyond the descriptor: 0
+        const auto x = __builtin_amdgcn_raw_buffer_load_b64(rb, b_lane + (uint32_t)g * 4u * b_step + t * b_step, 0, kAux);
+        b[t] = make_float2(__int_as_float(x[0]), __int_as_float(x[1]));
+    };
     // A first: its addresses come from the row list, which has landed; the four loads of B follow
     // (measured against B first: 1 to 2 % faster)
     auto load_operands = [&](int g, const dintx4& rows) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            if constexpr (PAIRS) {
-                const auto x = __builtin_amdgcn_raw_buffer_load_b64(ra, a_offset(a_lane[0], rows[t]), 0, 0);
-                a[t][0] = __int_as_float(x[0]);
-                a[t][1] = __int_as_float(x[1]);
-            } else {
-#pragma unroll
-                for (int hb = 0; hb < HB; ++hb)
-                    a[t][hb] = __int_as_float(
-                        __builtin_amdgcn_raw_buffer_load_b32(ra, a_offset(a_lane[hb], rows[t]), 0, 0));
-            }
-        }
+        for (int t = 0; t < 4; ++t)
+            load_a_step(t, rows);
         __builtin_amdgcn_sched_barrier(0);
-        const uint32_t b_group = b_lane + (uint32_t)g * 4u * b_step;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            // rows at or beyond W (the tail of the last group) lie beyond the descriptor: 0
-            const auto x = __builtin_amdgcn_raw_buffer_load_b64(rb, b_group + t * b_step, 0, kAux);
-            b[t] = make_float2(__int_as_float(x[0]), __int_as_float(x[1]));
+        for (int t = 0; t < 4; ++t)
+            load_b_step(t, g);
+    };
+    auto multiply_step = [&](int t) {
+#pragma unroll
+        for (int hb = 0; hb < HB; ++hb) {
+            acc_e[hb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t][hb], b[t].x, acc_e[hb], 0, 0, 0);
+            acc_o[hb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t][hb], b[t].y, acc_o[hb], 0, 0, 0);
         }
     };
     // Software pipeline of depth one: while a group is multiplied the next group's operands and
@@ -171,11 +198,7 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
     for (int i = 0; i < cnt; ++i) {
 #pragma unroll
         for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int hb = 0; hb < HB; ++hb) {
-                acc_e[hb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t][hb], b[t].x, acc_e[hb], 0, 0, 0);
-                acc_o[hb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t][hb], b[t].y, acc_o[hb], 0, 0, 0);
-            }
+            multiply_step(t);
         if (i + 1 < cnt) {
             load_operands(group_of(x_next), rows_next);
             x_next = after(x_next);
@@ -183,30 +206,52 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
         }
     }
 
-    // the waves' tiles are added in wave order.  Value x of a lane: register x % 4 of the even
-    // (x % 8 < 4) or odd columns of half x / 8; register r of lane (kq, jl) is tile row 4 kq + r
-#pragma unroll
-    for (int hb = 0; hb < HB; ++hb)
-#pragma unroll
-        for (int x = 0; x < 4; ++x) {
-            red[wave][8 * hb + x][lane] = acc_e[hb][x];
-            red[wave][8 * hb + 4 + x][lane] = acc_o[hb][x];
+    // The waves' tiles are added in wave order, HBC halves per pass through LDS.  Value x of a lane:
+    // register x % 4 of the even (x % 8 < 4) or odd columns of half x / 8; register r of lane
+    // (kq, jl) is tile row 4 kq + r.
+    auto row_of = [&](int x) {
+        const int tile_row = 4 * kq + (x % 4), hb = x / 8;
+        return WIDE ? 16 * HBW * (hb / HBW) + HBW * tile_row + hb % HBW : 16 * hb + tile_row;
+    };
+    auto store_c = [&](int x, float s) {
+        const int row = row_of(x);
+        if (row < M) {
+            float* const dst = p.C + (size_t)row * N + (size_t)v * 32 + 2 * jl + (x % 8) / 4;
+            *dst = p.accumulate ? *dst + s : s;
         }
-    __syncthreads();
-    if constexpr (SPLIT) {
-        // Partial tile to scratch with device-scope stores (they reach the point where the other
-        // dies see them), wait for their acknowledgement, take a ticket.  No workgroup ever waits for
-        // another: whoever draws the last ticket of its vector finds all partial tiles complete.
-        constexpr int kTile = 8 * HB * 64;
-        __shared__ unsigned int ticket;
-        float* const mine = p.part + ((size_t)v * p.slices + slice) * kTile;
-        for (int x = wave; x < 8 * HB; x += kDecodeWaves) {
-            float s = red[0][x][lane];
+    };
+    constexpr int kTile = 8 * HB * 64;
+    float* const mine = SPLIT ? p.part + ((size_t)v * p.slices + slice) * kTile : nullptr;
+#pragma unroll
+    for (int pass = 0; pass < HB / HBC; ++pass) {
+        if (pass > 0)
+            __syncthreads();  // the previous pass has been read
+#pragma unroll
+        for (int hh = 0; hh < HBC; ++hh)
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                red[wave][8 * hh + x][lane] = acc_e[pass * HBC + hh][x];
+                red[wave][8 * hh + 4 + x][lane] = acc_o[pass * HBC + hh][x];
+            }
+        __syncthreads();
+        for (int xl = wave; xl < 8 * HBC; xl += kDecodeWaves) {
+            float s = red[0][xl][lane];
 #pragma unroll
             for (int y = 1; y < kDecodeWaves; ++y)
-                s += red[y][x][lane];
-            __hip_atomic_store(&mine[x * 64 + lane], s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                s += red[y][xl][lane];
+            const int x = pass * 8 * HBC + xl;
+            if constexpr (SPLIT)
+                // partial tile to scratch with device-scope stores (they reach the point where the
+                // other dies see them)
+                __hip_atomic_store(&mine[x * 64 + lane], s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else
+                store_c(x, s);
         }
+    }
+    if constexpr (SPLIT) {
+        // Wait for the stores' acknowledgement, take a ticket.  No workgroup ever waits for another:
+        // whoever draws the last ticket of its vector finds all partial tiles complete.
+        __shared__ unsigned int ticket;
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (tid == 0)
@@ -219,36 +264,21 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
             for (int z = 0; z < p.slices; ++z)
                 s += __hip_atomic_load(&p.part[((size_t)v * p.slices + z) * kTile + x * 64 + lane], __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
-            const int tile_row = 4 * kq + (x % 4);
-            const int row = PAIRS ? 2 * tile_row + x / 8 : 16 * (x / 8) + tile_row;
-            if (row < M) {
-                float* const dst = p.C + (size_t)row * N + (size_t)v * 32 + 2 * jl + (x % 8) / 4;
-                *dst = p.accumulate ? *dst + s : s;
-            }
+            store_c(x, s);
         }
         if (tid == 0)
             __hip_atomic_store(&p.tickets[v], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
-        return;
-    }
-    for (int x = wave; x < 8 * HB; x += kDecodeWaves) {
-        float s = red[0][x][lane];
-#pragma unroll
-        for (int y = 1; y < kDecodeWaves; ++y)
-            s += red[y][x][lane];
-        const int tile_row = 4 * kq + (x % 4);
-        const int row = PAIRS ? 2 * tile_row + x / 8 : 16 * (x / 8) + tile_row;
-        if (row < M) {
-            float* const dst = p.C + (size_t)row * N + (size_t)v * 32 + 2 * jl + (x % 8) / 4;
-            *dst = p.accumulate ? *dst + s : s;
-        }
     }
 }
 
 bool decode_supported(const SpmmArgs& a)
 {
-    if (a.row_index == nullptr || a.M > 32 || a.vec_len != 32)
+    // up to 32 rows either layout of A; 33 to 64 rows only column-major (wide loads of A)
+    if (a.row_index == nullptr || a.M > 64 || a.vec_len != 32)
         return false;
     if (a.a_rowmajor) {
+        if (a.M > 32)
+            return false;
         if (a.lda < a.K || (size_t)a.M * a.lda * sizeof(float) >= 0x80000000ull)
             return false;
     } else {
@@ -282,7 +312,7 @@ hipError_t launch_decode(const SpmmArgs& a)
     const int vectors = a.N / 32;
     const int cus = machine().cus;
     const bool pairs = a.M > 16 && !a.a_rowmajor && a.lda % 2 == 0 && a.M % 2 == 0;
-    const dim3 block16(64 * 16), block8(64 * 8);
+    const int halves = a.M <= 16 ? 1 : a.M <= 32 ? 2 : 4;  // 16-row halves per wave
 
     // Fewer vectors than compute units: with scratch from the caller's flag, cut each reduction
     // across as many workgroups as fill the GPU once, as long as every wave of a slice keeps at
@@ -296,7 +326,7 @@ hipError_t launch_decode(const SpmmArgs& a)
             s = p.G / 64;
         if (s > 8)
             s = 8;
-        const size_t tile_bytes = (size_t)(a.M <= 16 ? 8 : 16) * 64 * sizeof(float);
+        const size_t tile_bytes = (size_t)8 * halves * 64 * sizeof(float);
         if (s >= 2 && vectors <= a.decode_ticket_count && (size_t)vectors * s * tile_bytes <= a.decode_part_bytes)
             slices = s;
     }
@@ -304,49 +334,44 @@ hipError_t launch_decode(const SpmmArgs& a)
     p.tickets = a.decode_tickets;
     p.slices = slices;
     p.vectors = vectors;
+    const bool nt = a.stream_b;
+#define NMSPMM_DECODE_LAUNCH(HB, WIDE, WAVES, SPLIT, GRID)                                                  \
+    do {                                                                                                    \
+        if (nt)                                                                                             \
+            spmm_decode_kernel<HB, WIDE, true, WAVES, SPLIT><<<GRID, dim3(64 * WAVES), 0, a.stream>>>(p);   \
+        else                                                                                                \
+            spmm_decode_kernel<HB, WIDE, false, WAVES, SPLIT><<<GRID, dim3(64 * WAVES), 0, a.stream>>>(p);  \
+    } while (0)
     if (slices > 1) {
         const dim3 grid((unsigned)(vectors * slices));
-        if (a.M <= 16) {
-            if (a.stream_b)
-                spmm_decode_kernel<1, false, true, 16, true><<<grid, block16, 0, a.stream>>>(p);
-            else
-                spmm_decode_kernel<1, false, false, 16, true><<<grid, block16, 0, a.stream>>>(p);
-        } else if (pairs) {
-            if (a.stream_b)
-                spmm_decode_kernel<2, true, true, 16, true><<<grid, block16, 0, a.stream>>>(p);
-            else
-                spmm_decode_kernel<2, true, false, 16, true><<<grid, block16, 0, a.stream>>>(p);
-        } else {
-            if (a.stream_b)
-                spmm_decode_kernel<2, false, true, 16, true><<<grid, block16, 0, a.stream>>>(p);
-            else
-                spmm_decode_kernel<2, false, false, 16, true><<<grid, block16, 0, a.stream>>>(p);
-        }
+        if (halves == 1)
+            NMSPMM_DECODE_LAUNCH(1, false, 16, true, grid);
+        else if (halves == 2 && pairs)
+            NMSPMM_DECODE_LAUNCH(2, true, 16, true, grid);
+        else if (halves == 2)
+            NMSPMM_DECODE_LAUNCH(2, false, 16, true, grid);
+        else
+            NMSPMM_DECODE_LAUNCH(4, true, 16, true, grid);
         return hipGetLastError();
     }
 
     const dim3 grid((unsigned)vectors);
-    if (a.M <= 16) {
-        if (a.stream_b) {
-            spmm_decode_kernel<1, false, true, 16><<<grid, block16, 0, a.stream>>>(p);
-        } else if (a.W >= 2048 && a.M >= 8 && vectors >= cus) {
+    if (halves == 1) {
+        if (!nt && a.W >= 2048 && a.M >= 8 && vectors >= cus) {
             // (with fewer workgroups than compute units 8 waves per CU are too few: 16 then)
             p.rotate = 5;
-            spmm_decode_kernel<1, false, false, 8><<<grid, block8, 0, a.stream>>>(p);
+            spmm_decode_kernel<1, false, false, 8><<<grid, dim3(64 * 8), 0, a.stream>>>(p);
         } else {
-            spmm_decode_kernel<1, false, false, 16><<<grid, block16, 0, a.stream>>>(p);
+            NMSPMM_DECODE_LAUNCH(1, false, 16, false, grid);
         }
-    } else if (pairs) {
-        if (a.stream_b)
-            spmm_decode_kernel<2, true, true, 16><<<grid, block16, 0, a.stream>>>(p);
-        else
-            spmm_decode_kernel<2, true, false, 16><<<grid, block16, 0, a.stream>>>(p);
+    } else if (halves == 2 && pairs) {
+        NMSPMM_DECODE_LAUNCH(2, true, 16, false, grid);
+    } else if (halves == 2) {
+        NMSPMM_DECODE_LAUNCH(2, false, 16, false, grid);
     } else {
-        if (a.stream_b)
-            spmm_decode_kernel<2, false, true, 16><<<grid, block16, 0, a.stream>>>(p);
-        else
-            spmm_decode_kernel<2, false, false, 16><<<grid, block16, 0, a.stream>>>(p);
+        NMSPMM_DECODE_LAUNCH(4, true, 16, false, grid);
     }
+#undef NMSPMM_DECODE_LAUNCH
     return hipGetLastError();
 }
 

@@ -34,7 +34,7 @@ class NMSparseLinear(torch.nn.Module):
     out_features % 32 == 0.  Leading dimensions of x are flattened into rows; any row count runs on
     the matrix-core kernels (the copy of x the row-major entry point makes is padded to a row pitch
     of a multiple of four floats).  single_stream=True promises that all forwards of such modules
-    are issued on one stream at a time; up to 32 rows they may then use more of the GPU when
+    are issued on one stream at a time; up to 64 rows they may then use more of the GPU when
     out_features is small (fewer than 256 groups of 32).
     """
 
@@ -65,7 +65,7 @@ class NMSparseLinear(torch.nn.Module):
                                 device=weight.device)
         got = _nm.preprocess_device(DT, n, m, self.W, self.Q, N, self.Ns, D, cinfo)
         assert got == (self.window, self.kept)
-        # the row list: the index form the decode kernel (up to 32 rows) reads
+        # the row list: the index form the decode kernel (up to 64 rows) reads
         rows = torch.empty(_nm.row_index_ints(self.W, N), dtype=torch.int32, device=weight.device)
         _nm.row_index_device(D, cinfo, self.W, N, self.window, self.kept, self.Ns, rows)
         self.register_buffer("values", BT)

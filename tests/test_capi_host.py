@@ -222,3 +222,36 @@ def test_split_rule_matches_reference_partition():
     begins = [z * (p + 1) if z < q else z * p + q for z in range(8)]
     assert counts == [3, 3, 3, 3, 2, 2, 2, 2]
     assert begins == list(np.cumsum([0] + counts[:-1]))
+
+
+def test_python_wrappers_refuse_tensors_smaller_than_the_shape_arguments():
+    """The C interface sees plain pointers; the Python mirror knows the tensors and raises before a
+    kernel could read or write beyond one (nothing here reaches the GPU: CPU tensors, the check
+    comes first)."""
+    import torch
+    M, N, K, W = 64, 128, 128, 64            # 2:4 on the (32, 16) geometry
+    f = lambda n: torch.zeros(n, dtype=torch.float32)
+    i = lambda n: torch.zeros(n, dtype=torch.int32)
+    good = dict(A=f(K * M), B=f(W * N), D=i(W * N // 32), C=f(M * N))
+    for short in ("A", "B", "D", "C"):
+        t = dict(good)
+        t[short] = t[short][:-1]
+        with pytest.raises(ValueError, match=short):
+            nmspmm.spmm(t["A"], t["B"], t["D"], None, t["C"], M, N, K, W, 32, 16)
+        with pytest.raises(ValueError, match=short):
+            nmspmm.spmm_ex(t["A"], t["B"], t["D"], None, t["C"], M, N, K, W, 32, 16)
+    # A for 32 rows passed as 64: the mistake that reads K * 32 floats beyond the tensor
+    with pytest.raises(ValueError, match="A holds"):
+        nmspmm.spmm_ex(f(K * 32), good["B"], good["D"], None, good["C"], M, N, K, W, 32, 16)
+    with pytest.raises(ValueError, match="row_index"):
+        nmspmm.spmm_ex(good["A"], good["B"], good["D"], None, good["C"], M, N, K, W, 32, 16,
+                       row_index=i(nmspmm.row_index_ints(W, N) - 1))
+    with pytest.raises(ValueError, match="column_info"):   # 2:8 on the (64, 16) geometry, K = 256
+        nmspmm.spmm(f(256 * M), good["B"], good["D"], i(nmspmm.column_info_ints(W, 16, 64, N, 128) - 1), good["C"],
+                    M, N, 256, W, 64, 16)
+    with pytest.raises(ValueError, match="dBT"):
+        nmspmm.compress_device(f(K * N), K, N, 2, 4, f(W * N - 1), i(W * N // 32))
+    with pytest.raises(ValueError, match="dDT_out"):
+        nmspmm.preprocess_low_device(i(W * 4), i(W * 4 - 1), W, 4, 128)
+    with pytest.raises(ValueError, match="dst"):
+        nmspmm.transpose_device(f(M * K), M, K, f(M * K - 1))

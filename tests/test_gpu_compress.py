@@ -116,8 +116,9 @@ def test_compress_preprocess_multiply_chain(n, m):
 
 def test_bad_arguments_are_rejected():
     x = torch.zeros((64, 64), dtype=torch.float32, device="cuda")
-    bt = torch.zeros((32, 64), dtype=torch.float32, device="cuda")
-    dt = torch.zeros((32, 2), dtype=torch.int32, device="cuda")
+    # buffers large enough for every case, so that the library's own checks are what refuses them
+    bt = torch.zeros((64, 64), dtype=torch.float32, device="cuda")
+    dt = torch.zeros((64, 64), dtype=torch.int32, device="cuda")
     for (K, N, n, m, vl) in ((64, 64, 4, 4, 32), (64, 64, 0, 4, 32), (64, 64, 2, 5, 32), (64, 64, 2, 4, 3), (63, 64, 2, 4, 32),
                              (64, 48, 2, 4, 32)):
         with pytest.raises(nmspmm.NmSpmmError):

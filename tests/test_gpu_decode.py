@@ -61,20 +61,20 @@ def test_row_list_bit_exact_at_full_size(oracle, N, K, n, m):
     assert np.array_equal(got, oracle.row_index(D, cinfo, d["W"], N, window, kept, 128))
 
 
-@pytest.mark.parametrize("M", [1, 2, 7, 8, 13, 16, 17, 24, 31, 32])
+@pytest.mark.parametrize("M", [1, 2, 7, 8, 13, 16, 17, 24, 31, 32, 33, 34, 39, 48, 57, 62, 63, 64])
 @pytest.mark.parametrize("n,m,K", [(1, 8, 1024), (2, 8, 1088), (2, 4, 1152), (3, 8, 96), (3, 8, 1120), (32, 32, 160), (4, 32, 960)])
 def test_decode_kernel_every_row_count(oracle, M, n, m, K):
-    """Row counts on both sides of 16 and 32, odd ones included (17 to 32 rows take one 64-bit
-    load of A per k-step when the row count is even, two 32-bit loads when it is odd); reductions
-    that give the 16 waves of a workgroup unequal shares, some none, and (3:8 with K = 96: 36 kept
-    rows) a last group of four rows."""
+    """Row counts on both sides of 16, 32 and 64, odd ones included (17 to 32 rows take one 64-bit
+    load of A per k-step when the row count is even, two 32-bit loads when it is odd, 33 to 64 rows
+    one 128-bit load whatever the count); reductions that give the 16 waves of a workgroup unequal
+    shares, some none, and (3:8 with K = 96: 36 kept rows) a last group of four rows."""
     d = datagen.init_data(M, 256, K, n, m, seed=M + K, dist="normal", b_scale=0.02)
     got, fam = run_decode(oracle, d)
     assert fam == "decode"
     assert np.isfinite(got).all() and scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
 
 
-@pytest.mark.parametrize("M", [1, 3, 9, 16, 19, 26])
+@pytest.mark.parametrize("M", [1, 3, 9, 16, 19, 26, 33, 41, 50, 61])
 @pytest.mark.parametrize("n,m,K", [(2, 8, 1088), (3, 8, 96), (1, 8, 2048)])
 def test_nothing_outside_a_leaks_into_c(oracle, M, n, m, K):
     """The lanes of a 16-row tile whose row of C does not exist read the last row that does, and
@@ -143,11 +143,24 @@ def test_decode_kernel_adds_to_c_when_asked_like_a_split_call_of_the_reference(o
     assert scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
 
 
-def test_larger_row_counts_ignore_the_list(oracle):
-    d = datagen.init_data(48, 256, 512, 2, 8, seed=3)
+@pytest.mark.parametrize("M", [65, 100, 128, 200])
+def test_larger_row_counts_ignore_the_list(oracle, M):
+    d = datagen.init_data(M, 256, 512, 2, 8, seed=3)
     got, fam = run_decode(oracle, d)
     assert fam in ("skinny", "mfma")
     assert scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
+
+
+@pytest.mark.parametrize("M", [48, 64])
+@pytest.mark.parametrize("n,m", [(1, 8), (2, 8)])
+def test_33_to_64_rows_at_full_size_on_the_row_list(oracle, M, n, m):
+    """K = Ncols = 8192, all of C against the checker, with and without the non-temporal hint."""
+    d = datagen.init_data(M, 8192, 8192, n, m, seed=150 + M + n, dist="normal", b_scale=0.02)
+    got, fam = run_decode(oracle, d)
+    assert fam == "decode"
+    assert np.isfinite(got).all() and scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
+    streamed, fam = run_decode(oracle, d, flags=nmspmm.STREAM_B)
+    assert fam == "decode" and scaled_max_error(streamed, want_c(oracle, d)) <= REL_TOL
 
 
 def test_a_list_off_a_sixteen_byte_boundary_is_rejected(oracle):
@@ -221,7 +234,7 @@ def test_row_major_activations_on_the_row_list(oracle, M, n, m):
     assert np.isfinite(got).all() and scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
 
 
-@pytest.mark.parametrize("M", [1, 7, 16, 19, 32])
+@pytest.mark.parametrize("M", [1, 7, 16, 19, 32, 45, 64])
 @pytest.mark.parametrize("n,m,K,N", [(2, 8, 11008, 4096), (2, 8, 8192, 2048), (1, 8, 16384, 1024), (2, 4, 4096, 4096), (2, 4, 16384, 1024), (3, 8, 8192, 2048)])
 def test_reductions_cut_across_workgroups(oracle, M, n, m, K, N):
     """NMSPMM_DECODE_SPLIT with fewer column vectors than compute units and a long reduction: two to
