@@ -305,8 +305,11 @@ def run_decode(torch, pkg, rows_list=(1, 8, 16, 32), shapes=((8192, 8192), (4096
                                                NS, 1, None, flags, op.R if rl else None)
 
                 alg = op.algorithmic_bytes()
+                # the launch can be no shorter than its bytes at the HBM rate or its flops at the
+                # fp32 matrix-core peak, whichever is longer (the latter from about 48 rows on)
+                floor_us = max(alg / (HBM_PEAK_GBS * 1e3), 2.0 * m_rows * n_cols * op.W / (FP32_MFMA_PEAK_TFLOPS * 1e6))
                 entry = {"M": m_rows, "K": k, "Ncols": n_cols, "pattern": "%d:%d" % (n, m),
-                         "algorithmic_bytes": int(alg)}
+                         "algorithmic_bytes": int(alg), "roofline_us": round(floor_us, 2)}
                 for label, flags, rl, cold in DECODE_MODES:
                     if label not in modes:
                         continue
