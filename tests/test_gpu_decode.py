@@ -182,7 +182,7 @@ def test_decode_kernel_with_131072_column_vectors(oracle):
     assert scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
 
 
-@pytest.mark.parametrize("M,n,m", [(8, 1, 8), (32, 2, 8)])
+@pytest.mark.parametrize("M,n,m", [(8, 1, 8), (32, 2, 8), (50, 2, 8), (64, 1, 8)])
 def test_graph_replays_of_the_decode_kernel_equal_eager_calls(oracle, M, n, m):
     N, K = 512, 1024
     d = datagen.init_data(M, N, K, n, m, seed=M, dist="normal", b_scale=0.02)
@@ -210,6 +210,7 @@ def test_graph_replays_of_the_decode_kernel_equal_eager_calls(oracle, M, n, m):
         graph.replay()
         call(C_e)
         torch.cuda.synchronize()
+        assert nmspmm.last_kernel() == "decode"
         assert torch.isfinite(C_g).all().item() and torch.equal(C_g, C_e), "replay %d" % rep
 
 
