@@ -65,14 +65,15 @@ __device__ inline __amdgpu_buffer_rsrc_t dc_rsrc(const void* base, uint32_t byte
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }
 
-// HB: 16-row halves (1: M <= 16, 2: M <= 32, 4: M <= 64).  WIDE (column-major A): one
-// load fetches the rows of several halves at once, instead of one 32-bit load per half: HB = 2 a
-// 64-bit load of rows 2 jl, 2 jl + 1; HB = 4 a 128-bit load of rows 4 jl .. 4 jl + 3 (half hb is then
-// the rows HB t + hb, t the tile row; written for any multiple of four halves, two such loads 64 rows
-// apart for eight, which was measured and dropped: at 128 rows and K = Ncols = 8192, 38.9 us on 16
-// waves and 41 us on 8 against the tile kernel's 36 at 2:8, 22.8 against 24.3 us at 1:8).  NT: B is loaded with the non-temporal hint (it is not kept in the caches).
-// SPLIT: the reduction of a vector is cut across p.slices workgroups (fewer vectors than compute
-// units would otherwise leave compute units idle).
+// HB: 16-row halves (1: M <= 16, 2: M <= 32, 4: M <= 64).  WIDE (column-major A): one load fetches
+// the rows of several halves at once, instead of one 32-bit load per half: HB = 2 a 64-bit load of
+// rows 2 jl, 2 jl + 1; HB = 4 a 128-bit load of rows 4 jl .. 4 jl + 3 (half hb is then the rows
+// HB t + hb, t the tile row).  The code is written for any multiple of four halves (two such loads
+// 64 rows apart for eight), but eight halves were measured and dropped: at 128 rows and
+// K = Ncols = 8192, 38.9 us on 16 waves and 41 us on 8 against the tile kernel's 36 at 2:8, 22.8
+// against 24.3 us at 1:8.  NT: B is loaded with the non-temporal hint (it is not kept in the
+// caches).  SPLIT: the reduction of a vector is cut across p.slices workgroups (fewer vectors than
+// compute units would otherwise leave compute units idle).
 template <int HB, bool WIDE, bool NT, int kDecodeWaves, bool SPLIT = false>
 __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const DecodeParams p)
 {
