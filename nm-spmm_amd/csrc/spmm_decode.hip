@@ -74,7 +74,7 @@ __device__ inline __amdgpu_buffer_rsrc_t dc_rsrc(const void* base, uint32_t byte
 // against 24.3 us at 1:8.  NT: B is loaded with the non-temporal hint (it is not kept in the
 // caches).  SPLIT: the reduction of a vector is cut across p.slices workgroups (fewer vectors than
 // compute units would otherwise leave compute units idle).
-template <int HB, bool WIDE, bool NT, int kDecodeWaves, bool SPLIT = false>
+template <int HB, bool WIDE, bool NT, int kDecodeWaves, bool SPLIT = false, int RING = 0>
 __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const DecodeParams p)
 {
     constexpr int HBW = HB < 4 ? HB : 4;   // halves that one wide load serves
@@ -144,67 +144,86 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
     const int first = cnt > 0 ? (int)((blockIdx.x / (unsigned)p.xcds) * (unsigned)p.rotate % (unsigned)cnt) : 0;
     auto after = [&](int x) { return x + 1 >= cnt ? 0 : x + 1; };
     auto group_of = [&](int x) { return g_first + wave + x * kDecodeWaves; };
-    float2 b[4];
-    float a[4][HB];
-    auto load_a_step = [&](int t, const dintx4& rows) {
+    auto load_a_step = [&](int row, float (&dst)[HB]) {
         if constexpr (WIDE && HBW == 2) {
-            const auto x = __builtin_amdgcn_raw_buffer_load_b64(ra, a_offset(a_lane[0], rows[t]), 0, 0);
-            a[t][0] = __int_as_float(x[0]);
-            a[t][1] = __int_as_float(x[1]);
+            const auto x = __builtin_amdgcn_raw_buffer_load_b64(ra, a_offset(a_lane[0], row), 0, 0);
+            dst[0] = __int_as_float(x[0]);
+            dst[1] = __int_as_float(x[1]);
         } else if constexpr (WIDE) {
 #pragma unroll
             for (int w = 0; w < NW; ++w) {
-                const auto x = __builtin_amdgcn_raw_buffer_load_b128(ra, a_offset(a_lane[w], rows[t]), 0, 0);
+                const auto x = __builtin_amdgcn_raw_buffer_load_b128(ra, a_offset(a_lane[w], row), 0, 0);
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    a[t][4 * w + e] = __int_as_float(x[e]);
+                    dst[4 * w + e] = __int_as_float(x[e]);
             }
         } else {
 #pragma unroll
             for (int hb = 0; hb < HB; ++hb)
-                a[t][hb] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(ra, a_offset(a_lane[hb], rows[t]), 0, 0));
+                dst[hb] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(ra, a_offset(a_lane[hb], row), 0, 0));
         }
     };
-    auto load_b_step = [&](int t, int g) {
+    auto load_b_step = [&](int t, int g, float2& dst) {
         // rows at or beyond W (the tail of the last group) lie beyond the descriptor: 0
         const auto x = __builtin_amdgcn_raw_buffer_load_b64(rb, b_lane + (uint32_t)g * 4u * b_step + t * b_step, 0, kAux);
-        b[t] = make_float2(__int_as_float(x[0]), __int_as_float(x[1]));
+        dst = make_float2(__int_as_float(x[0]), __int_as_float(x[1]));
     };
     // A first: its addresses come from the row list, which has landed; the four loads of B follow
     // (measured against B first: 1 to 2 % faster)
-    auto load_operands = [&](int g, const dintx4& rows) {
+    auto load_operands = [&](int g, const dintx4& rows, float (&av)[4][HB], float2 (&bv)[4]) {
 #pragma unroll
         for (int t = 0; t < 4; ++t)
-            load_a_step(t, rows);
+            load_a_step(rows[t], av[t]);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < 4; ++t)
-            load_b_step(t, g);
+            load_b_step(t, g, bv[t]);
     };
-    auto multiply_step = [&](int t) {
-#pragma unroll
-        for (int hb = 0; hb < HB; ++hb) {
-            acc_e[hb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t][hb], b[t].x, acc_e[hb], 0, 0, 0);
-            acc_o[hb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t][hb], b[t].y, acc_o[hb], 0, 0, 0);
-        }
-    };
-    // Software pipeline of depth one: while a group is multiplied the next group's operands and
-    // the rows of the group after it are in flight.
-    dintx4 rows_next;
-    int x_next = after(first);  // position whose rows are in rows_next
-    if (cnt > 0) {
-        const dintx4 rows = load_rows(group_of(first));
-        rows_next = load_rows(group_of(x_next));
-        load_operands(group_of(first), rows);
-    }
-    for (int i = 0; i < cnt; ++i) {
+    auto multiply_group = [&](const float (&av)[4][HB], const float2 (&bv)[4]) {
 #pragma unroll
         for (int t = 0; t < 4; ++t)
-            multiply_step(t);
-        if (i + 1 < cnt) {
-            load_operands(group_of(x_next), rows_next);
-            x_next = after(x_next);
-            rows_next = load_rows(group_of(x_next));  // after the last group: a group that is not used
+#pragma unroll
+            for (int hb = 0; hb < HB; ++hb) {
+                acc_e[hb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[t][hb], bv[t].x, acc_e[hb], 0, 0, 0);
+                acc_o[hb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[t][hb], bv[t].y, acc_o[hb], 0, 0, 0);
+            }
+    };
+    if constexpr (RING > 0) {
+        // Short reductions (every wave has exactly RING groups): the launch lasts a few trips to
+        // memory, so all of a wave's groups are requested at once - one trip for the lists, one for
+        // the operands - instead of one trip per group.  Straight-line code: with wave-uniform
+        // branches around the groups a wave does not have it was slower than the loop.
+        dintx4 rows[RING];
+        float av[RING][4][HB];
+        float2 bv[RING][4];
+#pragma unroll
+        for (int r = 0; r < RING; ++r)
+            rows[r] = load_rows(group_of(r));
+#pragma unroll
+        for (int r = 0; r < RING; ++r)
+            load_operands(group_of(r), rows[r], av[r], bv[r]);
+#pragma unroll
+        for (int r = 0; r < RING; ++r)
+            multiply_group(av[r], bv[r]);
+    } else {
+        // Software pipeline of depth one: while a group is multiplied the next group's operands and
+        // the rows of the group after it are in flight.
+        float2 b[4];
+        float a[4][HB];
+        dintx4 rows_next;
+        int x_next = after(first);  // position whose rows are in rows_next
+        if (cnt > 0) {
+            const dintx4 rows = load_rows(group_of(first));
+            rows_next = load_rows(group_of(x_next));
+            load_operands(group_of(first), rows, a, b);
+        }
+        for (int i = 0; i < cnt; ++i) {
+            multiply_group(a, b);
+            if (i + 1 < cnt) {
+                load_operands(group_of(x_next), rows_next, a, b);
+                x_next = after(x_next);
+                rows_next = load_rows(group_of(x_next));  // after the last group: a group that is not used
+            }
         }
     }
 
@@ -288,7 +307,9 @@ bool decode_supported(const SpmmArgs& a)
             return false;
     }
     // 32-bit offsets into B from a vector's first column, and into a vector's part of the list
-    if ((size_t)a.W * a.N * sizeof(float) >= 0xffffffffull || (size_t)a.W * 4 + 64 >= 0xffffffffull)
+    // (the last group's rows beyond W, and a group beyond the list, must stay beyond B's descriptor
+    // without wrapping: 16 rows more)
+    if (((size_t)a.W + 32) * a.N * sizeof(float) >= 0xffffffffull || (size_t)a.W * 4 + 64 >= 0xffffffffull)
         return false;
     return true;
 }
@@ -358,6 +379,37 @@ hipError_t launch_decode(const SpmmArgs& a)
     }
 
     const dim3 grid((unsigned)vectors);
+    // Short reductions, the same two to four groups for every wave (K = 4096 at 2:8 and 1:8): every
+    // group of a wave is requested at once.  Measured at K = 4096 on 14336 columns, 1 / 8 / 16 rows:
+    // 1:8 (two groups per wave) 6.2 / 6.8 / 7.0 -> 5.2 / 5.7 / 5.9 us, 2:8 (four) 11.4 / 12.4 / 12.5 ->
+    // 11.1 / 11.8 / 12.0 us; 17 to 32 rows gain at two groups per wave (9.3 -> 8.2 us) and nothing at four.
+    if (p.G % 16 == 0 && p.G >= 32 && p.G <= (halves == 1 ? 64 : halves == 2 ? 32 : 0)) {
+#define NMSPMM_DECODE_RING(HB, WIDE, RING)                                                                   \
+    do {                                                                                                      \
+        if (nt)                                                                                               \
+            spmm_decode_kernel<HB, WIDE, true, 16, false, RING><<<grid, dim3(64 * 16), 0, a.stream>>>(p);      \
+        else                                                                                                  \
+            spmm_decode_kernel<HB, WIDE, false, 16, false, RING><<<grid, dim3(64 * 16), 0, a.stream>>>(p);     \
+    } while (0)
+#define NMSPMM_DECODE_RINGS(HB, WIDE)                                                                        \
+    do {                                                                                                      \
+        if (p.G == 32)                                                                                        \
+            NMSPMM_DECODE_RING(HB, WIDE, 2);                                                                  \
+        else if (p.G == 48)                                                                                   \
+            NMSPMM_DECODE_RING(HB, WIDE, 3);                                                                  \
+        else                                                                                                  \
+            NMSPMM_DECODE_RING(HB, WIDE, 4);                                                                  \
+    } while (0)
+        if (halves == 1)
+            NMSPMM_DECODE_RINGS(1, false);
+        else if (pairs)
+            NMSPMM_DECODE_RING(2, true, 2);
+        else
+            NMSPMM_DECODE_RING(2, false, 2);
+#undef NMSPMM_DECODE_RINGS
+#undef NMSPMM_DECODE_RING
+        return hipGetLastError();
+    }
     if (halves == 1) {
         if (!nt && a.W >= 2048 && a.M >= 8 && vectors >= cus) {
             // (with fewer workgroups than compute units 8 waves per CU are too few: 16 then)
