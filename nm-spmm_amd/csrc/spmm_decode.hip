@@ -58,6 +58,9 @@ struct DecodeParams {
     float* part;
     unsigned int* tickets;
     int slices, vectors;
+    // rows cut across workgroups: the launch has `vectors` = Ncols / 32 x `parts` workgroups (per
+    // slice), workgroup (v, q) computes rows [q * part_rows, min(M, (q + 1) * part_rows)) of vector v
+    int parts, part_rows, real_vectors;
 };
 
 __device__ inline __amdgpu_buffer_rsrc_t dc_rsrc(const void* base, uint32_t bytes)
@@ -85,15 +88,30 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kq = lane >> 4, jl = lane & 15;
-    const int v = SPLIT ? (int)(blockIdx.x % (unsigned)p.vectors) : (int)blockIdx.x;
+    // vv: (vector, row part).  The parts of a vector get ids that differ by the number of XCDs, so
+    // that they run on the same XCD at about the same time and share its L2's copy of B.
+    const int vv = SPLIT ? (int)(blockIdx.x % (unsigned)p.vectors) : (int)blockIdx.x;
     const int slice = SPLIT ? (int)(blockIdx.x / (unsigned)p.vectors) : 0;
-    const int M = p.M, N = p.N;
+    int v = vv, part = 0;
+    if (p.parts > 1) {
+        if (p.real_vectors % p.xcds == 0) {
+            const int slot = vv / p.xcds;
+            part = slot % p.parts;
+            v = (slot / p.parts) * p.xcds + vv % p.xcds;
+        } else {
+            part = vv % p.parts;
+            v = vv / p.parts;
+        }
+    }
+    const int m0 = part * p.part_rows;
+    const int M = min(p.M - m0, p.part_rows), N = p.N;
 
     // every offset that relies on the descriptor's range check is a vector offset: the scalar
     // offset of a buffer load is not part of that check
     const __amdgpu_buffer_rsrc_t rb = dc_rsrc(p.B + (size_t)v * 32, p.b_bytes);
     const __amdgpu_buffer_rsrc_t rr = dc_rsrc(p.R + (size_t)v * p.G * 16, (uint32_t)p.G * 64u);
-    const __amdgpu_buffer_rsrc_t ra = dc_rsrc(p.A, p.a_bytes);
+    const __amdgpu_buffer_rsrc_t ra = dc_rsrc(reinterpret_cast<const char*>(p.A) + (size_t)m0 * p.a_row_stride,
+                                              p.a_bytes - (uint32_t)m0 * p.a_row_stride);
     const uint32_t a_stride = p.a_k_stride;
     // Lanes whose row of C does not exist read the last row that does (their tile rows are never
     // stored): out-of-range lanes would be dropped by the descriptor as well, but loads with most
@@ -237,12 +255,12 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
     auto store_c = [&](int x, float s) {
         const int row = row_of(x);
         if (row < M) {
-            float* const dst = p.C + (size_t)row * N + (size_t)v * 32 + 2 * jl + (x % 8) / 4;
+            float* const dst = p.C + (size_t)(m0 + row) * N + (size_t)v * 32 + 2 * jl + (x % 8) / 4;
             *dst = p.accumulate ? *dst + s : s;
         }
     };
     constexpr int kTile = 8 * HB * 64;
-    float* const mine = SPLIT ? p.part + ((size_t)v * p.slices + slice) * kTile : nullptr;
+    float* const mine = SPLIT ? p.part + ((size_t)vv * p.slices + slice) * kTile : nullptr;
 #pragma unroll
     for (int pass = 0; pass < HB / HBC; ++pass) {
         if (pass > 0)
@@ -276,19 +294,19 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (tid == 0)
-            ticket = __hip_atomic_fetch_add(&p.tickets[v], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            ticket = __hip_atomic_fetch_add(&p.tickets[vv], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (ticket != (unsigned int)(p.slices - 1))
             return;
         for (int x = wave; x < 8 * HB; x += kDecodeWaves) {
             float s = 0.0f;
             for (int z = 0; z < p.slices; ++z)
-                s += __hip_atomic_load(&p.part[((size_t)v * p.slices + z) * kTile + x * 64 + lane], __ATOMIC_RELAXED,
+                s += __hip_atomic_load(&p.part[((size_t)vv * p.slices + z) * kTile + x * 64 + lane], __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
             store_c(x, s);
         }
         if (tid == 0)
-            __hip_atomic_store(&p.tickets[v], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+            __hip_atomic_store(&p.tickets[vv], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
     }
 }
 
@@ -332,10 +350,32 @@ hipError_t launch_decode(const SpmmArgs& a)
     p.accumulate = (a.accumulate && a.split_k > 1) ? 1 : 0;
     p.rotate = 0;
     p.xcds = machine().xcds;
-    const int vectors = a.N / 32;
+    const int real_vectors = a.N / 32;
     const int cus = machine().cus;
-    const bool pairs = a.M > 16 && !a.a_rowmajor && a.lda % 2 == 0 && a.M % 2 == 0;
-    const int halves = a.M <= 16 ? 1 : a.M <= 32 ? 2 : 4;  // 16-row halves per wave
+    // More than 16 rows on few vectors: the rows are cut into parts of 16 (or 32) with a workgroup
+    // each, as far as that fills compute units that would idle otherwise.  The parts of a vector read
+    // the same B (the second one from the L2 of their XCD) and disjoint rows of A and C: nothing to
+    // add up, and each CU keeps the request count of the 16-row form.
+    int parts = 1, part_rows = a.M;
+    if (a.M > 16 && real_vectors * 2 <= cus) {
+        part_rows = ((a.M + 15) / 16) * real_vectors <= cus ? 16 : 32;
+        parts = (a.M + part_rows - 1) / part_rows;
+        // Up to 32 rows, where the caller's flag allows cut reductions and there is room for either
+        // two slices or two parts but not both, the slices win (K = 11008 on 4096 columns, 32 rows:
+        // 12.9 us with two slices, 15.9 us with two parts, 17.7 us with neither)
+        const bool scratch = a.decode_part != nullptr && a.decode_tickets != nullptr;
+        if (scratch && a.M <= 32 && cus / real_vectors >= 2 && p.G / 64 >= 2 && cus / (real_vectors * parts) < 2)
+            parts = 1;
+        if (parts == 1)
+            part_rows = a.M;
+    }
+    const int vectors = real_vectors * parts;  // workgroups per slice
+    const int m_wg = parts > 1 ? part_rows : a.M;
+    const bool pairs = m_wg > 16 && !a.a_rowmajor && a.lda % 2 == 0 && a.M % 2 == 0;
+    const int halves = m_wg <= 16 ? 1 : m_wg <= 32 ? 2 : 4;  // 16-row halves per wave
+    p.parts = parts;
+    p.part_rows = part_rows;
+    p.real_vectors = real_vectors;
 
     // Fewer vectors than compute units: with scratch from the caller's flag, cut each reduction
     // across as many workgroups as fill the GPU once, as long as every wave of a slice keeps at
