@@ -632,7 +632,7 @@ def main():
         configs["decode_llm"] = run_decode(torch, pkg, (1, 16, 32), DECODE_LLM_SHAPES, ((2, 8),), DECODE_LLM_MODES)
     if "decode_wide" in parts:
         # beyond the baseline's row counts: 33 to 64 rows on the row list (serving batches)
-        configs["decode_wide"] = run_decode(torch, pkg, (48, 64), ((8192, 8192),), ((1, 8), (2, 8)),
+        configs["decode_wide"] = run_decode(torch, pkg, (48, 64), ((8192, 8192), (4096, 4096)), ((1, 8), (2, 8)),
                                             ("hot", "cold", "hot_reference_layout", "cold_reference_layout"))
     if "fine" in parts:
         configs["fine"] = run_fine(torch, pkg, tuple(
