@@ -352,14 +352,34 @@ inline double model_tile_seconds(int M, int N, int nwin, int kept, int split)
         t += (2.0 * split + 1.0) * c_bytes / 8e12 + 4e-6;
     return t;
 }
-// Whole multiplication on the decode kernel (M <= 128): one workgroup per 32-column vector, 256
-// of them at a time, each needing kept/2 k-steps x (1, 2 or 4) MFMAs per window on the four
-// matrix pipes of its CU (4.2 ns per kept row and 32-row block, measured), plus 5 us.
+// Rows per workgroup of the kernels that take one workgroup per 32-column vector: with at most
+// half as many vectors as compute units, more than 16 rows are cut into parts of 16 rows, or of 32
+// where 16-row parts would be more workgroups than compute units, one workgroup per vector and
+// part.  The parts of a vector read the same B and disjoint rows of A and C, so nothing has to be
+// added up.  Returns M where the rows are not cut.  (Parts of 64 rows for 65 to 128 rows were
+// measured too: 4 to 12 % slower than the tile kernel on 4096 columns.)
+inline int decode_part_rows(int M, int vectors)
+{
+    const long long cus = machine().cus;
+    if (M <= 16 || 2LL * vectors > cus)
+        return M;
+    for (int rows = 16; rows <= 32 && rows < M; rows *= 2)
+        if ((long long)((M + rows - 1) / rows) * vectors <= cus)
+            return rows;
+    return M;
+}
+
+// Whole multiplication on the decode kernel (M <= 128): one workgroup per 32-column vector (and
+// part of the rows), 256 of them at a time, each needing kept/2 k-steps x (1, 2 or 4) MFMAs per
+// window on the four matrix pipes of its CU (4.2 ns per kept row and 32-row block, measured),
+// plus 5 us.
 inline double model_decode_seconds(int M, int N, int nwin, int kept)
 {
-    const int blocks = M <= 32 ? 1 : M <= 64 ? 2 : 4;
+    const int vectors = (N + 31) / 32;
+    const int rows = decode_part_rows(M, vectors);
+    const int blocks = rows <= 32 ? 1 : rows <= 64 ? 2 : 4;
     const long long cus = machine().cus;
-    const long long rounds = ((N + 31) / 32 + cus - 1) / cus;
+    const long long rounds = ((long long)vectors * ((M + rows - 1) / rows) + cus - 1) / cus;
     return 5e-6 + (double)rounds * nwin * kept * blocks * (10.08 / machine().clock);
 }
 

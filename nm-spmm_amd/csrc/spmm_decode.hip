@@ -357,8 +357,8 @@ hipError_t launch_decode(const SpmmArgs& a)
     // the same B (the second one from the L2 of their XCD) and disjoint rows of A and C: nothing to
     // add up, and each CU keeps the request count of the 16-row form.
     int parts = 1, part_rows = a.M;
-    if (a.M > 16 && real_vectors * 2 <= cus) {
-        part_rows = ((a.M + 15) / 16) * real_vectors <= cus ? 16 : 32;
+    if (decode_part_rows(a.M, real_vectors) < a.M) {
+        part_rows = decode_part_rows(a.M, real_vectors);
         parts = (a.M + part_rows - 1) / part_rows;
         // Up to 32 rows, where the caller's flag allows cut reductions and there is room for either
         // two slices or two parts but not both, the slices win (K = 11008 on 4096 columns, 32 rows:

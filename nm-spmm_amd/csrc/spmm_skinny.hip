@@ -35,7 +35,10 @@ struct SkinnyParams {
     // (4, 4 * lda) for the column-major operand, (4 * lda, 4) for a row-major one (up to 32 rows)
     uint32_t a_row_stride, a_k_stride, a_bytes;
     int accumulate;  // the result is added to what C holds instead of replacing it
+    int part_rows;   // workgroup (x, y) computes rows [y * part_rows, min(M, (y + 1) * part_rows)) of vector x
 };
+
+static int skinny_part_rows(const SpmmArgs& a);
 
 __device__ inline __amdgpu_buffer_rsrc_t sk_rsrc(const void* base, uint32_t bytes)
 {
@@ -98,7 +101,8 @@ spmm_skinny_kernel(const SkinnyParams p)
     const int vec_g = blockIdx.x;     // global column vector
     const int jb = vec_g / QS;        // preprocessed column block
     const int vec = vec_g % QS;       // vector inside it
-    const int M = p.M, N = p.N;
+    const int m0 = blockIdx.y * p.part_rows;
+    const int M = min(p.M - m0, p.part_rows), N = p.N;
 
     // windows of this wave: the same partition rule the large-tile kernels use for split-K
     int w_begin, w_count;
@@ -111,7 +115,7 @@ spmm_skinny_kernel(const SkinnyParams p)
     const uint32_t a_bytes = p.a_bytes;
     // lanes beyond the last row read the last fragment that exists (their tile rows are never stored):
     // loads with most lanes out of range are slow
-    const uint32_t a_lane = (uint32_t)min(RB * j, (M - 1) / RB * RB) * p.a_row_stride;
+    const uint32_t a_lane = (uint32_t)(m0 + min(RB * j, (M - 1) / RB * RB)) * p.a_row_stride;
     const uint32_t row_bytes = p.a_k_stride;
     const uint32_t b_lane = (uint32_t)(((size_t)h * N + j) * sizeof(float));
     const uint32_t b_step = (uint32_t)(2 * (size_t)N * sizeof(float));
@@ -233,7 +237,7 @@ spmm_skinny_kernel(const SkinnyParams p)
                 s += red[x][v][lane];
             const int row = RB * (8 * (v / 4) + 4 * h + (v % 4)) + b;
             if (row < M) {
-                float* const dst = p.C + (size_t)row * N + (size_t)vec_g * 32 + j;
+                float* const dst = p.C + (size_t)(m0 + row) * N + (size_t)vec_g * 32 + j;
                 *dst = p.accumulate ? *dst + s : s;
             }
         }
@@ -266,7 +270,8 @@ spmm_skinny16_kernel(const SkinnyParams p)
     const int vec_g = blockIdx.x;
     const int jb = vec_g / QS;
     const int vec = vec_g % QS;
-    const int M = p.M, N = p.N;
+    const int m0 = blockIdx.y * p.part_rows;
+    const int M = min(p.M - m0, p.part_rows), N = p.N;
 
     int w_begin, w_count;
     split_windows(p.nwin, kSkinnyWaves, wave, &w_begin, &w_count);
@@ -278,7 +283,7 @@ spmm_skinny16_kernel(const SkinnyParams p)
     const uint32_t a_bytes = p.a_bytes;
     // lanes beyond the last row read the last row (their tile rows are never stored): loads with most
     // lanes out of range are slow
-    const uint32_t a_lane = (uint32_t)min(jl, M - 1) * p.a_row_stride;
+    const uint32_t a_lane = (uint32_t)(m0 + min(jl, M - 1)) * p.a_row_stride;
     const uint32_t row_bytes = p.a_k_stride;
     const uint32_t b_lane = (uint32_t)(((size_t)kq * N + 2 * jl) * sizeof(float));
     const uint32_t b_step = (uint32_t)(4 * (size_t)N * sizeof(float));
@@ -382,7 +387,7 @@ spmm_skinny16_kernel(const SkinnyParams p)
             s += red[y][x][lane];
         const int row = 4 * kq + (x % 4);
         if (row < M) {
-            float* const dst = p.C + (size_t)row * N + (size_t)vec_g * 32 + 2 * jl + x / 4;
+            float* const dst = p.C + (size_t)(m0 + row) * N + (size_t)vec_g * 32 + 2 * jl + x / 4;
             *dst = p.accumulate ? *dst + s : s;
         }
     }
@@ -407,7 +412,8 @@ static hipError_t launch_qs(const SpmmArgs& a)
     p.a_k_stride = (uint32_t)(a.a_rowmajor ? sizeof(float) : a.lda * sizeof(float));
     p.a_bytes = (uint32_t)((size_t)(a.a_rowmajor ? a.M : a.K) * a.lda * sizeof(float));
     p.accumulate = (a.accumulate && a.split_k > 1) ? 1 : 0;
-    const dim3 grid(a.N / 32), block(64 * kSkinnyWaves);
+    p.part_rows = skinny_part_rows(a);
+    const dim3 grid(a.N / 32, (a.M + p.part_rows - 1) / p.part_rows), block(64 * kSkinnyWaves);
     switch (a.Ns) {
     case 128: spmm_skinny_kernel<KS, WS, 4, HIGH, RB, U><<<grid, block, 0, a.stream>>>(p); break;
     case 64: spmm_skinny_kernel<KS, WS, 2, HIGH, RB, U><<<grid, block, 0, a.stream>>>(p); break;
@@ -436,7 +442,8 @@ static hipError_t launch_qs16(const SpmmArgs& a)
     p.a_k_stride = (uint32_t)(a.a_rowmajor ? sizeof(float) : a.lda * sizeof(float));
     p.a_bytes = (uint32_t)((size_t)(a.a_rowmajor ? a.M : a.K) * a.lda * sizeof(float));
     p.accumulate = (a.accumulate && a.split_k > 1) ? 1 : 0;
-    const dim3 grid(a.N / 32), block(64 * kSkinnyWaves);
+    p.part_rows = skinny_part_rows(a);
+    const dim3 grid(a.N / 32, (a.M + p.part_rows - 1) / p.part_rows), block(64 * kSkinnyWaves);
     switch (a.Ns) {
     case 128: spmm_skinny16_kernel<KS, WS, 4, HIGH, U><<<grid, block, 0, a.stream>>>(p); break;
     case 64: spmm_skinny16_kernel<KS, WS, 2, HIGH, U><<<grid, block, 0, a.stream>>>(p); break;
@@ -445,11 +452,21 @@ static hipError_t launch_qs16(const SpmmArgs& a)
     }
     return hipGetLastError();
 }
-// the 16-row form reads B with 64-bit loads; the C-ABI layer has checked that B is 16-byte aligned
-static bool skinny16_applies(const SpmmArgs& a) { return a.M <= 16; }
-
 // 32-row blocks per wave for a row count
 static int skinny_blocks(int M) { return M <= 32 ? 1 : M <= 64 ? 2 : 4; }
+
+// Rows per workgroup (decode_part_rows): a row-major A only has the one-block forms, and a
+// column-major one needs a pitch that the part's blocks divide.
+static int skinny_part_rows(const SpmmArgs& a)
+{
+    const int rows = decode_part_rows(a.M, a.N / 32);
+    if (!a.a_rowmajor && a.lda % skinny_blocks(rows) != 0)
+        return a.M;
+    return rows;
+}
+
+// the 16-row form reads B with 64-bit loads; the C-ABI layer has checked that B is 16-byte aligned
+static bool skinny16_applies(const SpmmArgs& a) { return skinny_part_rows(a) <= 16; }
 
 bool skinny_supported(const SpmmArgs& a)
 {
@@ -482,7 +499,7 @@ static hipError_t launch_rb(const SpmmArgs& a)
     constexpr int U16 = 32 / WS > 0 ? 32 / WS : 1;
     if (skinny16_applies(a))
         return launch_qs16<KS, WS, HIGH, U16>(a);
-    switch (skinny_blocks(a.M)) {
+    switch (skinny_blocks(skinny_part_rows(a))) {
     case 1: return launch_qs<KS, WS, HIGH, 1, UN>(a);
     case 2: return launch_qs<KS, WS, HIGH, 2, UN>(a);
     default: return launch_qs<KS, WS, HIGH, 4, UN>(a);
