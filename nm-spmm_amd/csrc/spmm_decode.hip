@@ -312,8 +312,11 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
 
 bool decode_supported(const SpmmArgs& a)
 {
-    // up to 32 rows either layout of A; 33 to 64 rows only column-major (wide loads of A)
-    if (a.row_index == nullptr || a.M > 64 || a.vec_len != 32)
+    // up to 32 rows either layout of A; 33 to 64 rows only column-major (wide loads of A); 65 to 128
+    // rows where they are cut into parts of at most 32 rows (few column vectors)
+    if (a.row_index == nullptr || a.M > 128 || a.vec_len != 32)
+        return false;
+    if (a.M > 64 && decode_part_rows(a.M, a.N / 32) > 32)
         return false;
     if (a.a_rowmajor) {
         if (a.M > 32)

@@ -143,12 +143,25 @@ def test_decode_kernel_adds_to_c_when_asked_like_a_split_call_of_the_reference(o
     assert scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
 
 
-@pytest.mark.parametrize("M", [65, 100, 128, 200])
-def test_larger_row_counts_ignore_the_list(oracle, M):
-    d = datagen.init_data(M, 256, 512, 2, 8, seed=3)
+@pytest.mark.parametrize("M,N", [(200, 256), (129, 256), (65, 8192), (128, 8192)])
+def test_larger_row_counts_ignore_the_list(oracle, M, N):
+    """More than 128 rows, and 65 to 128 rows on more column vectors than their 32-row parts could
+    share the compute units with."""
+    d = datagen.init_data(M, N, 512, 2, 8, seed=3)
     got, fam = run_decode(oracle, d)
     assert fam in ("skinny", "mfma")
     assert scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
+
+
+@pytest.mark.parametrize("M", [65, 77, 96, 100, 127, 128])
+@pytest.mark.parametrize("n,m,K,N", [(2, 8, 1088, 256), (1, 8, 2048, 512), (2, 4, 1152, 2048), (3, 8, 96, 128)])
+def test_65_to_128_rows_on_few_column_vectors_are_cut_into_parts(oracle, M, n, m, K, N):
+    """With at most 64 column vectors (2048 columns) 65 to 128 rows run as 32-row parts on the row
+    list, one workgroup per vector and part; the last part may be short or odd."""
+    d = datagen.init_data(M, N, K, n, m, seed=M + K, dist="normal", b_scale=0.02)
+    got, fam = run_decode(oracle, d)
+    assert fam == "decode"
+    assert np.isfinite(got).all() and scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
 
 
 @pytest.mark.parametrize("M", [48, 64])
