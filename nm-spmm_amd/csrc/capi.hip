@@ -499,6 +499,10 @@ size_t nmspmm_workspace_bytes(int M, int N, int split_k)
 // a_rowmajor: A is row-major M x K with `lda` floats between rows; only the decode kernels take
 // that, and kNotTaken comes back (nothing launched) when they do not take the shape.
 constexpr int kNotTaken = -1000;
+// Factor on model_decode_seconds when it is compared with model_tile_seconds (33 to 128 rows; see
+// spmm_impl)
+constexpr double kDecodeBias = 1.25;
+
 static int spmm_impl(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C, int M,
                      int N, int K, int W, int window, int kept, int vec_len, int Ns, int split_k, void* workspace,
                      size_t workspace_bytes, void* stream, int lda, bool dry_run, int* lda_out, bool a_rowmajor = false,
@@ -572,8 +576,17 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
         return kNotTaken;
     hipError_t e;
     // up to 32 rows the kernels with one workgroup per vector always win; up to 128 they compete
-    // with the tile kernel at the caller's split
-    const bool decode_wins = model_decode_seconds(M, N, W / kept, kept) < model_tile_seconds(M, N, W / kept, kept, split_k);
+    // with the tile kernel at the caller's split.  The two models are compared with a bias: on 340
+    // shapes of 33 to 128 rows (2048 to 28672 columns, reductions of 2048 to 11008, four patterns,
+    // each kernel forced in turn, B re-read from the caches and, for 84 of them, streamed from HBM
+    // too) the tile model is 10 to 12 % pessimistic at these row counts and the other 3 to 13 %
+    // optimistic from 4096 columns on.  With the factor the choice is within 1 % of always taking
+    // the faster kernel on average (worst case 16 %), without it 4 to 8 % behind (worst 54 %).  The
+    // kernel on the row list is the faster of the two vector kernels up to 64 rows, most of all with
+    // B from HBM, and gets the smaller factor.
+    const double decode_bias = (row_index != nullptr && M <= 64) ? 1.15 : kDecodeBias;
+    const bool decode_wins = decode_bias * model_decode_seconds(M, N, W / kept, kept) <
+                             model_tile_seconds(M, N, W / kept, kept, split_k);
     if (decode_supported(a) && (M <= 32 || decode_wins || !mfma_supported(a))) {
         // decode sizes with the row list: one launch, reduction inside the workgroup (or, on request,
         // across a few workgroups through the library's device-resident scratch)
@@ -825,7 +838,7 @@ int nmspmm_suggest_split_k(int M, int N, int W, int kept)
             best_t = t;
         }
     }
-    if (M <= 128 && model_decode_seconds(M, N, nwin, kept) < best_t)
+    if (M <= 128 && kDecodeBias * model_decode_seconds(M, N, nwin, kept) < best_t)  // the dispatcher's comparison
         return 1;
     return best;
 }

@@ -52,7 +52,7 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert len(cfg["decode_llm"]) == 9
     for x in cfg["decode_llm"]:
         assert x["kernel"] == "decode" and x["hot_split"]["us"] > 0 and x["cold_split"]["us"] > 0
-    assert len(cfg["decode_wide"]) == 8 and all(x["kernel"] == "decode" and x["M"] in (48, 64) for x in cfg["decode_wide"])
+    assert len(cfg["decode_wide"]) == 8 and all(x["kernel"] in ("decode", "mfma") and x["M"] in (48, 64) for x in cfg["decode_wide"])
     assert [x["pattern"] for x in cfg["fine"]][:4] == ["4:32", "8:32", "16:32", "2:4"] and cfg["fine"][3]["vec_len"] == 4
     assert len(cfg["launch_constant"]) == 3 and len(cfg["compress"]) == 12 and len(cfg["rowmajor"]) == 5
     for x in d["preprocess"]:

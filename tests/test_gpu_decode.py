@@ -165,15 +165,18 @@ def test_65_to_128_rows_on_few_column_vectors_are_cut_into_parts(oracle, M, n, m
 
 
 @pytest.mark.parametrize("M", [48, 64])
-@pytest.mark.parametrize("n,m", [(1, 8), (2, 8)])
-def test_33_to_64_rows_at_full_size_on_the_row_list(oracle, M, n, m):
-    """K = Ncols = 8192, all of C against the checker, with and without the non-temporal hint."""
-    d = datagen.init_data(M, 8192, 8192, n, m, seed=150 + M + n, dist="normal", b_scale=0.02)
+@pytest.mark.parametrize("n,m,K", [(1, 8, 8192), (2, 8, 8192), (1, 8, 256), (2, 8, 256)])
+def test_33_to_64_rows_on_8192_columns_on_the_row_list(oracle, M, n, m, K):
+    """Ncols = 8192 (one workgroup per vector fills the GPU, so the rows are not cut into parts), all
+    of C against the checker, with and without the non-temporal hint.  With a short reduction the
+    library takes the decode kernel's four-halves form; at K = 8192 that form and the tile kernel
+    are within a few per cent of each other and either may be chosen."""
+    d = datagen.init_data(M, 8192, K, n, m, seed=150 + M + n, dist="normal", b_scale=0.02)
     got, fam = run_decode(oracle, d)
-    assert fam == "decode"
+    assert fam == "decode" if K == 256 else fam in ("decode", "mfma")
     assert np.isfinite(got).all() and scaled_max_error(got, want_c(oracle, d)) <= REL_TOL
     streamed, fam = run_decode(oracle, d, flags=nmspmm.STREAM_B)
-    assert fam == "decode" and scaled_max_error(streamed, want_c(oracle, d)) <= REL_TOL
+    assert fam in ("decode", "mfma") and scaled_max_error(streamed, want_c(oracle, d)) <= REL_TOL
 
 
 def test_a_list_off_a_sixteen_byte_boundary_is_rejected(oracle):

@@ -76,12 +76,12 @@ def test_ragged_row_counts(oracle, M, n, m, Ns):
 @pytest.mark.parametrize("M", [34, 48, 64, 68, 96, 100, 128])
 @pytest.mark.parametrize("n,m,Ns", [(1, 8, 128), (2, 8, 64), (2, 4, 32), (3, 8, 128)])
 def test_decode_kernel_up_to_128_rows(oracle, M, n, m, Ns):
-    """Two and four 32-row blocks per wave; K gives the waves of a workgroup unequal shares.  The
-    shape (many columns, short reduction) is one where the run-time model prefers this kernel."""
-    K = 512 if m == 8 else 576
-    d = datagen.init_data(M, 8192, K, n, m, seed=M + Ns, dist="normal", b_scale=0.02)
+    """Two and four 32-row blocks per wave; K gives the waves of a workgroup unequal shares, some
+    none.  The shape (many columns, a short reduction) is one where the run-time model prefers this
+    kernel to the tile kernel: clearly at 1:8 and 2:8, by a hair at 2:4 and 3:8."""
+    d = datagen.init_data(M, 8192, 256, n, m, seed=M + Ns, dist="normal", b_scale=0.02)
     got, fam = run_gpu(oracle, d, Ns)
-    assert fam == "skinny"
+    assert fam == "skinny" if m == 8 and n <= 2 else fam in ("skinny", "mfma")
     check(oracle, d, got)
 
 
