@@ -581,11 +581,10 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     // each kernel forced in turn, B re-read from the caches and, for 84 of them, streamed from HBM
     // too) the tile model is 10 to 12 % pessimistic at these row counts and the other 3 to 13 %
     // optimistic from 4096 columns on.  With the factor the choice is within 1 % of always taking
-    // the faster kernel on average (worst case 16 %), without it 4 to 8 % behind (worst 54 %).  The
-    // kernel on the row list is the faster of the two vector kernels up to 64 rows, most of all with
-    // B from HBM, and gets the smaller factor.
-    const double decode_bias = (row_index != nullptr && M <= 64) ? 1.15 : kDecodeBias;
-    const bool decode_wins = decode_bias * model_decode_seconds(M, N, W / kept, kept) <
+    // the faster kernel on average, without it 4 to 8 % behind (worst 54 %).  (Fitted before the tile
+    // kernel's launches of at most one 64-row workgroup per CU got eight waves along K, which only
+    // moved ties towards the tile kernel.)
+    const bool decode_wins = kDecodeBias * model_decode_seconds(M, N, W / kept, kept) <
                              model_tile_seconds(M, N, W / kept, kept, split_k);
     if (decode_supported(a) && (M <= 32 || decode_wins || !mfma_supported(a))) {
         // decode sizes with the row list: one launch, reduction inside the workgroup (or, on request,

@@ -421,6 +421,19 @@ def test_reduction_shared_between_the_waves_of_a_workgroup(oracle, M, N, K, n, m
     check_every_tile_once(oracle, M, N, K, n, m, Ns)
 
 
+@pytest.mark.parametrize("M,N,K,n,m", [(100, 4096, 1088, 2, 8), (160, 2048, 1472, 2, 4), (192, 2048, 1216, 1, 8), (256, 2048, 1120, 3, 8),
+                                       (96, 4096, 2048, 1, 8), (130, 1024, 544, 2, 4)])
+@pytest.mark.parametrize("Ns", [128, 64, 32])
+def test_eight_waves_along_k_where_every_workgroup_has_a_cu(oracle, M, N, K, n, m, Ns):
+    """At most one 64-row workgroup per compute unit and at least sixteen windows: eight waves share
+    the reduction (17, 46, 19, 35 and 17 windows: unequal eighths; 32: equal ones).  Every tile
+    exactly once, every index layout, every width of the column blocks."""
+    window, kept, _ = kernel_geometry(n, m)
+    assert nmspmm.waves_along_k_rows(M, N, K // window * kept, kept) == 64
+    assert -(-M // 64) * (N // 32) <= nmspmm.device_figures()[0] and K // window >= 16
+    check_every_tile_once(oracle, M, N, K, n, m, Ns)
+
+
 def test_larger_problems_stay_on_whole_tiles():
     assert nmspmm.waves_along_k_rows(2048, 4096, 2048, 16) == 0    # 512 tiles
     assert nmspmm.waves_along_k_rows(256, 2048, 64, 16) == 0       # four windows: nothing to share
