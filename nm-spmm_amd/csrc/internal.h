@@ -296,6 +296,7 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
 struct InnerPlan {
     bool pays;     // eligible at all
     int rows;      // 128 or 64 rows per workgroup
+    int waves;     // 4, or 8 where every workgroup has a compute unit to itself
     double seconds;  // modelled kernel time
 };
 inline InnerPlan plan_inner(int M, int N, int nwin, int kept)
@@ -303,6 +304,7 @@ inline InnerPlan plan_inner(int M, int N, int nwin, int kept)
     InnerPlan r;
     r.pays = false;
     r.rows = 128;
+    r.waves = 4;
     r.seconds = 0.0;
     const long long cus = machine().cus;
     const long long tiles = (long long)((M + 127) / 128) * ((N + 127) / 128);
@@ -317,6 +319,22 @@ inline InnerPlan plan_inner(int M, int N, int nwin, int kept)
     r.pays = true;
     r.rows = c2 < c4 ? 64 : 128;
     r.seconds = (c2 < c4 ? c2 : c4) * unit + 1e-6;
+    // Eight waves along K (two per SIMD; 64 or 128 KB of LDS) where every workgroup gets a compute
+    // unit to itself and there are at least 16 windows: on 64 rows if that is the form chosen and its
+    // workgroups fit the compute units once, else on 128 rows if those do.  Measured: 64 rows 6 to
+    // 16 % shorter than four waves with B in the caches and 12 to 30 % with B from HBM (K = 11008 on
+    // 4096 columns at 1:8, 96 rows: 18.1 -> 15.2 and 23.7 -> 16.7 us); 128 rows against the two
+    // 64-row workgroups per CU they replace (4096 columns, 129 to 256 rows) level with B in the
+    // caches, 5 to 17 % shorter with B from HBM.  With more workgroups than compute units eight
+    // waves are level to 5 % longer.
+    if (nwin >= 16) {
+        if (r.rows == 64 && g2 <= cus) {
+            r.waves = 8;
+        } else if (g4 <= cus) {
+            r.rows = 128;
+            r.waves = 8;
+        }
+    }
     return r;
 }
 

@@ -345,7 +345,7 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
         // Waves along K: every wave leaves its sums in LDS, and the groups of four result registers
         // are dealt out to the waves, group g to wave g % KW, which adds the KW partial sums in wave
         // order (the order of the windows) and stores the group's four rows.
-        static_assert(KW * RM <= 16, "64 KB of LDS");
+        static_assert(KW * RM <= 32, "128 KB of LDS for one workgroup per CU, 64 KB where two share a CU");
         __shared__ float4 partial[KW][RM * 4][64];
 #pragma unroll
         for (int b = 0; b < RM; ++b)
@@ -449,11 +449,12 @@ __global__ void __launch_bounds__(256, 2) spmm_direct_inner_kernel(const DirectP
     direct_uniform_launch<KS, WS, QS, 1, RM, HIGH, DEEP, 4>(p, blockIdx.x);
 }
 
-// Eight waves along K, 64 rows: for launches of at most one such workgroup per CU.
-template <int KS, int WS, int QS, bool HIGH, bool DEEP>
+// Eight waves along K, 64 or 128 rows (64 or 128 KB of LDS): for launches of at most one such
+// workgroup per CU.
+template <int KS, int WS, int QS, int RM, bool HIGH, bool DEEP>
 __global__ void __launch_bounds__(512, 1) spmm_direct_inner8_kernel(const DirectParams p)
 {
-    direct_uniform_launch<KS, WS, QS, 1, 2, HIGH, DEEP, 8>(p, blockIdx.x);
+    direct_uniform_launch<KS, WS, QS, 1, RM, HIGH, DEEP, 8>(p, blockIdx.x);
 }
 
 // The first p.head_units workgroups compute whole tiles; the ones after them the tiles from
@@ -633,8 +634,10 @@ template <int KS, int WS, int QS, bool HIGH>
 static hipError_t launch_inner(const SpmmArgs& a)
 {
     const long long vecs = a.N / 32;
-    const int rows = plan_inner(a.M, a.N, a.W / WS, WS).rows;
+    const InnerPlan plan = plan_inner(a.M, a.N, a.W / WS, WS);
+    const int rows = plan.rows;
     const bool tall = rows == 128;
+    const bool eight = plan.waves == 8;
     DirectParams p;
     p.A = a.A;
     p.B = a.B;
@@ -662,18 +665,15 @@ static hipError_t launch_inner(const SpmmArgs& a)
     p.head_units = (int)groups;
     const dim3 grid((unsigned)groups), block(256);
     const bool lone = groups <= machine().cus;
-    if (tall) {
+    if (tall && eight) {
+        spmm_direct_inner8_kernel<KS, WS, QS, 4, HIGH, has_lone_form<WS, 4, HIGH>()><<<grid, dim3(512), 0, a.stream>>>(p);
+    } else if (tall) {
         if (lone && has_lone_form<WS, 4, HIGH>())
             spmm_direct_inner_kernel<KS, WS, QS, 4, HIGH, has_lone_form<WS, 4, HIGH>()><<<grid, block, 0, a.stream>>>(p);
         else
             spmm_direct_inner_kernel<KS, WS, QS, 4, HIGH, false><<<grid, block, 0, a.stream>>>(p);
-    } else if (lone && a.W / WS >= 16) {
-        // at most one 64-row workgroup per CU: eight waves along K instead of four (two per SIMD,
-        // the same 64 KB of LDS).  Measured on 4096 columns at 96 and 128 rows and on 8192 columns
-        // at 40 and 64 rows: 6 to 16 % shorter with B in the caches, 12 to 30 % with B from HBM
-        // (K = 11008 on 4096 columns at 1:8, 96 rows: 18.1 -> 15.2 and 23.7 -> 16.7 us); with more
-        // workgroups than CUs level to 5 % longer, which is why only here.
-        spmm_direct_inner8_kernel<KS, WS, QS, HIGH, has_lone_form<WS, 2, HIGH>()><<<grid, dim3(512), 0, a.stream>>>(p);
+    } else if (eight) {
+        spmm_direct_inner8_kernel<KS, WS, QS, 2, HIGH, has_lone_form<WS, 2, HIGH>()><<<grid, dim3(512), 0, a.stream>>>(p);
     } else {
         if (lone && has_lone_form<WS, 2, HIGH>())
             spmm_direct_inner_kernel<KS, WS, QS, 2, HIGH, has_lone_form<WS, 2, HIGH>()><<<grid, block, 0, a.stream>>>(p);

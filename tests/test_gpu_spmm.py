@@ -409,12 +409,14 @@ def test_waves_that_load_b_two_windows_ahead(oracle, M, N, K, n, m, Ns):
 
 @pytest.mark.parametrize("M,N,K,n,m,rows", [(256, 2048, 512, 2, 4, 64), (512, 4096, 1024, 1, 8, 128), (192, 1024, 1024, 2, 8, 64),
                                             (1000, 2048, 1056, 3, 8, 128), (300, 1024, 352, 32, 32, 64), (132, 2048, 512, 2, 4, 64),
-                                            (768, 4096, 2112, 1, 8, 64), (256, 8192, 2112, 2, 8, 128)])
+                                            (768, 4096, 2112, 1, 8, 64), (256, 8192, 2112, 2, 8, 128),
+                                            (200, 4096, 1088, 2, 8, 128), (256, 4096, 1056, 2, 4, 128), (250, 4096, 1216, 1, 8, 128)])
 @pytest.mark.parametrize("Ns", [128, 64, 32])
 def test_reduction_shared_between_the_waves_of_a_workgroup(oracle, M, N, K, n, m, rows, Ns):
     """Problems of few tiles: one workgroup per 128 or 64 rows of one 32-column vector, its four
     waves each over a quarter of the windows (33 and eleven windows: unequal quarters), partial
-    sums added in LDS.  Ragged row counts, every index layout, every width of the column blocks;
+    sums added in LDS; the last three cases are at most one 128-row workgroup per compute unit,
+    which take eight waves (17, 33 and 19 windows).  Ragged row counts, every index layout, every width of the column blocks;
     every tile exactly once."""
     window, kept, _ = kernel_geometry(n, m)
     assert nmspmm.waves_along_k_rows(M, N, K // window * kept, kept) == rows
