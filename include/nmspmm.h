@@ -181,8 +181,9 @@ int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t*
  * row_index: NULL, or the row list nmspmm_row_index_device() made from these same D / column_info
  * (16-byte aligned).  With it, M <= 32 runs on the decode kernel that reads the list instead of
  * D and column_info, and so does M of 33 to 64 with column-major A wherever the library expects
- * one workgroup per vector to beat the tile kernel (K = Ncols = 8192 at 48 or 64 rows: 22.5 against
- * 24.3 us at 2:8, 13.8 against 15.7 us at 1:8), and M up to 128 on so few columns that its 32-row
+ * one workgroup per vector to beat the tile kernel (short reductions, or few columns: K = Ncols =
+ * 4096 at 64 rows 8.4 us on the list against 8.8 us on D / column_info at 2:8, 5.4 against 6.1 us
+ * at 1:8), and M up to 128 on so few columns that its 32-row
  * parts get a workgroup each (one per 32 columns and part, at most as many as compute units:
  * Ncols <= 2048 on an MI355X); larger M ignore it. */
 #define NMSPMM_ACCUMULATE 1u
