@@ -233,8 +233,10 @@ def tile_kernel_name(pkg, case):
     if rows == 0:
         return "spmm_direct_inner_kernel (waves along K, %d rows)" % pkg.waves_along_k_rows(M, N, case.W, case.kept)
     qs = NS // 32
-    return "spmm_direct_kernel<%d,%d,%d,%d,%d,%s>" % (case.window, case.kept, qs, 4 // qs, rows // 32,
-                                                     "true" if case.cinfo is not None else "false")
+    high = "true" if case.cinfo is not None else "false"
+    if pkg.tile_wave_sets(M, N, case.W, case.kept, NS, 1) == 2:
+        return "spmm_direct_halves_kernel<%d,%d,%d,%d,%s>" % (case.window, case.kept, qs, 4 // qs, high)
+    return "spmm_direct_kernel<%d,%d,%d,%d,%d,%s>" % (case.window, case.kept, qs, 4 // qs, rows // 32, high)
 
 
 def profiled_traffic():

@@ -297,6 +297,11 @@ int nmspmm_device_figures(int* compute_units, int* dies, double* clock_hz);
  * with waves along K (nmspmm_waves_along_k_rows) or the arguments are invalid.  Informational,
  * for profiles and benchmarks that want to name the kernel instance that ran. */
 int nmspmm_tile_wave_rows(int M, int N, int W, int kept, int Ns, int split_k);
+/* No counterpart in the reference.  Sets of four waves per workgroup of the matrix-core tile
+ * kernel for this shape: 2 when a whole unsplit problem is at most one workgroup of 256-row waves
+ * per compute unit and long enough along K (each set then takes half of the windows and the halves
+ * are added up in LDS), 1 otherwise, 0 where nmspmm_tile_wave_rows returns 0.  Informational. */
+int nmspmm_tile_wave_sets(int M, int N, int W, int kept, int Ns, int split_k);
 int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int32_t* column_info,
                      float* C, int M, int N, int K, int W, float sparsity, void* stream);
 

@@ -78,6 +78,7 @@ def lib():
         L.nmspmm_suggest_split_k.argtypes = [c_int] * 4
         L.nmspmm_waves_along_k_rows.argtypes = [c_int] * 4
         L.nmspmm_tile_wave_rows.argtypes = [c_int] * 6
+        L.nmspmm_tile_wave_sets.argtypes = [c_int] * 6
         L.nmspmm_device_figures.argtypes = [ip, ip, ctypes.POINTER(ctypes.c_double)]
         L.nmspmm_gemm_auto.argtypes = [c_void_p] * 5 + [c_int] * 4 + [c_float, c_void_p]
         L.nmspmm_release.restype = c_int
@@ -287,6 +288,11 @@ def device_figures():
 def tile_wave_rows(M, N, W, kept, Ns=128, split_k=1):
     """Rows per wave of the tile kernel for this call (256, 128, 64), 0 for the launch with waves along K."""
     return lib().nmspmm_tile_wave_rows(M, N, W, kept, Ns, split_k)
+
+
+def tile_wave_sets(M, N, W, kept, Ns=128, split_k=1):
+    """Sets of four waves per workgroup of the tile kernel for this call (2: each set takes half of the windows)."""
+    return lib().nmspmm_tile_wave_sets(M, N, W, kept, Ns, split_k)
 
 
 def gemm_auto(A, B, D, cinfo, C, M, N, K, W, sparsity):

@@ -874,6 +874,21 @@ int nmspmm_tile_wave_rows(int M, int N, int W, int kept, int Ns, int split_k)
     return 32 * blocks;
 }
 
+int nmspmm_tile_wave_sets(int M, int N, int W, int kept, int Ns, int split_k)
+{
+    const int rows = nmspmm_tile_wave_rows(M, N, W, kept, Ns, split_k);
+    if (rows == 0)
+        return 0;
+    if (rows != 256 || split_k != 1)
+        return 1;
+    const int wr = 128 / Ns;  // waves along M: a workgroup is 256 * wr rows by Ns columns
+    const long long tiles = (long long)((M + 256 * wr - 1) / (256 * wr)) * (N / Ns);
+    const TailPlan t = plan_tail(M, N, W / kept, kept, wr);
+    if (t.separate && t.blocks == 8)
+        return 1;  // leftover tiles in a launch of their own: no launch is the whole problem
+    return wave_sets_pay(tiles, W / kept, kept) ? 2 : 1;
+}
+
 int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int32_t* column_info, float* C,
                      int M, int N, int K, int W, float sparsity, void* stream)
 {

@@ -350,6 +350,19 @@ inline bool inner_split_pays(int M, int N, int nwin, int kept)
     return inner.seconds < model_kernel_seconds(M, N, nwin, kept, blocks, 1);
 }
 
+// Whether a launch of whole tiles of 256-row waves runs each workgroup as two sets of four waves,
+// each set over half of the windows, added up in LDS (128 KB).  Such waves fit two to a SIMD, so a
+// launch of at most one workgroup per CU leaves every SIMD with a single wave; with the second set
+// the matrix pipe has another wave to issue from while one waits for its operands.  Measured over
+// 2:8, 1:4 and 2:4 at 1024 to 4096 rows: 2 to 4 % shorter from 768 kept rows per vector up (2048 x
+// 4096 x 4096 at 2:8: 126.8 -> 124.1 us; at 2:4: 246.7 -> 238.5), 1 to 3 % at 512, level at 384,
+// 1 to 2 % longer at 256, where the second set's prologue and the exchange weigh more than the
+// overlap gives.
+inline bool wave_sets_pay(long long workgroups, int nwin, int kept)
+{
+    return workgroups <= machine().cus && (long long)nwin * kept >= 512;
+}
+
 // Whole multiplication on the tile kernel: 6 us per launch, C written at about 8 TB/s, the kernel,
 // and for a split the second pass that moves (2 * split + 1) * M * N floats at about 8 TB/s (the
 // slices are cache resident) plus 4 us for its launch behind the first.

@@ -111,7 +111,7 @@ constexpr bool has_lone_form()
 // K.  With KW > 1 (WR == 1) the workgroup's KW waves compute the same RM*32 rows of ONE 32-column
 // vector, each over its share of the windows, and add their results up through LDS in wave order;
 // QS then only describes the index layout, and the tile walk counts vectors, not column blocks.
-template <int KS, int WS, int QS, int WR, int RM, bool HIGH, bool DEEP = false, int KW = 1>
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH, bool DEEP = false, int KW = 1, int KH = 1>
 __device__ __forceinline__ void direct_unit(const DirectParams& p, const int logical, const int sub, const int sub_tiles,
                                             const bool tail_unit, const int unit)
 {
@@ -141,10 +141,15 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
         tile_n = in_band / rows;
     }
     const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    static_assert(KH == 1 || (KH == 2 && KW == 1 && RM == 8), "two sets of waves only on whole 256-row waves");
+    const int wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave = KH > 1 ? wave_all % (QS * WR) : wave_all;
+    const int kh = KH > 1 ? wave_all / (QS * WR) : 0;
     int w_begin, w_count;
     if constexpr (KW > 1)
         split_windows(p.nwin, KW, wave, &w_begin, &w_count);
+    else if constexpr (KH > 1)
+        split_windows(p.nwin, KH, kh, &w_begin, &w_count);
     else if (!tail_unit)
         split_windows(p.nwin, p.split_k, blockIdx.y, &w_begin, &w_count);
     else
@@ -384,11 +389,11 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
     // the launch 1 to 1.7 us less at its end than lines left dirty in L2 (4096 x 4096 x 1024 at 1:8:
     // 41.0 -> 39.3 us).  Slices of a cut reduction keep the default policy (stored this way too they
     // were measured within -6 to +1 %, most shapes level).
-    const auto store_all = [&](auto policy) {
+    const auto store_blocks = [&](auto policy, auto first, auto count) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
 #pragma unroll
-            for (int b = 0; b < RM; ++b) {
+            for (int b = decltype(first)::value; b < decltype(first)::value + decltype(count)::value; ++b) {
                 // row inside the wave, without the lane's 4*IL*h: IL * (8*(v/4) + v%4) + b%IL, second group + 128
                 const uint32_t row = (b / 4) * 128 + IL * (8 * (v / 4) + (v % 4)) + (b % IL);
                 __builtin_amdgcn_raw_buffer_store_b32(__float_as_int(acc[b][v]), rc, c_lane + row * n_bytes, 0,
@@ -396,17 +401,63 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
             }
         }
     };
+    if constexpr (KH == 2) {
+        // Two sets of waves, each over half of the windows: every wave hands the half of its result
+        // blocks that the other set stores to its partner through LDS, adds what it is handed (one
+        // addition per element, so the order does not matter) and stores its own half.
+        constexpr int HB = RM / 2;
+        __shared__ float4 handed[2][QS * WR][HB * 4][64];
+        const auto hand = [&](auto first) {
+#pragma unroll
+            for (int b = 0; b < HB; ++b)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const floatx16& r = acc[decltype(first)::value + b];
+                    handed[kh][wave][b * 4 + q][lane] = make_float4(r[4 * q], r[4 * q + 1], r[4 * q + 2], r[4 * q + 3]);
+                }
+        };
+        const auto take = [&](auto first) {
+#pragma unroll
+            for (int b = 0; b < HB; ++b)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 t = handed[1 - kh][wave][b * 4 + q][lane];
+                    floatx16& r = acc[decltype(first)::value + b];
+                    r[4 * q] += t.x;
+                    r[4 * q + 1] += t.y;
+                    r[4 * q + 2] += t.z;
+                    r[4 * q + 3] += t.w;
+                }
+        };
+        typedef std::integral_constant<int, 0> lower;
+        typedef std::integral_constant<int, HB> upper;
+        if (kh == 0)
+            hand(upper{});
+        else
+            hand(lower{});
+        __syncthreads();
+        if (kh == 0) {
+            take(lower{});
+            store_blocks(std::integral_constant<int, 16>{}, lower{}, upper{});
+        } else {
+            take(upper{});
+            store_blocks(std::integral_constant<int, 16>{}, upper{}, upper{});
+        }
+        return;
+    }
+    typedef std::integral_constant<int, 0> first_block;
+    typedef std::integral_constant<int, RM> all_blocks;
     if (!tail_unit && p.split_k == 1)
-        store_all(std::integral_constant<int, 16>{});
+        store_blocks(std::integral_constant<int, 16>{}, first_block{}, all_blocks{});
     else
-        store_all(std::integral_constant<int, 0>{});
+        store_blocks(std::integral_constant<int, 0>{}, first_block{}, all_blocks{});
 }
 
 // Workgroup `id` of a launch whose workgroups all compute the same kind of unit.  Whole tiles: a
 // walk that gives each XCD (consecutive ids go to different XCDs) a contiguous run of the
 // p.head_units logical tiles.  In a launch of K slices (p.tail_slices > 1) consecutive ids are the
 // slices of one tile, in a launch of pieces along M (p.sub_tiles > 1) the pieces of one tile.
-template <int KS, int WS, int QS, int WR, int RM, bool HIGH, bool DEEP = false, int KW = 1>
+template <int KS, int WS, int QS, int WR, int RM, bool HIGH, bool DEEP = false, int KW = 1, int KH = 1>
 __device__ __forceinline__ void direct_uniform_launch(const DirectParams& p, const int id)
 {
     const bool tail_unit = p.tail_slices > 1;
@@ -422,7 +473,7 @@ __device__ __forceinline__ void direct_uniform_launch(const DirectParams& p, con
         const int xcd = id % p.xcds, loc = id / p.xcds;
         logical = p.tile_offset + (xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc);
     }
-    direct_unit<KS, WS, QS, WR, RM, HIGH, DEEP, KW>(p, logical, sub, p.sub_tiles, tail_unit, id);
+    direct_unit<KS, WS, QS, WR, RM, HIGH, DEEP, KW, KH>(p, logical, sub, p.sub_tiles, tail_unit, id);
 }
 
 #define NMSPMM_DIRECT_BOUNDS __launch_bounds__(64 * QS * WR, RM == 8 ? 2 : (HIGH && WS == 16) ? 4 : kWavesPerSimd)
@@ -438,6 +489,15 @@ template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
 __global__ void NMSPMM_DIRECT_BOUNDS spmm_direct_lone_kernel(const DirectParams p)
 {
     direct_uniform_launch<KS, WS, QS, WR, RM, HIGH, true>(p, blockIdx.x);
+}
+
+// Whole tiles of 256-row waves with two sets of waves, each over half of the windows (128 KB of
+// LDS): for launches of at most one such workgroup per CU, which would otherwise leave every SIMD
+// with a single wave.
+template <int KS, int WS, int QS, int WR, bool HIGH>
+__global__ void __launch_bounds__(128 * QS * WR, 1) spmm_direct_halves_kernel(const DirectParams p)
+{
+    direct_uniform_launch<KS, WS, QS, WR, 8, HIGH, false, 1, 2>(p, blockIdx.x);
 }
 
 // Four waves along K: one workgroup per RM*32 rows of one 32-column vector (p.tiles_n counts
@@ -524,14 +584,23 @@ tail_reduce_kernel(const float* __restrict__ ws, float* __restrict__ C, int M, i
 }
 
 // One launch of uniform workgroups.  A launch of at most one workgroup per CU (each wave alone on
-// its SIMD) takes the form that loads B two windows ahead where the tile shape has one.
+// its SIMD) takes the form that loads B two windows ahead where the tile shape has one; a whole
+// problem of at most that many tiles of 256-row waves the form with two sets of waves
+// (wave_sets_pay).
 template <int KS, int WS, int QS, int WR, int RM, bool HIGH>
-static hipError_t launch_uniform(const dim3 grid, const dim3 block, hipStream_t stream, const DirectParams& p)
+static hipError_t launch_uniform(const dim3 grid, const dim3 block, hipStream_t stream, const DirectParams& p,
+                                 const bool whole_problem = false)
 {
     bool lone = false;
     if constexpr (has_lone_form<WS, RM, HIGH>())
         lone = (long long)grid.x * grid.y <= machine().cus;
-    if (lone) {
+    bool halves = false;
+    if constexpr (RM == 8)
+        halves = whole_problem && p.split_k == 1 && wave_sets_pay(grid.x, p.nwin, WS);
+    if (halves) {
+        if constexpr (RM == 8)
+            spmm_direct_halves_kernel<KS, WS, QS, WR, HIGH><<<grid, dim3(2 * block.x), 0, stream>>>(p);
+    } else if (lone) {
         if constexpr (has_lone_form<WS, RM, HIGH>())
             spmm_direct_lone_kernel<KS, WS, QS, WR, RM, HIGH><<<grid, block, 0, stream>>>(p);
     } else {
@@ -572,7 +641,7 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     dim3 grid(p.tiles_m * p.tiles_n, a.split_k, 1);
     p.head_units = (int)grid.x;
     if (!own_tail)
-        return launch_uniform<KS, WS, QS, WR, RM, HIGH>(grid, block, a.stream, p);
+        return launch_uniform<KS, WS, QS, WR, RM, HIGH>(grid, block, a.stream, p, true);
     p.head_units = (int)plan.head;
     if (plan.slices == 1 && plan.sub > 1 && plan.fused) {
         // shorter waves for the leftovers, in the same launch: each leftover tile in two pieces

@@ -61,6 +61,23 @@ def test_device_figures_without_a_gpu_are_those_of_an_mi355x():
     assert nmspmm.device_figures() == (256, 8, 2.4e9)
 
 
+def test_wave_sets_of_the_tile_kernel():
+    """Two sets of waves per workgroup only for a whole unsplit problem of at most one workgroup of
+    256-row waves per compute unit (256 without a GPU) with at least 512 kept rows per vector."""
+    import torch
+    if torch.cuda.is_available() and nmspmm.device_figures()[0] != 256:
+        pytest.skip("the shapes below are sized for 256 compute units")
+    for Ns in (128, 64, 32):
+        assert nmspmm.tile_wave_rows(2048, 4096, 1024, 16, Ns) == 256
+        assert nmspmm.tile_wave_sets(2048, 4096, 1024, 16, Ns) == 2      # 256 workgroups
+        assert nmspmm.tile_wave_sets(2048, 8192, 1024, 16, Ns) == 1      # 512 workgroups
+        assert nmspmm.tile_wave_sets(2048, 4096, 256, 16, Ns) == 1       # short along K
+        assert nmspmm.tile_wave_sets(2048, 4096, 1024, 16, Ns, 2) == 1   # split by the caller
+    assert nmspmm.tile_wave_sets(2048, 4096, 512, 8) == 1                # 128-row waves
+    assert nmspmm.tile_wave_sets(64, 4096, 1024, 16) == 0                # waves along K: another launch
+    assert nmspmm.tile_wave_sets(0, 4096, 1024, 16) == 0 and nmspmm.tile_wave_sets(64, 4096, 1000, 16) == 0
+
+
 def test_pattern_table():
     assert nmspmm.pattern_from_sparsity(0.0) == (32, 32, False)
     assert nmspmm.pattern_from_sparsity(0.5) == (32, 16, False)

@@ -436,7 +436,26 @@ def test_eight_waves_along_k_where_every_workgroup_has_a_cu(oracle, M, N, K, n, 
     check_every_tile_once(oracle, M, N, K, n, m, Ns)
 
 
+@pytest.mark.parametrize("M,N,K,n,m", [(2048, 4096, 2112, 2, 8), (2000, 4096, 1056, 2, 4), (1024, 8192, 2240, 2, 8), (4096, 2048, 1120, 2, 4),
+                                       (2048, 4096, 544, 32, 32), (2048, 4096, 2048, 2, 8), (1990, 4096, 2368, 8, 32)])
+@pytest.mark.parametrize("Ns", [128, 64, 32])
+def test_two_sets_of_waves_where_every_workgroup_has_a_cu(oracle, M, N, K, n, m, Ns):
+    """A whole problem of at most one workgroup of 256-row waves per compute unit and at least 512
+    kept rows per vector: each workgroup runs two sets of four waves, one per half of the windows
+    (33, 33, 35, 35, 17 and 37 windows: unequal halves; 32: equal ones; two ragged row counts),
+    and the sets exchange half of their sums through LDS.  Every tile exactly once, every index
+    layout, every width of the column blocks."""
+    window, kept, _ = kernel_geometry(n, m)
+    assert nmspmm.tile_wave_rows(M, N, K // window * kept, kept, Ns) == 256
+    assert nmspmm.tile_wave_sets(M, N, K // window * kept, kept, Ns) == 2
+    check_every_tile_once(oracle, M, N, K, n, m, Ns)
+
+
 def test_larger_problems_stay_on_whole_tiles():
+    assert nmspmm.tile_wave_sets(2048, 8192, 512, 16) == 1         # 512 tiles of 256-row waves
+    assert nmspmm.tile_wave_sets(2048, 4096, 256, 16) == 1         # 256 kept rows: too short along K
+    assert nmspmm.tile_wave_sets(2048, 4096, 1024, 16, 128, 2) == 1
+    assert nmspmm.tile_wave_sets(0, 4096, 1024, 16) == 0
     assert nmspmm.waves_along_k_rows(2048, 4096, 2048, 16) == 0    # 512 tiles
     assert nmspmm.waves_along_k_rows(256, 2048, 64, 16) == 0       # four windows: nothing to share
     assert nmspmm.waves_along_k_rows(0, 2048, 64, 16) == 0
