@@ -285,6 +285,10 @@ int nmspmm_suggest_split_k(int M, int N, int W, int kept);
  * workspace, one launch), 0 when it is computed tile by tile or the arguments are invalid.
  * Informational: the choice is the library's. */
 int nmspmm_waves_along_k_rows(int M, int N, int W, int kept);
+/* No counterpart in the reference.  Waves of each workgroup of that launch (4 or 8: with eight, a
+ * compute unit holds half as many workgroups, each with twice the waves), 0 where
+ * nmspmm_waves_along_k_rows returns 0.  Informational. */
+int nmspmm_waves_along_k_count(int M, int N, int W, int kept);
 /* No counterpart in the reference.  What the library's planning (split choice, wave height, tile
  * walk) assumes about the current device: compute units, accelerator dies (each with its own L2)
  * and shader clock, read from the HIP runtime once per device; the figures of an MI355X

@@ -77,6 +77,7 @@ def lib():
         L.nmspmm_spmm_rowmajor_ex.argtypes = [c_void_p] * 6 + [c_int] * 9 + [c_void_p, c_size_t, ctypes.c_uint, c_void_p]
         L.nmspmm_suggest_split_k.argtypes = [c_int] * 4
         L.nmspmm_waves_along_k_rows.argtypes = [c_int] * 4
+        L.nmspmm_waves_along_k_count.argtypes = [c_int] * 4
         L.nmspmm_tile_wave_rows.argtypes = [c_int] * 6
         L.nmspmm_tile_wave_sets.argtypes = [c_int] * 6
         L.nmspmm_device_figures.argtypes = [ip, ip, ctypes.POINTER(ctypes.c_double)]
@@ -276,6 +277,11 @@ def waves_along_k_rows(M, N, W, kept):
     """128 or 64 when an unsplit multiplication of this shape shares the reduction between the
     waves of a workgroup, 0 otherwise."""
     return lib().nmspmm_waves_along_k_rows(M, N, W, kept)
+
+
+def waves_along_k_count(M, N, W, kept):
+    """Waves per workgroup (4 or 8) of the launch with waves along K, 0 where that launch is not taken."""
+    return lib().nmspmm_waves_along_k_count(M, N, W, kept)
 
 
 def device_figures():

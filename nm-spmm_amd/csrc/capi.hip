@@ -849,6 +849,13 @@ int nmspmm_waves_along_k_rows(int M, int N, int W, int kept)
     return inner_split_pays(M, N, W / kept, kept) ? plan_inner(M, N, W / kept, kept).rows : 0;
 }
 
+int nmspmm_waves_along_k_count(int M, int N, int W, int kept)
+{
+    if (nmspmm_waves_along_k_rows(M, N, W, kept) == 0)
+        return 0;
+    return plan_inner(M, N, W / kept, kept).waves;
+}
+
 int nmspmm_device_figures(int* compute_units, int* dies, double* clock_hz)
 {
     const Machine& m = machine();

@@ -335,6 +335,49 @@ inline InnerPlan plan_inner(int M, int N, int nwin, int kept)
             r.waves = 8;
         }
     }
+    // More than two layers of 64-row workgroups: the four forms (64 or 128 rows, four or eight
+    // waves) are priced by a fit on 123 shapes with each form forced (320 to 2048 rows on 2048 to
+    // 8192 columns, K = 4096 to 14336, 2:8, 2:4 and 1:8; mean error 1 to 2.5 % per form), in
+    // `unit`s per workgroup per CU plus a fixed cost per layer and launch (the latter less the
+    // 6 us that the tile kernel's launches of 100 to 256 tiles cost beyond their model, which
+    // prices none: the two are compared).  A layer that is not
+    // full costs 0.4 to 1 of a full one.  64-row workgroups cost 0.60 a layer; on four waves a CU
+    // holds four of them and the few workgroups left after a full round of 1024 land packed on
+    // the CUs that free up first (+0.38 and +0.12 with up to one and two layers left), on eight
+    // waves it holds two and ends evenly.  128-row workgroups cost 0.95 a layer plus 0.155 per
+    // workgroup; on four waves an odd layer runs one wave per SIMD (+0.22), on eight waves every
+    // layer has two, for 1.5 us more per layer (the exchange between eight waves through 128 KB of
+    // LDS).  The choice lands within 0.3 % of the best form on average (2.2 % before, when only
+    // the two four-wave forms were priced; 768 x 4096 x 14336 at 2:8: 194 -> 169 us, 640 x 4096 x
+    // 8192 at 2:4: 189 -> 170 us).  Up to 128 rows the earlier pricing stays (the choice between this
+    // kernel and the ones for few rows was fitted against it), and below 32 windows, where the fixed
+    // costs decide and the forms were measured within 7 % of each other either way.
+    if (g2 > 2 * cus && M > 128 && nwin >= 32) {
+        const double q2 = (double)g2 / (double)cus, q4 = (double)g4 / (double)cus;
+        const double frac2 = q2 - (double)(g2 / cus);
+        const double layers2 = (double)(g2 / cus) + (frac2 > 0.0 ? 0.4 + 0.6 * frac2 : 0.0);
+        const double left = q2 > 4.0 ? q2 - 4.0 * (double)(g2 / (4 * cus)) : 0.0;  // layers after full rounds of four
+        const double packed = left > 0.0 && left <= 1.0 ? 0.38 : left > 1.0 && left <= 2.0 ? 0.12 : 0.0;
+        const double c64 = 0.60 * layers2;
+        const double c128 = 0.95 * (double)b4 + 0.155 * q4;
+        const double odd = b4 % 2 == 1 && b4 >= 3 ? 0.22 : 0.0;
+        struct Form { int rows, waves; double seconds; };
+        const Form forms[4] = {
+            {64, 4, (c64 + packed) * unit + 0.67e-6 * (double)b2 - 3.8e-6},
+            {128, 4, (c128 + odd) * unit + 1.47e-6 * (double)b4 - 3.1e-6},
+            {64, 8, c64 * unit + 1.13e-6 * (double)b2 - 3.3e-6},
+            {128, 8, c128 * unit + 3.0e-6 * (double)b4 - 3.3e-6},
+        };
+        int best = 0;
+        for (int i = 1; i < 4; ++i)
+            if (forms[i].seconds < forms[best].seconds)
+                best = i;
+        r.rows = forms[best].rows;
+        r.waves = forms[best].waves;
+        // 0.97: where the two models tie (1024 rows on 4096 columns: 256 tiles, one per CU) the tile
+        // kernel was measured level to 10 % behind this launch, never ahead
+        r.seconds = 0.97 * forms[best].seconds;
+    }
     return r;
 }
 

@@ -451,7 +451,25 @@ def test_two_sets_of_waves_where_every_workgroup_has_a_cu(oracle, M, N, K, n, m,
     check_every_tile_once(oracle, M, N, K, n, m, Ns)
 
 
+@pytest.mark.parametrize("M,N,K,n,m,rows", [(620, 4096, 2112, 2, 4, 64), (1280, 2048, 1120, 2, 4, 64), (640, 4096, 4160, 2, 8, 64),
+                                            (600, 4096, 4128, 3, 8, 64), (1270, 2048, 8256, 1, 8, 64), (760, 4096, 6208, 2, 8, 128),
+                                            (750, 4096, 8256, 2, 4, 128), (768, 4096, 6144, 3, 8, 128), (384, 8192, 8192, 2, 8, 128)])
+@pytest.mark.parametrize("Ns", [128, 64, 32])
+def test_eight_waves_along_k_over_several_layers_of_workgroups(oracle, M, N, K, n, m, rows, Ns):
+    """More than two layers of 64-row workgroups on at most 256 tiles: where the pricing of the four
+    forms picks eight waves, a compute unit runs two 64-row or one 128-row workgroup at a time,
+    layer after layer (five 64-row layers, a ragged last row of workgroups, and three layers of
+    128-row ones; window counts that leave the eight waves unequal shares).  Every tile exactly
+    once, every index layout, every width of the column blocks."""
+    window, kept, _ = kernel_geometry(n, m)
+    W = K // window * kept
+    assert nmspmm.waves_along_k_rows(M, N, W, kept) == rows and nmspmm.waves_along_k_count(M, N, W, kept) == 8
+    assert -(-M // 64) * (N // 32) > 2 * nmspmm.device_figures()[0]
+    check_every_tile_once(oracle, M, N, K, n, m, Ns)
+
+
 def test_larger_problems_stay_on_whole_tiles():
+    assert nmspmm.waves_along_k_count(2048, 4096, 2048, 16) == 0
     assert nmspmm.tile_wave_sets(2048, 8192, 512, 16) == 1         # 512 tiles of 256-row waves
     assert nmspmm.tile_wave_sets(2048, 4096, 256, 16) == 1         # 256 kept rows: too short along K
     assert nmspmm.tile_wave_sets(2048, 4096, 1024, 16, 128, 2) == 1
