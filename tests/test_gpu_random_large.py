@@ -30,7 +30,20 @@ def draw_case(rng):
     return M, N, K, n, m, split_k, rng.random() < 0.3, rng.choice([128, 128, 64, 32])
 
 
-CASES = [draw_case(random.Random(SEED + 9000 + i)) for i in range(60)]
+def draw_few_tiles_case(rng):
+    """At most 256 tiles of 128 or 256 rows and a long reduction: the launches with waves along K in
+    their four forms (64 or 128 rows, four or eight waves), whole tiles on two sets of waves."""
+    n, m = rng.choice(list(GEOMETRY))
+    N = 128 * rng.choice([8, 16, 16, 24, 32, 32, 40, 64])
+    M = rng.randint(129, (128 if rng.random() < 0.6 else 256) * (256 // (N // 128)))
+    K = 64 * rng.randint(32, 130)
+    while M * N * K > 3.5e10:
+        K -= 64 * 8
+    return M, N, K, n, m, 1, rng.random() < 0.2, rng.choice([128, 128, 64, 32])
+
+
+CASES = [draw_case(random.Random(SEED + 9000 + i)) for i in range(60)] + \
+        [draw_few_tiles_case(random.Random(SEED + 9500 + i)) for i in range(40)]
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "M%d-N%d-K%d-%dof%d-s%d-%s-Ns%d" % (c[:6] + ("rm" if c[6] else "cm", c[7])))
