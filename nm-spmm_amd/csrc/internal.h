@@ -81,6 +81,16 @@ inline bool tail_along_k(long long tiles, int nwin)
     const long long cus = machine().cus;
     return tiles > cus && tiles <= cus + cus / 4 && nwin >= 8;
 }
+// The same with 65 to 96 tiles after the whole layer: eight workgroups per tile, each 64 rows of
+// one 32-column vector (32 KB of LDS, so that a CU holds the three that fall to it at once).
+// Measured against the 64-row pieces on 60 shapes of 320 to 384 tiles: 5 to 7 % faster at 336 to
+// 352 tiles (2 to 4 % at 1:8; 512 x 11008 x 4096 at 2:8: 93.9 -> 88.3 us), level to 4 % slower at 384
+// (four to a CU), and slower below 16 windows at 1:8.
+inline bool tail_along_k_eighths(long long tiles, int nwin)
+{
+    const long long cus = machine().cus;
+    return tiles > cus + cus / 4 && tiles <= cus + 3 * cus / 8 && nwin >= 16;
+}
 
 // Leftover tiles of 256-row waves (two workgroups per CU) after at least one full round: `rest`
 // tiles, each `unit` seconds of a CU's pipes.  Left in the launch they land packed on the CUs that
@@ -142,6 +152,8 @@ inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks,
         if (full == 0 && layer > 0 && layer <= cus / 2) {
             if (tail_along_k(rest, nwin))  // a quarter of a tile each, one per CU at 0.9 of the rate
                 return (whole + 0.25 / 0.9) * unit + 1e-6;
+            if (tail_along_k_eighths(rest, nwin))  // an eighth of a tile each, three to a CU
+                return (whole + 0.46) * unit + 1e-6;
             return whole == 0 ? lone * unit : (whole + 0.55) * unit;
         }
         if (full >= 1 && rest > 0 && rest <= cus / 2 * slots) {
@@ -196,6 +208,7 @@ struct TailPlan {
     int sub;         // > 1: the tail tiles run as `sub` pieces along M each, on waves of blocks / sub blocks
     size_t ws_bytes; // scratch needed
     bool fused;      // the pieces along M are part of the launch of the whole tiles, after them
+    bool eighths;    // along_k with eight workgroups per tile (64 rows of one 32-column vector each)
     bool along_k;    // fused, and the tail tiles run as four workgroups each (one per 128 rows of one
                      // 32-column vector) whose four waves share the reduction, instead of pieces along M
     bool separate;   // without scratch: give the tail tiles a launch of their own (they then spread
@@ -220,6 +233,7 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
     t.separate = false;
     t.fused = false;
     t.along_k = false;
+    t.eighths = false;
     if (t.blocks == 4 && max_pieces >= 4) {
         // 128-row waves.  Fewer tiles than the CUs hold at once spread one per CU, then two per CU,
         // ..., and the launch lasts as long as the busiest CU: a last layer that covers at most half
@@ -239,7 +253,8 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
         } else if (layer > 0 && layer <= cus / 2) {
             t.tail = layer;
             t.fused = true;
-            t.along_k = tail_along_k(tiles, nwin);
+            t.eighths = tail_along_k_eighths(tiles, nwin);
+            t.along_k = t.eighths || tail_along_k(tiles, nwin);
         } else {
             t.separate = false;
             t.sub = 1;

@@ -533,6 +533,20 @@ __global__ void __launch_bounds__(256, 2) spmm_direct_mixed_inner_kernel(const D
     direct_uniform_launch<KS, WS, QS, WR, 4, HIGH>(p, id);
 }
 
+// The same with eight workgroups per leftover tile, each 64 rows of one 32-column vector (32 KB of
+// LDS: a CU holds several at once).
+template <int KS, int WS, int QS, int WR, bool HIGH>
+__global__ void __launch_bounds__(256, 2) spmm_direct_mixed_eighths_kernel(const DirectParams p)
+{
+    const int id = blockIdx.x;
+    if (id >= p.head_units) {
+        const int u = id - p.head_units;
+        direct_unit<KS, WS, QS, 2 * WR, 2, HIGH, false, 4>(p, p.tail_offset + u / 8, u % 8, 0, false, u);
+        return;
+    }
+    direct_uniform_launch<KS, WS, QS, WR, 4, HIGH>(p, id);
+}
+
 // The first p.head_units workgroups compute whole tiles; the ones after them are the pieces, two
 // per tile along M, of the tiles from p.tail_offset on, computed on waves of RM / 2 blocks.  They
 // are dispatched last and fill the CUs that run out of whole tiles, in pieces fine enough to even
@@ -648,9 +662,13 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
         // along M, so that the pieces fill the CUs more evenly than whole tiles would
         p.tail_offset = (int)plan.head;
         if (plan.along_k) {
-            grid.x = (unsigned)(plan.head + plan.tail * 4);
-            if constexpr (RM == 4)
-                spmm_direct_mixed_inner_kernel<KS, WS, QS, WR, HIGH><<<grid, block, 0, a.stream>>>(p);
+            grid.x = (unsigned)(plan.head + plan.tail * (plan.eighths ? 8 : 4));
+            if constexpr (RM == 4) {
+                if (plan.eighths)
+                    spmm_direct_mixed_eighths_kernel<KS, WS, QS, WR, HIGH><<<grid, block, 0, a.stream>>>(p);
+                else
+                    spmm_direct_mixed_inner_kernel<KS, WS, QS, WR, HIGH><<<grid, block, 0, a.stream>>>(p);
+            }
             return hipGetLastError();
         }
         grid.x = (unsigned)(plan.head + plan.tail * plan.sub);
@@ -769,6 +787,7 @@ static TailPlan tail_plan_for(const SpmmArgs& a, bool have_scratch)
     none.sub = 1;
     none.fused = false;
     none.along_k = false;
+    none.eighths = false;
     if (a.split_k != 1)
         return none;
     TailPlan t = plan_tail(a.M, a.N, a.W / a.kept, a.kept, 128 / a.Ns);
