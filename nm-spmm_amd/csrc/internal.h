@@ -81,15 +81,20 @@ inline bool tail_along_k(long long tiles, int nwin)
     const long long cus = machine().cus;
     return tiles > cus && tiles <= cus + cus / 4 && nwin >= 8;
 }
-// The same with 65 to 96 tiles after the whole layer: eight workgroups per tile, each 64 rows of
-// one 32-column vector (32 KB of LDS, so that a CU holds the three that fall to it at once).
-// Measured against the 64-row pieces on 60 shapes of 320 to 384 tiles: 5 to 7 % faster at 336 to
-// 352 tiles (2 to 4 % at 1:8; 512 x 11008 x 4096 at 2:8: 93.9 -> 88.3 us), level to 4 % slower at 384
-// (four to a CU), and slower below 16 windows at 1:8.
+// With at least sixteen windows the last layer is cut finer: eight workgroups per tile, each 64 rows
+// of one 32-column vector (32 KB of LDS, so that a CU holds the two or three that fall to it at
+// once, next to whole tiles too), for up to 96 tiles after one to three whole layers.  Measured
+// on 108 shapes (2:8, 2:4, 1:8, 3:8): after one whole layer 7 to 10 % faster than the four
+// workgroups per tile with up to 32 tiles left, level to 3 % faster with 48 to 64, and 5 to 7 %
+// faster than the 64-row pieces with 80 to 96 (2 to 4 % at 1:8; 512 x 11008 x 4096 at 2:8: 93.9 ->
+// 88.3 us), level to 4 % slower with 128 (four to a CU); after two and three whole layers 11 to
+// 14 % faster than the pieces with up to 32 tiles left, 4 to 10 % with 48 to 64, 0 to 3 % with 96;
+// below sixteen windows slower at 1:8.  Same sums in the same order as the four per tile.
 inline bool tail_along_k_eighths(long long tiles, int nwin)
 {
     const long long cus = machine().cus;
-    return tiles > cus + cus / 4 && tiles <= cus + 3 * cus / 8 && nwin >= 16;
+    const long long whole = tiles / cus, layer = tiles % cus;
+    return nwin >= 16 && whole >= 1 && whole <= 3 && layer > 0 && layer <= 3 * cus / 8;
 }
 
 // Leftover tiles of 256-row waves (two workgroups per CU) after at least one full round: `rest`
@@ -150,10 +155,10 @@ inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks,
         const double lone = kept <= 8 ? 0.7 : 0.65;
         const long long whole = rest / cus, layer = rest % cus;
         if (full == 0 && layer > 0 && layer <= cus / 2) {
+            if (tail_along_k_eighths(rest, nwin))  // an eighth of a tile each: 0.105 of a tile's time per workgroup of the busiest CU
+                return (whole + 0.105 * (double)((8 * layer + cus - 1) / cus)) * unit + 1e-6;
             if (tail_along_k(rest, nwin))  // a quarter of a tile each, one per CU at 0.9 of the rate
                 return (whole + 0.25 / 0.9) * unit + 1e-6;
-            if (tail_along_k_eighths(rest, nwin))  // an eighth of a tile each, three to a CU
-                return (whole + 0.46) * unit + 1e-6;
             return whole == 0 ? lone * unit : (whole + 0.55) * unit;
         }
         if (full >= 1 && rest > 0 && rest <= cus / 2 * slots) {

@@ -503,15 +503,17 @@ def test_last_layer_of_a_small_launch_with_the_reduction_shared(oracle, M, N, K,
 
 
 @pytest.mark.parametrize("M,N,K,n,m", [(512, 11008, 1056, 2, 4), (1024, 5632, 1088, 2, 8), (1000, 5632, 608, 3, 8), (768, 7168, 1280, 1, 8),
-                                       (1280, 4352, 544, 32, 32)])
+                                       (1280, 4352, 544, 32, 32), (1024, 4352, 608, 3, 8), (1024, 8704, 1088, 2, 8),
+                                       (1024, 12800, 544, 2, 4), (1000, 9216, 1280, 1, 8)])
 @pytest.mark.parametrize("Ns", [128, 64, 32])
 def test_last_layer_of_a_small_launch_as_eighths_of_tiles(oracle, M, N, K, n, m, Ns):
-    """321 to 352 tiles of 128 rows and at least sixteen windows: the tiles beyond the first 256 are
+    """Up to 96 tiles of 128 rows after one, two or three whole layers of 256 (344, 352, 352, 336,
+    340, 272, 544, 800 and 576 tiles) and at least sixteen windows: the tiles of the last layer are
     computed by eight workgroups each at the end of the same launch, 64 rows of one 32-column
-    vector with the reduction shared between the four waves (33, 17, 19, 20 and 17 windows; a
-    ragged row count).  Every tile exactly once, for every width of the column blocks (the whole
-    tile is then 128 x 128, 256 x 64 or 512 x 32; 1280 rows in tiles of 512 give 408 tiles, which
-    take another plan)."""
+    vector with the reduction shared between the four waves (33, 17, 19, 20, 17, 19, 17, 17 and 20
+    windows; ragged row counts).  Every tile exactly once, for every width of the column blocks
+    (the whole tile is then 128 x 128, 256 x 64 or 512 x 32; 1280 rows in tiles of 512 give 408
+    tiles, which take another plan)."""
     window, kept, _ = kernel_geometry(n, m)
     assert nmspmm.tile_wave_rows(M, N, K // window * kept, kept, Ns) == 128 and K // window >= 16
     check_every_tile_once(oracle, M, N, K, n, m, Ns)
