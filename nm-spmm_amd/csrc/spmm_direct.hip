@@ -111,6 +111,9 @@ constexpr bool has_lone_form()
 // K.  With KW > 1 (WR == 1) the workgroup's KW waves compute the same RM*32 rows of ONE 32-column
 // vector, each over its share of the windows, and add their results up through LDS in wave order;
 // QS then only describes the index layout, and the tile walk counts vectors, not column blocks.
+// KH: sets of QS * WR waves per workgroup (1 or 2).  With two, the workgroup computes the same
+// whole tile twice over, each set over half of the windows, and the sets exchange half of their
+// sums through LDS before they store.
 template <int KS, int WS, int QS, int WR, int RM, bool HIGH, bool DEEP = false, int KW = 1, int KH = 1>
 __device__ __forceinline__ void direct_unit(const DirectParams& p, const int logical, const int sub, const int sub_tiles,
                                             const bool tail_unit, const int unit)
