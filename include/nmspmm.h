@@ -132,24 +132,13 @@ int nmspmm_decompress_device(const float* dBT, const int32_t* dDT, int K, int N,
  * split_k partial M x N fp32 results that a second pass sums in a fixed order. */
 size_t nmspmm_workspace_bytes(int M, int N, int split_k);
 
-/* Bytes of optional scratch with which nmspmm_spmm, called with split_k == 1 (sized for Ns == 128;
- * with other widths the scratch is used when it suffices), cuts
- * the few leftover tiles of a ragged last round into four pieces along K so that they occupy four
- * times as many CUs (0 when there is nothing to gain).  The pieces are summed in a fixed order,
- * but not in the order of an unsplit reduction: with the scratch the affected tiles of C may
- * differ from a call without it in the last bits (both within the 1e-4 bound).  Without scratch
- * leftover tiles still get a launch of their own where that pays, whole or in shorter pieces
- * along M, which changes no bit.  No counterpart in the reference. */
-size_t nmspmm_tail_workspace_bytes(int M, int N, int W, int kept);
-
 /* General entry point: C = A . B for one (window, kept, vec_len, Ns) geometry.
  * column_info == NULL selects the low-sparsity layout (all window rows staged), non-NULL the
  * high-sparsity layout (only the rows column_info lists are staged, D holds ranks).
  * split_k > 1 requires `workspace` of at least nmspmm_workspace_bytes(); C is overwritten
  * whatever the split (the reference's atomicAdd reduction, include/ptx.h:34-40, adds to C when
  * SPLIT_K > 1: nmspmm_spmm_ex with NMSPMM_ACCUMULATE does that).  With
- * split_k == 1 the workspace is optional: NULL, or nmspmm_tail_workspace_bytes() bytes (16-byte
- * aligned) that enable the tail split; a smaller one is ignored.
+ * split_k == 1 the workspace is not used and may be NULL.
  * Requirements: N % Ns == 0, Ns % vec_len == 0, W % kept == 0, 1 <= split_k <= W / kept,
  * K * kept == W * window, 16-byte aligned A, B and C. */
 int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t* column_info,

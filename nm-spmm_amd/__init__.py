@@ -58,8 +58,6 @@ def lib():
         L.nmspmm_preprocess_device.argtypes = [c_void_p] + [c_int] * 6 + [c_void_p, c_void_p, ip, ip, c_void_p]
         L.nmspmm_column_info_ints.restype = c_size_t
         L.nmspmm_column_info_ints.argtypes = [c_int] * 5
-        L.nmspmm_tail_workspace_bytes.restype = c_size_t
-        L.nmspmm_tail_workspace_bytes.argtypes = [c_int] * 4
         L.nmspmm_workspace_bytes.restype = c_size_t
         L.nmspmm_workspace_bytes.argtypes = [c_int] * 3
         L.nmspmm_spmm.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_size_t, c_void_p]
@@ -184,10 +182,6 @@ def preprocess_device(dDT_in, n, m, W, Q, N, Ns, dD_out, d_cinfo):
 
 def column_info_ints(W, pN, pM, N, Ns):
     return lib().nmspmm_column_info_ints(W, pN, pM, N, Ns)
-
-
-def tail_workspace_bytes(M, N, W, kept):
-    return lib().nmspmm_tail_workspace_bytes(M, N, W, kept)
 
 
 def workspace_bytes(M, N, split_k):

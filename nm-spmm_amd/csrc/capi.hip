@@ -480,13 +480,6 @@ int nmspmm_decompress_device(const float* dBT, const int32_t* dDT, int K, int N,
                                                                                                      : NMSPMM_ERR_HIP;
 }
 
-size_t nmspmm_tail_workspace_bytes(int M, int N, int W, int kept)
-{
-    if (M <= 128 || N <= 0 || W <= 0 || kept <= 0 || W % kept != 0)
-        return 0;
-    return plan_tail(M, N, W / kept, kept).ws_bytes;
-}
-
 size_t nmspmm_workspace_bytes(int M, int N, int split_k)
 {
     if (M <= 0 || N <= 0 || split_k <= 1)
@@ -555,10 +548,6 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     a.Ns = Ns;
     a.split_k = split_k;
     a.accumulate = (flags & NMSPMM_ACCUMULATE) != 0 && split_k > 1;
-    // without a split the workspace, if any, serves the tail split of the tile kernel
-    const bool scratch = split_k == 1 && workspace != nullptr && aligned16(workspace);
-    a.tail_ws = scratch ? (float*)workspace : nullptr;
-    a.tail_ws_bytes = scratch ? workspace_bytes : 0;
     a.stream = (hipStream_t)stream;
 
     if (lda == 0 && M > 32 && M % 4 != 0) {
@@ -789,9 +778,8 @@ static int named_gemm(int want_high, int tile, const float* A, const float* B, c
         return NMSPMM_ERR_BAD_SHAPE;
     if (split_k < 1 || split_k > W / kept)
         return NMSPMM_ERR_BAD_SPLIT;
-    // Only a split reduction uses the library's per-device workspace.  (The optional scratch that
-    // cuts a few leftover tiles along K, nmspmm_tail_workspace_bytes, is for callers of nmspmm_spmm
-    // who own it: unsplit calls here touch no shared memory and may run on any number of streams.)
+    // Only a split reduction uses the library's per-device workspace: unsplit calls touch no shared
+    // memory and may run on any number of streams.
     void* ws = nullptr;
     const size_t ws_bytes = nmspmm_workspace_bytes(M, N, split_k);
     if (ws_bytes > 0) {

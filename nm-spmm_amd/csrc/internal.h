@@ -32,8 +32,6 @@ struct SpmmArgs {
     int split_k;
     bool accumulate;       // split_k > 1 only: the sum of the slices is added to what C holds (the
                            // reference's atomicAdd reduction, include/ptx.h:34-40) instead of replacing it
-    float* tail_ws;        // optional scratch for splitting the tiles of a ragged last round (split_k == 1)
-    size_t tail_ws_bytes;
     hipStream_t stream;
 };
 
@@ -107,8 +105,13 @@ inline bool tail_along_k_eighths(long long tiles, int nwin)
 // launch costs about 12 us (the gap, and the first launch draining).  Returns the modelled time
 // of the cheapest way and its piece count (0: leave the tiles in the launch).  Over 96 ragged
 // LLM-layer shapes this choice is 4.1 % faster on average than leaving the tiles in the launch
-// (best choice per shape: 4.3 %), up to 30 % on single shapes.
-inline double tall_tail_seconds(long long rest, double unit, int* pieces, int max_pieces = 4)
+// (best choice per shape: 4.3 %), up to 30 % on single shapes.  `pieces` 16 stands for the cut
+// into workgroups of 64 rows of one vector (spmm_direct_units_kernel), measured against the
+// pieces along M on 42 shapes of 16 to 96 leftover tiles (2:8, 1:8, 3:8): 6 to 9 % of the whole
+// multiplication faster with 16 tiles left over, 4 to 8 % with 32, 2 to 5 % with 48, level beyond
+// (4096 x 4224 x 4096 at 2:8: 276.7 -> 252.6 us); the same cut of 128-row tiles into eight
+// (plan_tail), up to 96 tiles left over: 1 to 8 %.
+inline double tall_tail_seconds(long long rest, double unit, int* pieces, int max_pieces = 4, int nwin = 0)
 {
     static const double piece_cost[3] = {1.0, 1.04, 1.2};
     const long long cus = machine().cus;
@@ -120,6 +123,17 @@ inline double tall_tail_seconds(long long rest, double unit, int* pieces, int ma
         if (s < best) {
             best = s;
             best_sub = sub;
+        }
+    }
+    // Or as sixteen workgroups per tile in that launch, each 64 rows of one 32-column vector with the
+    // reduction shared between its four waves (from sixteen windows up; up to four to a CU): 0.13,
+    // 0.21, 0.29 and 0.37 of a tile's time with one to four on the busiest CU.
+    if (max_pieces >= 4 && nwin >= 16 && 16 * rest <= 4 * cus) {
+        const long long busiest = (16 * rest + cus - 1) / cus;
+        const double s = (0.05 + 0.08 * (double)busiest) * unit + 12e-6;
+        if (s < best) {
+            best = s;
+            best_sub = 16;
         }
     }
     if (pieces)
@@ -161,6 +175,12 @@ inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks,
                 return (whole + 0.25 / 0.9) * unit + 1e-6;
             return whole == 0 ? lone * unit : (whole + 0.55) * unit;
         }
+        if (full >= 1 && rest > 0 && 8 * rest <= 3 * cus && nwin >= 16) {
+            // eight workgroups per leftover tile, in a launch of their own (plan_tail): an eighth of a
+            // 128-row tile costs what a sixteenth of a 256-row one does in tall_tail_seconds
+            const long long busiest_unit = (8 * rest + cus - 1) / cus;
+            return (double)full * slots * unit + (0.095 + 0.152 * (double)busiest_unit) * unit + 10e-6;
+        }
         if (full >= 1 && rest > 0 && rest <= cus / 2 * slots) {
             const long long busiest_piece = (2 * rest + cus - 1) / cus;
             return (double)full * slots * unit + (busiest_piece == 1 ? lone : 0.55 * busiest_piece) * unit + 10e-6;
@@ -168,7 +188,7 @@ inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks,
     }
     double t = (double)full * slots * unit;
     if (busiest > 0 && blocks == 8 && split == 1 && full >= 1) {
-        t += tall_tail_seconds(rest, unit, nullptr);  // plan_tail gives these leftovers a launch of shorter pieces
+        t += tall_tail_seconds(rest, unit, nullptr, 4, nwin);  // plan_tail gives these leftovers a launch of shorter pieces
     } else if (busiest > 0) {
         // one workgroup per CU: a 128-row wave alone on its SIMD runs at 0.9 of the rate; a 256-row
         // wave with 16 or more kept rows per chunk keeps its pipe busy by itself (measured 3 to 5 %
@@ -202,22 +222,23 @@ inline int choose_wave_blocks(int M, int N, int nwin, int kept, int split)
 
 // Tail handling of the tile kernel (split_k == 1): the 256 CUs retire 128 x 128 tiles 1024 at a
 // time (256 x 128 tiles 512 at a time); when the last round is ragged, its `tail` tiles get a
-// launch of their own, and with scratch they are also cut into `slices` pieces along K so that they
-// fill the machine once more, written to scratch and summed by a small extra kernel.  A launch of
-// fewer than 1024 128-row tiles has no rounds; its last layer of tiles is cut along M instead.
+// launch of their own, whole, in pieces along M, or as workgroups of 64 rows of one vector that
+// share the reduction between their waves.  A launch of fewer than 1024 128-row tiles has no
+// rounds; its last layer of tiles is cut in the same launch instead.
 struct TailPlan {
     int blocks;      // 32-row blocks per wave (4 or 8)
     long long head;  // tiles computed whole
-    long long tail;  // tiles computed in slices
-    int slices;
+    long long tail;  // tiles computed apart from them
     int sub;         // > 1: the tail tiles run as `sub` pieces along M each, on waves of blocks / sub blocks
-    size_t ws_bytes; // scratch needed
     bool fused;      // the pieces along M are part of the launch of the whole tiles, after them
     bool eighths;    // along_k with eight workgroups per tile (64 rows of one 32-column vector each)
+    bool units;      // the tail tiles run in a launch of their own as `sub` workgroups each, 64 rows of one
+                     // 32-column vector with the reduction shared between the four waves
     bool along_k;    // fused, and the tail tiles run as four workgroups each (one per 128 rows of one
                      // 32-column vector) whose four waves share the reduction, instead of pieces along M
-    bool separate;   // without scratch: give the tail tiles a launch of their own (they then spread
-                     // one or two per CU instead of landing packed on the CUs that free up last)
+    bool separate;   // the tail tiles are planned apart from the whole tiles: in a launch of their own
+                     // (they then spread over the CUs instead of landing packed on the ones that
+                     // free up last) or, fused, as the last workgroups of the same launch
 };
 // `wr`: waves of a workgroup along M (1, 2 or 4 for column blocks of 128, 64 or 32): a tile is
 // 32 * blocks * wr rows x 128 / wr columns.  `max_pieces`: the shortest waves the kernel has,
@@ -232,13 +253,12 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
     const long long slots = cus * (t.blocks == 8 ? 2 : 4);
     t.head = tiles;
     t.tail = 0;
-    t.slices = 1;
     t.sub = 1;
-    t.ws_bytes = 0;
     t.separate = false;
     t.fused = false;
     t.along_k = false;
     t.eighths = false;
+    t.units = false;
     if (t.blocks == 4 && max_pieces >= 4) {
         // 128-row waves.  Fewer tiles than the CUs hold at once spread one per CU, then two per CU,
         // ..., and the launch lasts as long as the busiest CU: a last layer that covers at most half
@@ -255,6 +275,10 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
         t.sub = 2;
         if (tiles >= slots && rest > 0 && rest <= slots / 2) {
             t.tail = rest;  // in a launch of their own: at the end of the first they would land packed too
+            if (8 * rest <= 3 * cus && nwin >= 16) {  // eight workgroups per tile with the reduction shared between the waves
+                t.units = true;
+                t.sub = 8;
+            }
         } else if (layer > 0 && layer <= cus / 2) {
             t.tail = layer;
             t.fused = true;
@@ -273,13 +297,14 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
         return t;
     if (t.blocks == 8) {
         int pieces = 0;
-        tall_tail_seconds(rest, kept * kept_row_seconds() * tall_wave_cost(kept) * nwin, &pieces, max_pieces);
+        tall_tail_seconds(rest, kept * kept_row_seconds() * tall_wave_cost(kept) * nwin, &pieces, max_pieces, nwin);
         if (pieces == 0)
             return t;
         t.separate = true;
         t.head = tiles - rest;
         t.tail = rest;
         t.sub = pieces;
+        t.units = pieces == 16;
     } else {
         // 128-row form of the short-vector kernel (it has no 64-row pieces), four workgroups per
         // CU: the finer grain already fills the last round well after one full round (a launch of
@@ -291,14 +316,6 @@ inline TailPlan plan_tail(int M, int N, int nwin, int kept, int wr = 1, int max_
         t.head = tiles - rest;
         t.tail = rest;
     }
-    // With scratch, a handful of leftover tiles (at most an eighth of the slots) is instead cut into
-    // four pieces along K, so that their launch occupies four times as many CUs for a quarter of
-    // the time.  The pieces pay a second pass: measured +2 % to +5 % up to that size, a loss beyond.
-    if (rest > slots / 8 || nwin / 4 < 4)
-        return t;
-    const int slices = 4;
-    t.slices = slices;
-    t.ws_bytes = (size_t)rest * slices * (32 * t.blocks) * 128 * sizeof(float);
     return t;
 }
 
@@ -481,7 +498,6 @@ inline double model_decode_seconds(int M, int N, int nwin, int kept)
 bool mfma_supported(const SpmmArgs& a);
 hipError_t launch_mfma(const SpmmArgs& a);
 // Scratch bytes with which launch_mfma splits a ragged last round (0: nothing to gain or unsupported).
-size_t mfma_tail_workspace_bytes(const SpmmArgs& a);
 
 // Matrix-core path for index vectors of 4, 8 or 16 columns (spmm_short.hip): low-sparsity layout,
 // windows of 4, 8 or 16 rows, N a multiple of 128, K a multiple of 16.

@@ -48,8 +48,6 @@ struct DirectParams {
     int split_k;
     int tiles_m, tiles_n;
     int tile_offset;     // first logical tile of this launch (the tail tiles may get a launch of their own)
-    int tail_slices;     // > 1: every workgroup of this launch is one of tail_slices pieces of a tile along K
-    float* tail_ws;      // [tile of this launch][slice][MS][NS] partial tiles
     int head_units;      // workgroups of this launch that compute whole tiles (the first ones)
     int tail_offset;     // first logical tile computed in pieces along M by the workgroups after them
     int sub_tiles;       // > 1: every workgroup of this launch is one of sub_tiles pieces, along M, of a
@@ -115,8 +113,7 @@ constexpr bool has_lone_form()
 // whole tile twice over, each set over half of the windows, and the sets exchange half of their
 // sums through LDS before they store.
 template <int KS, int WS, int QS, int WR, int RM, bool HIGH, bool DEEP = false, int KW = 1, int KH = 1>
-__device__ __forceinline__ void direct_unit(const DirectParams& p, const int logical, const int sub, const int sub_tiles,
-                                            const bool tail_unit, const int unit)
+__device__ __forceinline__ void direct_unit(const DirectParams& p, const int logical, const int sub, const int sub_tiles)
 {
     static_assert(RM == 2 || RM == 4 || RM == 8, "64-, 128- or 256-row waves");
     constexpr int IL = RM < 4 ? RM : 4;  // rows interleaved per lane: block b holds rows IL*r + b%IL (+128 for b >= 4)
@@ -153,10 +150,8 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
         split_windows(p.nwin, KW, wave, &w_begin, &w_count);
     else if constexpr (KH > 1)
         split_windows(p.nwin, KH, kh, &w_begin, &w_count);
-    else if (!tail_unit)
-        split_windows(p.nwin, p.split_k, blockIdx.y, &w_begin, &w_count);
     else
-        split_windows(p.nwin, p.tail_slices, unit % p.tail_slices, &w_begin, &w_count);
+        split_windows(p.nwin, p.split_k, blockIdx.y, &w_begin, &w_count);
     const int w_last = w_begin + w_count - 1;
 
     // column vector inside its preprocessed column block, and that block.  With waves along K the
@@ -339,16 +334,13 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
     // column j; block b of the wave holds rows (b/4)*128 + IL*r + b%IL.  Stores go through a
     // descriptor that ends with the last live row of this wave, so rows beyond M are dropped
     // without a branch; the per-register part of the offset is a scalar.
-    // A slice of a tail tile goes to its own MS x NS block of the scratch instead, all rows.
     float* const out = p.out + (size_t)blockIdx.y * p.slice_elems;
-    const int pitch = tail_unit ? NS : N;
-    const int rows_here = tail_unit ? MW : min(M - bi, MW);
-    float* const c_base = tail_unit ? p.tail_ws + ((size_t)unit * MS + wr * MW) * NS + vec * 32
-                                    : out + (size_t)min(bi, M) * N + bj;
-    const uint32_t c_bytes = rows_here > 0 ? (uint32_t)(((size_t)(rows_here - 1) * pitch + 32) * sizeof(float)) : 0u;
+    const int rows_here = min(M - bi, MW);
+    float* const c_base = out + (size_t)min(bi, M) * N + bj;
+    const uint32_t c_bytes = rows_here > 0 ? (uint32_t)(((size_t)(rows_here - 1) * N + 32) * sizeof(float)) : 0u;
     const __amdgpu_buffer_rsrc_t rc = make_rsrc(c_base, c_bytes);
-    const uint32_t c_lane = (uint32_t)(((size_t)4 * IL * h * pitch + j) * sizeof(float));
-    const uint32_t n_bytes = (uint32_t)((size_t)pitch * sizeof(float));
+    const uint32_t c_lane = (uint32_t)(((size_t)4 * IL * h * N + j) * sizeof(float));
+    const uint32_t n_bytes = (uint32_t)((size_t)N * sizeof(float));
     if constexpr (KW > 1) {
         // Waves along K: every wave leaves its sums in LDS, and the groups of four result registers
         // are dealt out to the waves, group g to wave g % KW, which adds the KW partial sums in wave
@@ -450,7 +442,7 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
     }
     typedef std::integral_constant<int, 0> first_block;
     typedef std::integral_constant<int, RM> all_blocks;
-    if (!tail_unit && p.split_k == 1)
+    if (p.split_k == 1)
         store_blocks(std::integral_constant<int, 16>{}, first_block{}, all_blocks{});
     else
         store_blocks(std::integral_constant<int, 0>{}, first_block{}, all_blocks{});
@@ -458,25 +450,22 @@ __device__ __forceinline__ void direct_unit(const DirectParams& p, const int log
 
 // Workgroup `id` of a launch whose workgroups all compute the same kind of unit.  Whole tiles: a
 // walk that gives each XCD (consecutive ids go to different XCDs) a contiguous run of the
-// p.head_units logical tiles.  In a launch of K slices (p.tail_slices > 1) consecutive ids are the
-// slices of one tile, in a launch of pieces along M (p.sub_tiles > 1) the pieces of one tile.
+// p.head_units logical tiles.  In a launch of pieces along M (p.sub_tiles > 1) consecutive ids are
+// the pieces of one tile.
 template <int KS, int WS, int QS, int WR, int RM, bool HIGH, bool DEEP = false, int KW = 1, int KH = 1>
 __device__ __forceinline__ void direct_uniform_launch(const DirectParams& p, const int id)
 {
-    const bool tail_unit = p.tail_slices > 1;
     int logical, sub = 0;
     if (p.sub_tiles > 1) {
         logical = p.tile_offset + id / p.sub_tiles;
         sub = id % p.sub_tiles;
-    } else if (tail_unit) {
-        logical = p.tile_offset + id / p.tail_slices;
     } else {
         const int total = p.head_units;
         const int q = total / p.xcds, r = total % p.xcds;
         const int xcd = id % p.xcds, loc = id / p.xcds;
         logical = p.tile_offset + (xcd < r ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc);
     }
-    direct_unit<KS, WS, QS, WR, RM, HIGH, DEEP, KW, KH>(p, logical, sub, p.sub_tiles, tail_unit, id);
+    direct_unit<KS, WS, QS, WR, RM, HIGH, DEEP, KW, KH>(p, logical, sub, p.sub_tiles);
 }
 
 #define NMSPMM_DIRECT_BOUNDS __launch_bounds__(64 * QS * WR, RM == 8 ? 2 : (HIGH && WS == 16) ? 4 : kWavesPerSimd)
@@ -530,7 +519,7 @@ __global__ void __launch_bounds__(256, 2) spmm_direct_mixed_inner_kernel(const D
     const int id = blockIdx.x;
     if (id >= p.head_units) {
         const int u = id - p.head_units;
-        direct_unit<KS, WS, QS, WR, 4, HIGH, false, 4>(p, p.tail_offset + u / 4, u % 4, 0, false, u);
+        direct_unit<KS, WS, QS, WR, 4, HIGH, false, 4>(p, p.tail_offset + u / 4, u % 4, 0);
         return;
     }
     direct_uniform_launch<KS, WS, QS, WR, 4, HIGH>(p, id);
@@ -544,10 +533,20 @@ __global__ void __launch_bounds__(256, 2) spmm_direct_mixed_eighths_kernel(const
     const int id = blockIdx.x;
     if (id >= p.head_units) {
         const int u = id - p.head_units;
-        direct_unit<KS, WS, QS, 2 * WR, 2, HIGH, false, 4>(p, p.tail_offset + u / 8, u % 8, 0, false, u);
+        direct_unit<KS, WS, QS, 2 * WR, 2, HIGH, false, 4>(p, p.tail_offset + u / 8, u % 8, 0);
         return;
     }
     direct_uniform_launch<KS, WS, QS, WR, 4, HIGH>(p, id);
+}
+
+// Every workgroup is one of the WRU * QS units of a whole tile of the walk over tiles (from
+// p.tail_offset on), 64 rows of one 32-column vector, the reduction shared between its four waves:
+// for the leftover tiles of a launch of several rounds, in a launch of their own.
+template <int KS, int WS, int QS, int WRU, bool HIGH>
+__global__ void __launch_bounds__(256, 2) spmm_direct_units_kernel(const DirectParams p)
+{
+    const int id = blockIdx.x;
+    direct_unit<KS, WS, QS, WRU, 2, HIGH, false, 4>(p, p.tail_offset + id / (WRU * QS), id % (WRU * QS), 0);
 }
 
 // The first p.head_units workgroups compute whole tiles; the ones after them are the pieces, two
@@ -560,44 +559,10 @@ __global__ void NMSPMM_DIRECT_BOUNDS spmm_direct_mixed_kernel(const DirectParams
     const int id = blockIdx.x;
     if (id >= p.head_units) {
         const int u = id - p.head_units;
-        direct_unit<KS, WS, QS, WR, RM / 2, HIGH, DEEP>(p, p.tail_offset + u / 2, u % 2, 2, false, u);
+        direct_unit<KS, WS, QS, WR, RM / 2, HIGH, DEEP>(p, p.tail_offset + u / 2, u % 2, 2);
         return;
     }
     direct_uniform_launch<KS, WS, QS, WR, RM, HIGH, DEEP>(p, id);
-}
-
-// Sums the slices of the tail tiles in slice order into C (second pass of the tail split).  One
-// workgroup per tail tile; the tile is found by the same walk as in the main kernel.
-template <int MS, int NS>
-__global__ void __launch_bounds__(256)
-tail_reduce_kernel(const float* __restrict__ ws, float* __restrict__ C, int M, int N, int tiles_m, int tiles_n,
-                   int head_tiles, int slices)
-{
-    constexpr int GROUP = kBandTiles;
-    const int logical = head_tiles + blockIdx.x;
-    const int band = logical / (GROUP * tiles_n);
-    const int first_m = band * GROUP;
-    const int rows = min(GROUP, tiles_m - first_m);
-    const int in_band = logical - band * GROUP * tiles_n;
-    const int tile_m = first_m + in_band % rows;
-    const int tile_n = in_band / rows;
-    const float* const src = ws + (size_t)blockIdx.x * slices * MS * NS;
-    constexpr int F4_ROW = NS / 4;
-    for (int e = threadIdx.x; e < MS * F4_ROW; e += 256) {
-        const int r = e / F4_ROW, c4 = e % F4_ROW;
-        const int row = tile_m * MS + r;
-        if (row >= M)
-            break;  // rows grow with e
-        float4 sum = reinterpret_cast<const float4*>(src)[e];
-        for (int z = 1; z < slices; ++z) {
-            const float4 v = reinterpret_cast<const float4*>(src + (size_t)z * MS * NS)[e];
-            sum.x += v.x;
-            sum.y += v.y;
-            sum.z += v.z;
-            sum.w += v.w;
-        }
-        *reinterpret_cast<float4*>(C + (size_t)row * N + (size_t)tile_n * NS + c4 * 4) = sum;
-    }
 }
 
 // One launch of uniform workgroups.  A launch of at most one workgroup per CU (each wave alone on
@@ -647,8 +612,6 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     p.tiles_m = (a.M + MS - 1) / MS;
     p.tiles_n = a.N / NS;
     p.tile_offset = 0;
-    p.tail_slices = 1;
-    p.tail_ws = nullptr;
     p.tail_offset = 0;
     p.sub_tiles = 1;
     p.xcds = machine().xcds;
@@ -660,7 +623,7 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     if (!own_tail)
         return launch_uniform<KS, WS, QS, WR, RM, HIGH>(grid, block, a.stream, p, true);
     p.head_units = (int)plan.head;
-    if (plan.slices == 1 && plan.sub > 1 && plan.fused) {
+    if (plan.sub > 1 && plan.fused) {
         // shorter waves for the leftovers, in the same launch: each leftover tile in two pieces
         // along M, so that the pieces fill the CUs more evenly than whole tiles would
         p.tail_offset = (int)plan.head;
@@ -683,16 +646,25 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
         }
         return hipGetLastError();
     }
-    // head tiles, then the leftover tiles in a launch of their own, whole or in slices along K
+    // head tiles, then the leftover tiles in a launch of their own
     grid.x = (unsigned)plan.head;
     hipError_t e = launch_uniform<KS, WS, QS, WR, RM, HIGH>(grid, block, a.stream, p);
     if (e != hipSuccess)
         return e;
     p.tile_offset = (int)plan.head;
-    if (plan.slices == 1 && plan.sub > 1) {
+    if (plan.units) {
+        // 64 rows of one 32-column vector per workgroup, the reduction shared between its four waves
+        p.tail_offset = (int)plan.head;
+        grid.x = (unsigned)(plan.tail * plan.sub);
+        p.head_units = (int)grid.x;
+        if constexpr (RM >= 4)
+            spmm_direct_units_kernel<KS, WS, QS, WR * RM / 2, HIGH><<<grid, dim3(256), 0, a.stream>>>(p);
+        return hipGetLastError();
+    }
+    if (plan.sub > 1) {
         // shorter waves for the leftovers, in a launch of the kernel built for such waves (which
         // more workgroups per CU can run): each tile in plan.sub pieces along M; same sums in the
-        // same order as whole tiles, no scratch
+        // same order as whole tiles
         p.sub_tiles = plan.sub;
         grid.x = (unsigned)(plan.tail * plan.sub);
         p.head_units = (int)grid.x;
@@ -705,17 +677,9 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
         }
         return hipErrorInvalidValue;
     }
-    p.tail_slices = plan.slices;
-    p.tail_ws = plan.slices > 1 ? a.tail_ws : nullptr;
-    grid.x = (unsigned)(plan.tail * plan.slices);
+    grid.x = (unsigned)plan.tail;  // whole tiles
     p.head_units = (int)grid.x;
-    e = launch_uniform<KS, WS, QS, WR, RM, HIGH>(grid, block, a.stream, p);
-    if (e == hipSuccess && plan.slices > 1) {
-        tail_reduce_kernel<MS, NS><<<dim3((unsigned)plan.tail), dim3(256), 0, a.stream>>>(
-            a.tail_ws, a.C, a.M, a.N, p.tiles_m, p.tiles_n, (int)plan.head, plan.slices);
-        e = hipGetLastError();
-    }
-    return e;
+    return launch_uniform<KS, WS, QS, WR, RM, HIGH>(grid, block, a.stream, p);
 }
 
 // The launch with four waves along K (spmm_direct_inner_kernel), on 128- or 64-row tiles as
@@ -744,8 +708,6 @@ static hipError_t launch_inner(const SpmmArgs& a)
     p.tiles_m = (a.M + rows - 1) / rows;
     p.tiles_n = (int)vecs;
     p.tile_offset = 0;
-    p.tail_slices = 1;
-    p.tail_ws = nullptr;
     p.tail_offset = 0;
     p.sub_tiles = 1;
     p.xcds = machine().xcds;
@@ -777,29 +739,23 @@ static hipError_t launch_inner(const SpmmArgs& a)
 // column-block width the indices were preprocessed for.  A wave is 256 or 128 rows tall, whichever
 // the run-time model expects to finish first: the taller wave halves the B and index loads per
 // MFMA, but only two such workgroups fit a CU, which quantises badly on mid-sized problems.
-// The tail handling is planned for a single reduction slice; its cut along K is used when the
-// caller's scratch holds it.
-static TailPlan tail_plan_for(const SpmmArgs& a, bool have_scratch)
+// The tail handling is planned for a single reduction slice.
+static TailPlan tail_plan_for(const SpmmArgs& a)
 {
     TailPlan none;
     none.blocks = choose_wave_blocks(a.M, a.N, a.W / a.kept, a.kept, a.split_k);
     none.head = none.tail = 0;
-    none.slices = 1;
-    none.ws_bytes = 0;
     none.separate = false;
     none.sub = 1;
     none.fused = false;
     none.along_k = false;
     none.eighths = false;
+    none.units = false;
     if (a.split_k != 1)
         return none;
     TailPlan t = plan_tail(a.M, a.N, a.W / a.kept, a.kept, 128 / a.Ns);
-    if (t.head + t.tail * t.slices * t.sub > 0x7fffffffLL)
+    if (t.head + t.tail * t.sub > 0x7fffffffLL)
         return none;
-    if (have_scratch && t.slices > 1 && (a.tail_ws == nullptr || a.tail_ws_bytes < t.ws_bytes)) {
-        t.slices = 1;  // no scratch: the tail can still have a launch of its own
-        t.ws_bytes = 0;
-    }
     return t;
 }
 
@@ -813,7 +769,7 @@ static hipError_t launch_ns(const SpmmArgs& a)
         case 32: return launch_inner<KS, WS, 1, HIGH>(a);
         }
     }
-    const TailPlan plan = tail_plan_for(a, true);
+    const TailPlan plan = tail_plan_for(a);
     const bool tall = plan.blocks == 8;
     if (!tall && a.Ns == 128 && short_waves_pay(a.M))
         return launch_cfg<KS, WS, 4, 1, 2, HIGH>(a, plan);
@@ -826,11 +782,6 @@ static hipError_t launch_ns(const SpmmArgs& a)
         return tall ? launch_cfg<KS, WS, 1, 4, 8, HIGH>(a, plan) : launch_cfg<KS, WS, 1, 4, 4, HIGH>(a, plan);
     }
     return hipErrorInvalidValue;
-}
-
-size_t mfma_tail_workspace_bytes(const SpmmArgs& a)
-{
-    return mfma_supported(a) ? tail_plan_for(a, false).ws_bytes : 0;
 }
 
 bool mfma_supported(const SpmmArgs& a)
