@@ -623,6 +623,16 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
     if (!own_tail)
         return launch_uniform<KS, WS, QS, WR, RM, HIGH>(grid, block, a.stream, p, true);
     p.head_units = (int)plan.head;
+    if (plan.units && RM == 4) {
+        // eight workgroups per leftover tile, dispatched after the whole tiles in the same launch (the
+        // 128-row kernel's register allocation lets a CU hold four of them): against a launch of
+        // their own 0 to 4 % faster at 1:8, -4 to +2 % at 2:8 and 3:8, more on short reductions
+        p.tail_offset = (int)plan.head;
+        grid.x = (unsigned)(plan.head + plan.tail * plan.sub);
+        if constexpr (RM == 4)
+            spmm_direct_mixed_eighths_kernel<KS, WS, QS, WR, HIGH><<<grid, block, 0, a.stream>>>(p);
+        return hipGetLastError();
+    }
     if (plan.sub > 1 && plan.fused) {
         // shorter waves for the leftovers, in the same launch: each leftover tile in two pieces
         // along M, so that the pieces fill the CUs more evenly than whole tiles would
@@ -653,12 +663,13 @@ static hipError_t launch_cfg(const SpmmArgs& a, const TailPlan& plan)
         return e;
     p.tile_offset = (int)plan.head;
     if (plan.units) {
-        // 64 rows of one 32-column vector per workgroup, the reduction shared between its four waves
+        // (256-row waves) sixteen workgroups per leftover tile in a launch of their own, 64 rows of one
+        // 32-column vector each, the reduction shared between its four waves
         p.tail_offset = (int)plan.head;
         grid.x = (unsigned)(plan.tail * plan.sub);
         p.head_units = (int)grid.x;
-        if constexpr (RM >= 4)
-            spmm_direct_units_kernel<KS, WS, QS, WR * RM / 2, HIGH><<<grid, dim3(256), 0, a.stream>>>(p);
+        if constexpr (RM == 8)
+            spmm_direct_units_kernel<KS, WS, QS, 4 * WR, HIGH><<<grid, dim3(256), 0, a.stream>>>(p);
         return hipGetLastError();
     }
     if (plan.sub > 1) {
