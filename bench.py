@@ -11,6 +11,8 @@ Prints ONE JSON line:
   sweep            3:8, 2:8, 1:8 beside 2:4: ms, useful TFLOP/s, speedup over the dense fp32 GEMM
   configs          the baseline's other workloads, each timed in this run:
                      llm     nine prefill-sized LLM-layer shapes at 2:8 against the dense fp32 GEMM
+                     ragged  eight shapes whose tiles do not fill whole rounds of the compute
+                             units, one per way the tile kernel cuts the leftovers
                      decode  M in {1, 8, 16, 32} x two weight shapes x {1:8, 2:8}: microseconds and
                              algorithmic GB/s against the 8 TB/s HBM bound, with B re-read from the
                              caches ("hot") and streamed from HBM ("cold"), row list on and off
@@ -47,7 +49,7 @@ M = N = K = 4096
 PATTERNS = [(2, 4), (3, 8), (2, 8), (1, 8)]  # first one is the headline
 NS = 128
 GEOMETRY = {(1, 1): (32, 32), (1, 2): (32, 16), (3, 8): (32, 12), (1, 4): (64, 16), (1, 8): (64, 8)}
-PARTS = ("sweep", "llm", "decode", "decode_llm", "decode_wide", "fine", "ksweep", "compress", "rowmajor", "preprocess", "dispatch", "cpu")
+PARTS = ("sweep", "llm", "ragged", "decode", "decode_llm", "decode_wide", "fine", "ksweep", "compress", "rowmajor", "preprocess", "dispatch", "cpu")
 
 
 def geometry(n, m):
@@ -271,6 +273,41 @@ def run_llm(torch, pkg):
                          "dense_ms": round(dms, 4), "speedup_vs_dense": round(dms / ms, 2),
                          "speedup_over_ideal": round(dms / ms / 4.0, 3)})
             del op, a, b
+    return rows
+
+
+# Shapes whose tile counts do not fill whole rounds of the 256 compute units, one per way the tile
+# kernel cuts the leftovers: (M, Ncols, K, n, m, what the launch is)
+RAGGED_SHAPES = (
+    (768, 4096, 14336, 2, 8, "192 tiles of 128 x 128: waves along K, three layers of 128-row workgroups on eight waves"),
+    (640, 4096, 8192, 2, 4, "160 tiles: waves along K, five layers of 64-row workgroups on eight waves"),
+    (2048, 4096, 8192, 2, 4, "256 tiles of 256 x 128, one per compute unit: two sets of waves per workgroup"),
+    (1024, 4352, 4096, 2, 8, "272 tiles of 128 rows: the last 16 as eight workgroups each in the same launch"),
+    (1024, 8704, 4096, 1, 8, "544 tiles of 128 rows, two whole layers: the last 32 as eight workgroups each"),
+    (4096, 4224, 4096, 2, 8, "528 tiles of 256 rows: the 16 beyond one round as sixteen workgroups each, in a launch of their own"),
+    (1152, 14848, 4096, 3, 8, "1044 tiles of 128 rows: the 20 beyond one round as eight workgroups each at the end of the launch"),
+    (2048, 11008, 4096, 2, 4, "688 tiles of 256 rows: the 176 beyond one round as 64-row pieces in a launch of their own"),
+)
+
+
+def run_ragged(torch, pkg):
+    """Unsplit multiplications of shapes with leftover tiles; `of_even` compares the useful rate with
+    the headline shape's (4096 cubed at the same pattern is not timed here: the fraction of the fp32
+    MFMA peak is the common scale)."""
+    rows = []
+    for (m_rows, n_cols, k, n, m, what) in RAGGED_SHAPES:
+        op = GpuOperands(torch, pkg, m_rows, n_cols, k, n, m)
+        call = lambda: pkg.spmm(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k, op.W, op.window, op.kept, 32, NS, 1, None)
+        ms, _ = time_launches(torch, call, 30, 5, 0.2)
+        useful = op.flops() / ms / 1e9
+        rows.append({"M": m_rows, "K": k, "Ncols": n_cols, "pattern": "%d:%d" % (n, m), "kernel": pkg.last_kernel(),
+                     "launch": what, "tile_wave_rows": pkg.tile_wave_rows(m_rows, n_cols, op.W, op.kept, NS, 1),
+                     "tile_wave_sets": pkg.tile_wave_sets(m_rows, n_cols, op.W, op.kept, NS, 1),
+                     "waves_along_k": [pkg.waves_along_k_rows(m_rows, n_cols, op.W, op.kept),
+                                       pkg.waves_along_k_count(m_rows, n_cols, op.W, op.kept)],
+                     "ms": round(ms, 4), "useful_tflops": round(useful, 1),
+                     "frac_fp32_mfma_peak": round(useful / FP32_MFMA_PEAK_TFLOPS, 3)})
+        del op
     return rows
 
 
@@ -624,6 +661,8 @@ def main():
     configs = {}
     if "llm" in parts:
         configs["llm"] = run_llm(torch, pkg)
+    if "ragged" in parts:
+        configs["ragged"] = run_ragged(torch, pkg)
     if "decode" in parts:
         configs["decode"] = run_decode(
             torch, pkg, tuple(int(x) for x in args.decode_rows.split(",")),
