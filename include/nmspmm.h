@@ -278,6 +278,11 @@ int nmspmm_waves_along_k_rows(int M, int N, int W, int kept);
  * compute unit holds half as many workgroups, each with twice the waves), 0 where
  * nmspmm_waves_along_k_rows returns 0.  Informational. */
 int nmspmm_waves_along_k_count(int M, int N, int W, int kept);
+/* No counterpart in the reference.  Rows that an unsplit multiplication of this shape on the
+ * matrix-core kernel hands to the decode-sized kernels: the last 1 to 32 rows of a row count a
+ * little above a multiple of 128, where the library expects the tile kernel's extra layer of
+ * 128-row workgroups to cost more than reading B once more; 0 otherwise.  Informational. */
+int nmspmm_rows_apart(int M, int N, int W, int kept);
 /* No counterpart in the reference.  What the library's planning (split choice, wave height, tile
  * walk) assumes about the current device: compute units, accelerator dies (each with its own L2)
  * and shader clock, read from the HIP runtime once per device; the figures of an MI355X
@@ -303,7 +308,8 @@ int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int
 int nmspmm_release(void);
 
 /* Name of the kernel family the last successful nmspmm_spmm call on this thread dispatched to
- * ("mfma", "short", "gather", "skinny", "decode", "simt"), for tests and profiles.  Never NULL. */
+ * ("mfma", "short", "gather", "skinny", "decode", "simt"), for tests and profiles; where a call
+ * hands its last 1 to 32 rows to another family than the rest, the family of the rest.  Never NULL. */
 const char* nmspmm_last_kernel(void);
 
 #ifdef __cplusplus

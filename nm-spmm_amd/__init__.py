@@ -76,6 +76,7 @@ def lib():
         L.nmspmm_suggest_split_k.argtypes = [c_int] * 4
         L.nmspmm_waves_along_k_rows.argtypes = [c_int] * 4
         L.nmspmm_waves_along_k_count.argtypes = [c_int] * 4
+        L.nmspmm_rows_apart.argtypes = [c_int] * 4
         L.nmspmm_tile_wave_rows.argtypes = [c_int] * 6
         L.nmspmm_tile_wave_sets.argtypes = [c_int] * 6
         L.nmspmm_device_figures.argtypes = [ip, ip, ctypes.POINTER(ctypes.c_double)]
@@ -271,6 +272,11 @@ def waves_along_k_rows(M, N, W, kept):
     """128 or 64 when an unsplit multiplication of this shape shares the reduction between the
     waves of a workgroup, 0 otherwise."""
     return lib().nmspmm_waves_along_k_rows(M, N, W, kept)
+
+
+def rows_apart(M, N, W, kept):
+    """Last rows (1 to 32) that an unsplit tile-kernel call of this shape hands to the decode-sized kernels, else 0."""
+    return lib().nmspmm_rows_apart(M, N, W, kept)
 
 
 def waves_along_k_count(M, N, W, kept):

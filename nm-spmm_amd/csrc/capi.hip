@@ -563,6 +563,35 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
 
     if (a_rowmajor && !(M <= 32 && (skinny_supported(a) || decode_supported(a))))
         return kNotTaken;
+    // A row count a little above a multiple of 128 (1 to 32 rows more): the tile kernel would spend a
+    // whole layer of 128-row workgroups, mostly padding, on the last rows.  Where the models expect
+    // it to be shorter, the rows up to the multiple go to the tile kernel and the last ones to the
+    // kernels with one workgroup per vector, which read B once more at the rate of HBM.  The
+    // comparison allows 3 us for what the two models both count.  Measured on 140 shapes (136 to 416
+    // rows, 2048 to 11008 columns, four patterns) with the two parts launched by hand: the rule is
+    // 0.8 % behind the better way on average where whole launches are 6.1 % behind (136 x 4096 x
+    // 11008 at 2:4: 83.2 -> 67.4 us; on 2048 columns, where the last rows add no layer, the whole
+    // launch stays).  With eight kept rows per window the two ways were within 2 us of each other
+    // nearly everywhere and the models cannot tell them apart: whole launches there.  Every row of C
+    // is computed by one kernel, in its own order.
+    const int last_rows = a_rowmajor || split_k != 1 || !mfma_supported(a) ? 0 : nmspmm_rows_apart(M, N, W, kept);
+    if (last_rows > 0) {
+        SpmmArgs tail = a;
+        tail.M = last_rows;
+        const bool tail_ok = (row_index && decode_supported(tail)) || skinny_supported(tail);
+        const int head_rows = M - last_rows;
+        if (tail_ok) {
+            int st = spmm_impl(A, B, D, column_info, C, head_rows, N, K, W, window, kept, vec_len, Ns, 1, nullptr, 0,
+                               stream, a.lda, false, nullptr, false, flags, row_index);
+            if (st != NMSPMM_OK)
+                return st;
+            const char* const head_kernel = g_last_kernel;
+            st = spmm_impl(A + head_rows, B, D, column_info, C + (size_t)head_rows * N, last_rows, N, K, W, window, kept,
+                           vec_len, Ns, 1, nullptr, 0, stream, a.lda, false, nullptr, false, flags, row_index);
+            g_last_kernel = head_kernel;  // the family that computed all rows but the last few
+            return st;
+        }
+    }
     hipError_t e;
     // up to 32 rows the kernels with one workgroup per vector always win; up to 128 they compete
     // with the tile kernel at the caller's split.  The two models are compared with a bias: on 340
@@ -835,6 +864,19 @@ int nmspmm_waves_along_k_rows(int M, int N, int W, int kept)
     if (M <= 0 || N <= 0 || W <= 0 || kept <= 0 || W % kept != 0)
         return 0;
     return inner_split_pays(M, N, W / kept, kept) ? plan_inner(M, N, W / kept, kept).rows : 0;
+}
+
+int nmspmm_rows_apart(int M, int N, int W, int kept)
+{
+    if (M <= 128 || N <= 0 || W <= 0 || kept < 12 || W % kept != 0)
+        return 0;
+    const int last_rows = M % 128, nwin = W / kept;
+    if (last_rows < 1 || last_rows > 32)
+        return 0;
+    return model_tile_seconds(M - last_rows, N, nwin, kept, 1) + model_decode_seconds(last_rows, N, nwin, kept) - 3e-6 <
+                   model_tile_seconds(M, N, nwin, kept, 1)
+               ? last_rows
+               : 0;
 }
 
 int nmspmm_waves_along_k_count(int M, int N, int W, int kept)

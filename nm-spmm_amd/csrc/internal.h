@@ -497,7 +497,6 @@ inline double model_decode_seconds(int M, int N, int nwin, int kept)
 // Matrix-core path (spmm_direct.hip).  Returns false when the geometry has no instantiation.
 bool mfma_supported(const SpmmArgs& a);
 hipError_t launch_mfma(const SpmmArgs& a);
-// Scratch bytes with which launch_mfma splits a ragged last round (0: nothing to gain or unsupported).
 
 // Matrix-core path for index vectors of 4, 8 or 16 columns (spmm_short.hip): low-sparsity layout,
 // windows of 4, 8 or 16 rows, N a multiple of 128, K a multiple of 16.

@@ -78,6 +78,21 @@ def test_wave_sets_of_the_tile_kernel():
     assert nmspmm.tile_wave_sets(0, 4096, 1024, 16) == 0 and nmspmm.tile_wave_sets(64, 4096, 1000, 16) == 0
 
 
+def test_rows_apart():
+    """The last rows of a row count a little above a multiple of 128 go to the decode-sized kernels only
+    where an extra layer of 128-row workgroups is expected to cost more than reading B again."""
+    import torch
+    if torch.cuda.is_available() and nmspmm.device_figures()[0] != 256:
+        pytest.skip("the shapes below are sized for 256 compute units")
+    assert nmspmm.rows_apart(136, 4096, 1024, 16) == 8          # 4096 columns, K = 2048 at 2:4
+    assert nmspmm.rows_apart(288, 8192, 512, 16) == 32
+    assert nmspmm.rows_apart(136, 2048, 1024, 16) == 0          # both row tiles fit one layer of workgroups
+    assert nmspmm.rows_apart(136, 4096, 512, 8) == 0            # eight kept rows per window: never
+    assert nmspmm.rows_apart(168, 4096, 1024, 16) == 0          # 40 rows above the multiple
+    assert nmspmm.rows_apart(128, 4096, 1024, 16) == 0 and nmspmm.rows_apart(100, 4096, 1024, 16) == 0
+    assert nmspmm.rows_apart(136, 4096, 1000, 16) == 0          # invalid: W is not a multiple of kept
+
+
 def test_pattern_table():
     assert nmspmm.pattern_from_sparsity(0.0) == (32, 32, False)
     assert nmspmm.pattern_from_sparsity(0.5) == (32, 16, False)

@@ -305,3 +305,33 @@ def test_the_split_flag_changes_nothing_where_every_compute_unit_has_a_vector(or
     nmspmm.spmm_ex(A, B, Dd, ci, C2, M, N, K, W, window, kept, 32, 128, 1, None, nmspmm.DECODE_SPLIT, R)
     torch.cuda.synchronize()
     assert torch.equal(C1, C2)
+
+
+@pytest.mark.parametrize("M,N,K,n,m", [(136, 4096, 2048, 2, 4), (137, 4096, 4096, 2, 4), (150, 4096, 2048, 32, 32), (160, 4096, 4096, 2, 8),
+                                       (280, 8192, 2048, 3, 8), (288, 8192, 2048, 2, 8)])
+@pytest.mark.parametrize("with_list", [False, True])
+@pytest.mark.parametrize("Ns", [128, 32])
+def test_last_rows_of_a_tile_kernel_call_on_the_decode_sized_kernels(oracle, M, N, K, n, m, with_list, Ns):
+    """Row counts 8 to 32 above a multiple of 128 where the library expects an extra layer of 128-row
+    workgroups to cost more than reading B again: the rows up to the multiple run on the tile kernel,
+    the last ones on the decode kernel (with the row list) or the kernel on the reference layout
+    (without).  Every row against the checker, the seam included; nothing outside C's M rows is
+    written."""
+    d = datagen.init_data(M, N, K, n, m, seed=M + N + K)
+    W = d["W"]
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, Ns)
+    apart = nmspmm.rows_apart(M, N, W, kept)
+    assert 8 <= apart <= 32 and apart == M % 128
+    R = gpu_row_list(D, cinfo, W, N, window, kept, Ns) if with_list else None
+    guard = 64
+    Cbuf = torch.full(((M + guard) * N,), float("nan"), dtype=torch.float32, device="cuda")
+    C = Cbuf[: M * N].view(M, N)
+    nmspmm.spmm_ex(dev(d["A_km"]), dev(d["BT"]), dev(D), None if cinfo is None else dev(cinfo), C, M, N, K, W, window,
+                   kept, 32, Ns, 1, None, 0, R)
+    torch.cuda.synchronize()
+    assert nmspmm.last_kernel() in ("mfma", "skinny", "decode")
+    assert bool(torch.isfinite(C).all()) and bool(torch.isnan(Cbuf[M * N:]).all())
+    want = oracle.gemm_cpu(d["A_km"].reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), M, N, W).reshape(M, N)
+    assert scaled_max_error(C.cpu().numpy(), want) <= REL_TOL
+    assert scaled_max_error(C[M - apart:].cpu().numpy(), want[M - apart:]) <= REL_TOL
+
