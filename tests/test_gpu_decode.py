@@ -335,3 +335,19 @@ def test_last_rows_of_a_tile_kernel_call_on_the_decode_sized_kernels(oracle, M, 
     assert scaled_max_error(C.cpu().numpy(), want) <= REL_TOL
     assert scaled_max_error(C[M - apart:].cpu().numpy(), want[M - apart:]) <= REL_TOL
 
+
+@pytest.mark.parametrize("M,N,K,n,m", [(137, 4096, 4096, 2, 4), (150, 4096, 2048, 32, 32), (281, 8192, 2048, 3, 8)])
+def test_last_rows_apart_with_row_major_activations(oracle, M, N, K, n, m):
+    """The same hand-over behind the row-major entry point: the copy of A has a pitch of M rounded up
+    to four floats, and the last rows start 128 or 256 floats into each of its rows."""
+    d = datagen.init_data(M, N, K, n, m, seed=M + N)
+    W = d["W"]
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    assert nmspmm.rows_apart(M, N, W, kept) == M % 128
+    X = dev(np.ascontiguousarray(d["A_km"].reshape(K, M).T))                         # M x K, K contiguous
+    ws = torch.empty(nmspmm.workspace_bytes_rowmajor(M, N, K, 1) // 4, dtype=torch.float32, device="cuda")
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    nmspmm.spmm_rowmajor(X, dev(d["BT"]), dev(D), None if cinfo is None else dev(cinfo), C, M, N, K, W, window, kept, ws)
+    torch.cuda.synchronize()
+    assert scaled_max_error(C.cpu().numpy(), want_c(oracle, d)) <= REL_TOL
+
