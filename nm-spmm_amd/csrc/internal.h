@@ -176,10 +176,10 @@ inline double model_kernel_seconds(int M, int N, int nwin, int kept, int blocks,
             return whole == 0 ? lone * unit : (whole + 0.55) * unit;
         }
         if (full >= 1 && rest > 0 && 8 * rest <= 3 * cus && nwin >= 16) {
-            // eight workgroups per leftover tile, in a launch of their own (plan_tail): an eighth of a
-            // 128-row tile costs what a sixteenth of a 256-row one does in tall_tail_seconds
+            // eight workgroups per leftover tile at the end of the launch (plan_tail): 0.2, 0.35 and 0.5
+            // of a tile's time with one, two and three on the busiest CU (measured after one round)
             const long long busiest_unit = (8 * rest + cus - 1) / cus;
-            return (double)full * slots * unit + (0.095 + 0.152 * (double)busiest_unit) * unit + 10e-6;
+            return (double)full * slots * unit + (0.05 + 0.15 * (double)busiest_unit) * unit + 1e-6;
         }
         if (full >= 1 && rest > 0 && rest <= cus / 2 * slots) {
             const long long busiest_piece = (2 * rest + cus - 1) / cus;
@@ -232,8 +232,9 @@ struct TailPlan {
     int sub;         // > 1: the tail tiles run as `sub` pieces along M each, on waves of blocks / sub blocks
     bool fused;      // the pieces along M are part of the launch of the whole tiles, after them
     bool eighths;    // along_k with eight workgroups per tile (64 rows of one 32-column vector each)
-    bool units;      // the tail tiles run in a launch of their own as `sub` workgroups each, 64 rows of one
-                     // 32-column vector with the reduction shared between the four waves
+    bool units;      // leftovers after full rounds run as `sub` workgroups each, 64 rows of one 32-column
+                     // vector with the reduction shared between the four waves: in a launch of their
+                     // own after 256-row waves, at the end of the same launch after 128-row waves
     bool along_k;    // fused, and the tail tiles run as four workgroups each (one per 128 rows of one
                      // 32-column vector) whose four waves share the reduction, instead of pieces along M
     bool separate;   // the tail tiles are planned apart from the whole tiles: in a launch of their own
