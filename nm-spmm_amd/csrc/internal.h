@@ -130,7 +130,7 @@ inline double tall_tail_seconds(long long rest, double unit, int* pieces, int ma
     // 0.21, 0.29 and 0.37 of a tile's time with one to four on the busiest CU.
     if (max_pieces >= 4 && nwin >= 16 && 16 * rest <= 4 * cus) {
         const long long busiest = (16 * rest + cus - 1) / cus;
-        const double s = (0.05 + 0.08 * (double)busiest) * unit + 12e-6;
+        const double s = (0.05 + 0.08 * (double)busiest) * unit + 1e-6;  // their launch starts while the first drains
         if (s < best) {
             best = s;
             best_sub = 16;
