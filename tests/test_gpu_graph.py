@@ -54,3 +54,38 @@ def test_graph_replays_equal_eager_calls(oracle, M, n, m, split_k, row_major):
         torch.cuda.synchronize()
         assert torch.isfinite(C_g).all().item()
         assert torch.equal(C_g, C_e), "replay %d" % rep
+
+
+def test_graph_replays_of_a_call_that_hands_its_last_rows_over(oracle):
+    """136 rows on 4096 columns: the tile kernel computes 128 rows and the kernel on the reference
+    layout the other eight, two launches that a graph holds like any other."""
+    M, N, K, n, m = 136, 4096, 2048, 2, 4
+    d = datagen.init_data(M, N, K, n, m, seed=M, dist="normal", b_scale=0.02)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    W = d["W"]
+    assert nmspmm.rows_apart(M, N, W, kept) == 8
+    A, B, Dd = dev(d["A_km"]), dev(d["BT"]), dev(D)
+    C_g = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    C_e = torch.empty_like(C_g)
+
+    def call(C):
+        nmspmm.spmm(A, B, Dd, None, C, M, N, K, W, window, kept, 32, 128, 1, None)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(C_g)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(C_g)
+    for rep in range(3):
+        A.mul_(1.25)
+        C_g.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        call(C_e)
+        torch.cuda.synchronize()
+        assert torch.isfinite(C_g).all().item()
+        assert torch.equal(C_g, C_e), "replay %d" % rep
+
