@@ -383,9 +383,11 @@ inline InnerPlan plan_inner(int M, int N, int nwin, int kept)
     // holds four of them and the few workgroups left after a full round of 1024 land packed on
     // the CUs that free up first (+0.38 and +0.12 with up to one and two layers left), on eight
     // waves it holds two and ends evenly.  128-row workgroups cost 0.95 a layer plus 0.155 per
-    // workgroup; on four waves an odd layer runs one wave per SIMD (+0.22), on eight waves every
-    // layer has two, for 1.5 us more per layer (the exchange between eight waves through 128 KB of
-    // LDS).  The choice lands within 0.3 % of the best form on average (2.2 % before, when only
+    // workgroup; on four waves an odd layer runs one wave per SIMD (+0.22 with B in the caches, +0.6
+    // to +0.8 with B streamed from HBM, which a single wave per SIMD hides badly: priced at 0.35,
+    // which costs 0.2 % with B in the caches and halves the distance to the best form with B from
+    // HBM, 1.1 -> 0.5 % on 51 shapes), on eight waves every layer has two, for 1.5 us more per layer
+    // (the exchange between eight waves through 128 KB of LDS).  The choice lands within 0.3 % of the best form on average (2.2 % before, when only
     // the two four-wave forms were priced; 768 x 4096 x 14336 at 2:8: 194 -> 169 us, 640 x 4096 x
     // 8192 at 2:4: 189 -> 170 us).  Up to 128 rows the earlier pricing stays (the choice between this
     // kernel and the ones for few rows was fitted against it), and below 32 windows, where the fixed
@@ -398,7 +400,7 @@ inline InnerPlan plan_inner(int M, int N, int nwin, int kept)
         const double packed = left > 0.0 && left <= 1.0 ? 0.38 : left > 1.0 && left <= 2.0 ? 0.12 : 0.0;
         const double c64 = 0.60 * layers2;
         const double c128 = 0.95 * (double)b4 + 0.155 * q4;
-        const double odd = b4 % 2 == 1 && b4 >= 3 ? 0.22 : 0.0;
+        const double odd = b4 % 2 == 1 && b4 >= 3 ? 0.35 : 0.0;
         struct Form { int rows, waves; double seconds; };
         const Form forms[4] = {
             {64, 4, (c64 + packed) * unit + 0.67e-6 * (double)b2 - 3.8e-6},
