@@ -10,7 +10,8 @@ Prints ONE JSON line:
   cpu_baseline     the reference project's own nmGEMM_on_cpu (oracle/_ref) on a row slice
   sweep            3:8, 2:8, 1:8 beside 2:4: ms, useful TFLOP/s, speedup over the dense fp32 GEMM
   configs          the baseline's other workloads, each timed in this run:
-                     llm     nine prefill-sized LLM-layer shapes at 2:8 against the dense fp32 GEMM
+                     llm     nine prefill-sized LLM-layer shapes at 2:8 against the dense fp32 GEMM,
+                             with B re-read from the caches and with B streamed from HBM
                      ragged  eight shapes whose tiles do not fill whole rounds of the compute
                              units, one per way the tile kernel cuts the leftovers
                      decode  M in {1, 8, 16, 32} x two weight shapes x {1:8, 2:8}: microseconds and
@@ -262,13 +263,24 @@ def run_llm(torch, pkg):
             ms, _ = time_launches(torch, lambda: pkg.gemm_auto(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k,
                                                                op.W, 0.75), 30, 5, 0.2)
             fam = pkg.last_kernel()
+            # the same with every launch on another copy of B, more than 640 MB in all: every byte of
+            # B then comes from HBM, as in a model whose layers do not fit the caches
+            copies = [op.B] + [op.B.clone() for _ in range(int(640e6 // (op.B.numel() * 4)))]
+            turn = [0]
+
+            def from_hbm():
+                turn[0] = (turn[0] + 1) % len(copies)
+                pkg.gemm_auto(op.A, copies[turn[0]], op.D, op.cinfo, op.C, m_rows, n_cols, k, op.W, 0.75)
+
+            cold_ms, _ = time_launches(torch, from_hbm, 3 * len(copies), len(copies), 0.1)
+            del copies
             a = op.A.t().contiguous()
             b = torch.randn((k, n_cols), dtype=torch.float32, device="cuda")
             dms, _ = time_launches(torch, lambda: torch.mm(a, b, out=op.C), 20, 3, 0.2)
             useful = op.flops() / ms / 1e9
             rows.append({"M": m_rows, "K": k, "Ncols": n_cols, "pattern": "2:8", "kernel": fam, "split_k": split,
                          "waves_along_k_rows": pkg.waves_along_k_rows(m_rows, n_cols, op.W, op.kept),
-                         "ms": round(ms, 4), "useful_tflops": round(useful, 1),
+                         "ms": round(ms, 4), "ms_b_from_hbm": round(cold_ms, 4), "useful_tflops": round(useful, 1),
                          "frac_fp32_mfma_peak": round(useful / FP32_MFMA_PEAK_TFLOPS, 3),
                          "dense_ms": round(dms, 4), "speedup_vs_dense": round(dms / ms, 2),
                          "speedup_over_ideal": round(dms / ms / 4.0, 3)})
