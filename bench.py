@@ -253,6 +253,20 @@ def profiled_traffic():
     return (float(m.group(1)), os.path.relpath(path, ROOT)) if m else (None, None)
 
 
+def time_b_from_hbm(torch, B, call):
+    """Milliseconds per call(b) with every launch on another copy of B, more than 640 MB in all:
+    every byte of B then comes from HBM, as in a model whose layers do not fit the caches."""
+    copies = [B] + [B.clone() for _ in range(int(640e6 // (B.numel() * 4)))]
+    turn = [0]
+
+    def step():
+        turn[0] = (turn[0] + 1) % len(copies)
+        call(copies[turn[0]])
+
+    ms, _ = time_launches(torch, step, 3 * len(copies), len(copies), 0.1)
+    return ms
+
+
 def run_llm(torch, pkg):
     """Config 3: nine prefill-sized layer shapes at 2:8, the library's own split, against torch.mm fp32."""
     rows = []
@@ -263,17 +277,8 @@ def run_llm(torch, pkg):
             ms, _ = time_launches(torch, lambda: pkg.gemm_auto(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k,
                                                                op.W, 0.75), 30, 5, 0.2)
             fam = pkg.last_kernel()
-            # the same with every launch on another copy of B, more than 640 MB in all: every byte of
-            # B then comes from HBM, as in a model whose layers do not fit the caches
-            copies = [op.B] + [op.B.clone() for _ in range(int(640e6 // (op.B.numel() * 4)))]
-            turn = [0]
-
-            def from_hbm():
-                turn[0] = (turn[0] + 1) % len(copies)
-                pkg.gemm_auto(op.A, copies[turn[0]], op.D, op.cinfo, op.C, m_rows, n_cols, k, op.W, 0.75)
-
-            cold_ms, _ = time_launches(torch, from_hbm, 3 * len(copies), len(copies), 0.1)
-            del copies
+            cold_ms = time_b_from_hbm(torch, op.B, lambda b: pkg.gemm_auto(op.A, b, op.D, op.cinfo, op.C, m_rows, n_cols, k,
+                                                                           op.W, 0.75))
             a = op.A.t().contiguous()
             b = torch.randn((k, n_cols), dtype=torch.float32, device="cuda")
             dms, _ = time_launches(torch, lambda: torch.mm(a, b, out=op.C), 20, 3, 0.2)
@@ -311,13 +316,15 @@ def run_ragged(torch, pkg):
         op = GpuOperands(torch, pkg, m_rows, n_cols, k, n, m)
         call = lambda: pkg.spmm(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k, op.W, op.window, op.kept, 32, NS, 1, None)
         ms, _ = time_launches(torch, call, 30, 5, 0.2)
+        cold_ms = time_b_from_hbm(torch, op.B, lambda b: pkg.spmm(op.A, b, op.D, op.cinfo, op.C, m_rows, n_cols, k, op.W,
+                                                                  op.window, op.kept, 32, NS, 1, None))
         useful = op.flops() / ms / 1e9
         rows.append({"M": m_rows, "K": k, "Ncols": n_cols, "pattern": "%d:%d" % (n, m), "kernel": pkg.last_kernel(),
                      "launch": what, "tile_wave_rows": pkg.tile_wave_rows(m_rows, n_cols, op.W, op.kept, NS, 1),
                      "tile_wave_sets": pkg.tile_wave_sets(m_rows, n_cols, op.W, op.kept, NS, 1),
                      "waves_along_k": [pkg.waves_along_k_rows(m_rows, n_cols, op.W, op.kept),
                                        pkg.waves_along_k_count(m_rows, n_cols, op.W, op.kept)],
-                     "ms": round(ms, 4), "useful_tflops": round(useful, 1),
+                     "ms": round(ms, 4), "ms_b_from_hbm": round(cold_ms, 4), "useful_tflops": round(useful, 1),
                      "frac_fp32_mfma_peak": round(useful / FP32_MFMA_PEAK_TFLOPS, 3)})
         del op
     return rows
