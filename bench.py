@@ -388,8 +388,8 @@ def run_decode(torch, pkg, rows_list=(1, 8, 16, 32), shapes=((8192, 8192), (4096
 def run_fine(torch, pkg, cases):
     """Config 5: the n:32 patterns and 2:4 with 4-column vectors at 4096 cubed, with the device
     preprocessing time of each (one launch for 32-column vectors, the re-blocking launch for
-    shorter ones); beyond the baseline's list, 2:8 and 1:8 with 4-column vectors and 1:8 with
-    8-column ones."""
+    shorter ones); beyond the baseline's list, 2:8 and 1:8 with 4-column vectors, 1:8 with
+    8-column ones, and the dense pattern 32:32 (the reference's geometry for a sparsity of 0)."""
     out = []
     for (n, m, vl) in cases:
         op = GpuOperands(torch, pkg, M, N, K, n, m, vec_len=vl, normal=False)
@@ -600,7 +600,7 @@ def main():
     ap.add_argument("--decode-patterns", default="1:8,2:8", help="patterns of the decode part")
     ap.add_argument("--decode-modes", default=",".join(DECODE_DEFAULT_MODES),
                     help="which of " + ", ".join(m[0] for m in DECODE_MODES) + " to time")
-    ap.add_argument("--fine-cases", default="4:32x32,8:32x32,16:32x32,2:4x4,2:8x4,1:8x4,1:8x8",
+    ap.add_argument("--fine-cases", default="4:32x32,8:32x32,16:32x32,2:4x4,2:8x4,1:8x4,1:8x8,32:32x32",
                     help="cases of the fine part, n:m x vector length")
     ap.add_argument("--ksweep-ks", default="64,1024,4096", help="reduction lengths of the ksweep part")
     ap.add_argument("--ksweep-patterns", default="2:4,1:8,4:32", help="patterns of the ksweep part")

@@ -59,6 +59,7 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
         assert x["kernel"] == "decode" and x["hot_split"]["us"] > 0 and x["cold_split"]["us"] > 0
     assert len(cfg["decode_wide"]) == 8 and all(x["kernel"] in ("decode", "mfma") and x["M"] in (48, 64) for x in cfg["decode_wide"])
     assert [x["pattern"] for x in cfg["fine"]][:4] == ["4:32", "8:32", "16:32", "2:4"] and cfg["fine"][3]["vec_len"] == 4
+    assert cfg["fine"][-1]["pattern"] == "32:32" and cfg["fine"][-1]["kernel"] == "mfma"
     assert len(cfg["launch_constant"]) == 3 and len(cfg["compress"]) == 12 and len(cfg["rowmajor"]) == 5
     for x in d["preprocess"]:
         assert x["host_pointer_dropin_wall_ms"] > 0 and x["cpu_restatement_wall_ms"] > 0
