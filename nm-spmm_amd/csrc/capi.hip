@@ -571,9 +571,10 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     // rows, 2048 to 11008 columns, four patterns) with the two parts launched by hand: the rule is
     // 0.8 % behind the better way on average where whole launches are 6.1 % behind (136 x 4096 x
     // 11008 at 2:4: 83.2 -> 67.4 us; on 2048 columns, where the last rows add no layer, the whole
-    // launch stays).  With eight kept rows per window the two ways were within 2 us of each other
-    // nearly everywhere and the models cannot tell them apart: whole launches there.  Every row of C
-    // is computed by one kernel, in its own order.
+    // launch stays).  With eight kept rows per window and fewer than 512 rows the two ways were
+    // within 2 us of each other nearly everywhere and the models cannot tell them apart: whole
+    // launches there (from 512 rows on the rule's choices were 1 to 10 % shorter on 15 of 17 shapes
+    // and 1 % longer on two).  Every row of C is computed by one kernel, in its own order.
     const int last_rows = a_rowmajor || split_k != 1 || !mfma_supported(a) ? 0 : nmspmm_rows_apart(M, N, W, kept);
     if (last_rows > 0) {
         SpmmArgs tail = a;
@@ -868,7 +869,9 @@ int nmspmm_waves_along_k_rows(int M, int N, int W, int kept)
 
 int nmspmm_rows_apart(int M, int N, int W, int kept)
 {
-    if (M <= 128 || N <= 0 || W <= 0 || kept < 12 || W % kept != 0)
+    if (M <= 128 || N <= 0 || W <= 0 || kept <= 0 || W % kept != 0)
+        return 0;
+    if (kept < 12 && M < 512)  // eight kept rows per window: the models only tell the two ways apart from 512 rows on
         return 0;
     const int last_rows = M % 128, nwin = W / kept;
     if (last_rows < 1 || last_rows > 32)

@@ -87,7 +87,8 @@ def test_rows_apart():
     assert nmspmm.rows_apart(136, 4096, 1024, 16) == 8          # 4096 columns, K = 2048 at 2:4
     assert nmspmm.rows_apart(288, 8192, 512, 16) == 32
     assert nmspmm.rows_apart(136, 2048, 1024, 16) == 0          # both row tiles fit one layer of workgroups
-    assert nmspmm.rows_apart(136, 4096, 512, 8) == 0            # eight kept rows per window: never
+    assert nmspmm.rows_apart(136, 4096, 512, 8) == 0            # eight kept rows per window: only from 512 rows on
+    assert nmspmm.rows_apart(520, 11008, 512, 8) == 8
     assert nmspmm.rows_apart(168, 4096, 1024, 16) == 0          # 40 rows above the multiple
     assert nmspmm.rows_apart(128, 4096, 1024, 16) == 0 and nmspmm.rows_apart(100, 4096, 1024, 16) == 0
     assert nmspmm.rows_apart(136, 4096, 1000, 16) == 0          # invalid: W is not a multiple of kept

@@ -308,7 +308,7 @@ def test_the_split_flag_changes_nothing_where_every_compute_unit_has_a_vector(or
 
 
 @pytest.mark.parametrize("M,N,K,n,m", [(136, 4096, 2048, 2, 4), (137, 4096, 4096, 2, 4), (150, 4096, 2048, 32, 32), (160, 4096, 4096, 2, 8),
-                                       (280, 8192, 2048, 3, 8), (288, 8192, 2048, 2, 8)])
+                                       (280, 8192, 2048, 3, 8), (288, 8192, 2048, 2, 8), (520, 11008, 4096, 1, 8)])
 @pytest.mark.parametrize("with_list", [False, True])
 @pytest.mark.parametrize("Ns", [128, 32])
 def test_last_rows_of_a_tile_kernel_call_on_the_decode_sized_kernels(oracle, M, N, K, n, m, with_list, Ns):
