@@ -12,8 +12,8 @@ Prints ONE JSON line:
   configs          the baseline's other workloads, each timed in this run:
                      llm     nine prefill-sized LLM-layer shapes at 2:8 against the dense fp32 GEMM,
                              with B re-read from the caches and with B streamed from HBM
-                     ragged  eight shapes whose tiles do not fill whole rounds of the compute
-                             units, one per way the tile kernel cuts the leftovers
+                     ragged  nine shapes whose tiles do not fill whole rounds of the compute
+                             units, one per way the library cuts the leftovers
                      decode  M in {1, 8, 16, 32} x two weight shapes x {1:8, 2:8}: microseconds and
                              algorithmic GB/s against the 8 TB/s HBM bound, with B re-read from the
                              caches ("hot") and streamed from HBM ("cold"), row list on and off
@@ -304,6 +304,7 @@ RAGGED_SHAPES = (
     (4096, 4224, 4096, 2, 8, "528 tiles of 256 rows: the 16 beyond one round as sixteen workgroups each, in a launch of their own"),
     (1152, 14848, 4096, 3, 8, "1044 tiles of 128 rows: the 20 beyond one round as eight workgroups each at the end of the launch"),
     (2048, 11008, 4096, 2, 4, "688 tiles of 256 rows: the 176 beyond one round as 64-row pieces in a launch of their own"),
+    (160, 4096, 11008, 3, 8, "160 rows: 128 on the tile kernel (waves along K), the last 32 on the kernel with one workgroup per vector"),
 )
 
 
@@ -320,7 +321,8 @@ def run_ragged(torch, pkg):
                                                                   op.window, op.kept, 32, NS, 1, None))
         useful = op.flops() / ms / 1e9
         rows.append({"M": m_rows, "K": k, "Ncols": n_cols, "pattern": "%d:%d" % (n, m), "kernel": pkg.last_kernel(),
-                     "launch": what, "tile_wave_rows": pkg.tile_wave_rows(m_rows, n_cols, op.W, op.kept, NS, 1),
+                     "launch": what, "rows_apart": pkg.rows_apart(m_rows, n_cols, op.W, op.kept),
+                     "tile_wave_rows": pkg.tile_wave_rows(m_rows, n_cols, op.W, op.kept, NS, 1),
                      "tile_wave_sets": pkg.tile_wave_sets(m_rows, n_cols, op.W, op.kept, NS, 1),
                      "waves_along_k": [pkg.waves_along_k_rows(m_rows, n_cols, op.W, op.kept),
                                        pkg.waves_along_k_count(m_rows, n_cols, op.W, op.kept)],

@@ -45,7 +45,7 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     cfg = d["configs"]
     assert len(cfg["llm"]) == 9 and all(x["kernel"] == "mfma" and x["speedup_vs_dense"] > 1 for x in cfg["llm"])
     assert all(0.9 * x["ms"] < x["ms_b_from_hbm"] < 1.5 * x["ms"] for x in cfg["llm"])
-    assert len(cfg["ragged"]) == 8 and all(x["kernel"] == "mfma" and 0.5 < x["frac_fp32_mfma_peak"] < 1 for x in cfg["ragged"])
+    assert len(cfg["ragged"]) == 9 and cfg["ragged"][8]["rows_apart"] == 32 and all(x["kernel"] == "mfma" and 0.5 < x["frac_fp32_mfma_peak"] < 1 for x in cfg["ragged"])
     assert all(0.9 * x["ms"] < x["ms_b_from_hbm"] < 1.5 * x["ms"] for x in cfg["ragged"])
     assert cfg["ragged"][0]["waves_along_k"] == [128, 8] and cfg["ragged"][1]["waves_along_k"] == [64, 8]
     assert cfg["ragged"][2]["tile_wave_sets"] == 2 and cfg["ragged"][5]["tile_wave_rows"] == 256
