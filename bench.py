@@ -50,7 +50,8 @@ M = N = K = 4096
 PATTERNS = [(2, 4), (3, 8), (2, 8), (1, 8)]  # first one is the headline
 NS = 128
 GEOMETRY = {(1, 1): (32, 32), (1, 2): (32, 16), (3, 8): (32, 12), (1, 4): (64, 16), (1, 8): (64, 8)}
-PARTS = ("sweep", "llm", "ragged", "decode", "decode_llm", "decode_wide", "fine", "ksweep", "compress", "rowmajor", "preprocess", "dispatch", "cpu")
+PARTS = ("sweep", "llm", "ragged", "decode", "decode_llm", "decode_wide", "fine", "ksweep", "compress", "rowmajor", "preprocess", "dispatch", "cpu", "sweep100")
+OPT_IN_PARTS = ("sweep100",)   # several minutes: run by name only
 
 
 def geometry(n, m):
@@ -267,6 +268,19 @@ def time_b_from_hbm(torch, B, call):
     return ms
 
 
+def rate_entry(us, nbytes, from_hbm, digits):
+    """Microseconds and algorithmic GB/s of one launch.  Only a launch whose operands come from HBM
+    is set against the HBM peak; one that re-reads what the previous launch left in the 256 MB
+    Infinity Cache is labelled so and carries no fraction."""
+    gbs = nbytes / us / 1e3
+    e = {"us": round(us, digits), "gbs": round(gbs, 0)}
+    if from_hbm:
+        e["frac_hbm"] = round(gbs / HBM_PEAK_GBS, 3)
+    else:
+        e["served_by"] = "infinity cache"
+    return e
+
+
 def run_llm(torch, pkg):
     """Config 3: nine prefill-sized layer shapes at 2:8, the library's own split, against torch.mm fp32."""
     rows = []
@@ -379,8 +393,7 @@ def run_decode(torch, pkg, rows_list=(1, 8, 16, 32), shapes=((8192, 8192), (4096
                         entry["kernel"] = pkg.last_kernel()
                     elif label == "hot_reference_layout":
                         entry["kernel_reference_layout"] = pkg.last_kernel()
-                    entry[label] = {"us": round(ms * 1e3, 2), "gbs": round(alg / ms / 1e6, 0),
-                                    "frac_hbm": round(alg / ms / 1e6 / HBM_PEAK_GBS, 3)}
+                    entry[label] = rate_entry(ms * 1e3, alg, cold, 2)
                 out.append(entry)
                 del a, c
             del op, copies
@@ -449,10 +462,27 @@ def run_compress(torch, pkg):
             for name, fn in (("compress", lambda: pkg.compress_device(dense, k, n_cols, n, m, bt, dt)),
                              ("decompress", lambda: pkg.decompress_device(bt, dt, k, n_cols, n, m, back))):
                 ms, _ = time_launches(torch, fn, 30, 5, 0.05)
-                row[name] = {"us": round(ms * 1e3, 1), "gbs": round(nbytes / ms / 1e6, 0),
-                             "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 3)}
+                row[name + "_hot"] = rate_entry(ms * 1e3, nbytes, False, 1)
+            # cold: every launch on another set of buffers, more than 640 MB touched between two
+            # uses of the same one, so that neither the input nor the output sits in a cache
+            sets = [(dense, bt, dt, back)]
+            for _ in range(int(640e6 // nbytes) + 1):
+                sets.append(tuple(t.clone() for t in sets[0]))
+            turn = [0]
+
+            def step(which):
+                turn[0] = (turn[0] + 1) % len(sets)
+                de, b_, d_, ba = sets[turn[0]]
+                if which == "compress":
+                    pkg.compress_device(de, k, n_cols, n, m, b_, d_)
+                else:
+                    pkg.decompress_device(b_, d_, k, n_cols, n, m, ba)
+
+            for name in ("compress", "decompress"):
+                ms, _ = time_launches(torch, lambda: step(name), 3 * len(sets), len(sets), 0.05)
+                row[name] = rate_entry(ms * 1e3, nbytes, True, 1)
             out.append(row)
-            del bt, dt, back
+            del bt, dt, back, sets
         del dense
     return out
 
@@ -554,6 +584,52 @@ def run_preprocess(torch, pkg, datagen):
     return out
 
 
+# The reference's kernel-performance sweep (benchmark/kernel_performance/run_test/nmspmm/run_nmspmm.sh:16-18):
+# five row counts x twenty (Ncols, K) pairs, at the n:32 patterns of its four sparsities (:29)
+SWEEP100_M = (256, 512, 1024, 2048, 4096)
+SWEEP100_N = (2048, 6144, 2048, 5632, 4096, 12288, 4096, 11008, 5120, 15360, 5120, 13824, 6656, 19968, 6656, 17920, 8192,
+              24576, 8192, 22016)
+SWEEP100_K = (2048, 2048, 5632, 2048, 4096, 4096, 11008, 4096, 5120, 5120, 13824, 5120, 6656, 6656, 17920, 6656, 8192,
+              8192, 22016, 8192)
+# mean speed-up over cuBLAS fp32 on the A100 over the same 100 shapes, from the reference's
+# benchmark/kernel_performance/result_data/{nmspmm_a100_*,cublas_a100}.txt
+SWEEP100_A100_MEAN = {"0.5": 1.83, "0.625": 2.38, "0.75": 3.46, "0.875": 6.34}
+
+
+def run_sweep100(torch, pkg):
+    """The 100 shapes of the reference's sweep at 50, 62.5, 75 and 87.5 % (16:32, 12:32, 8:32, 4:32):
+    the library's own choice of kernel and split (the reference takes the best of four tiles and
+    four splits by brute force, run_nmspmm.sh:19-36) against torch.mm fp32 of the same shape.  Line
+    20*mi + i of each list is M[mi] with (Ncols, K)[i], as in the reference's result files."""
+    by = {}
+    dense_ms = []
+    for m_rows in SWEEP100_M:
+        for n_cols, k in zip(SWEEP100_N, SWEEP100_K):
+            a = torch.randn((m_rows, k), dtype=torch.float32, device="cuda")
+            b = torch.randn((k, n_cols), dtype=torch.float32, device="cuda")
+            c = torch.empty((m_rows, n_cols), dtype=torch.float32, device="cuda")
+            ms, _ = time_launches(torch, lambda: torch.mm(a, b, out=c), 10, 2, 0.05)
+            dense_ms.append(ms)
+            del a, b, c
+    for kept, label in ((16, "0.5"), (12, "0.625"), (8, "0.75"), (4, "0.875")):
+        rows, idx = [], 0
+        for m_rows in SWEEP100_M:
+            for n_cols, k in zip(SWEEP100_N, SWEEP100_K):
+                op = GpuOperands(torch, pkg, m_rows, n_cols, k, kept, 32, normal=False)
+                ms, _ = time_launches(torch, lambda: pkg.gemm_auto(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k,
+                                                                   op.W, float(label)), 10, 2, 0.05)
+                rows.append({"M": m_rows, "Ncols": n_cols, "K": k, "ms": round(ms, 4), "dense_ms": round(dense_ms[idx], 4),
+                             "dense_equiv_tflops": round(2.0 * m_rows * n_cols * k / ms / 1e9, 2),
+                             "speedup_vs_dense": round(dense_ms[idx] / ms, 3)})
+                idx += 1
+                del op
+        sp = [r["speedup_vs_dense"] for r in rows]
+        by[label] = {"pattern": "%d:32" % kept, "shapes": len(rows), "mean_speedup_vs_dense": round(float(np.mean(sp)), 3),
+                     "min_speedup_vs_dense": min(sp), "max_speedup_vs_dense": max(sp),
+                     "a100_reference_mean_speedup": SWEEP100_A100_MEAN[label], "rows": rows}
+    return {"dense": "torch.mm fp32 (rocBLAS/hipBLASLt)", "by_sparsity": by}
+
+
 def run_dispatch(torch, pkg):
     """The library's own choice (nmspmm_gemm_auto: split from its run-time model, kernel from the
     shape) against the best of the splits 1, 2, 4, 8 of nmspmm_spmm, on shapes from the reference's
@@ -588,6 +664,62 @@ def run_dispatch(torch, pkg):
     return {"shapes": rows, "mean_ratio": round(float(np.mean(ratios)), 3), "worst_ratio": round(float(np.max(ratios)), 3)}
 
 
+MAX_LINE_BYTES = 4096
+
+
+def digest(rows, value, name, higher_is_better=True):
+    """[cases, min, median, max, worst case] of value(row) over the rows."""
+    vals = [(value(r), name(r)) for r in rows]
+    nums = sorted(v for v, _ in vals)
+    worst = (min if higher_is_better else max)(vals)
+    return {"n": len(rows), "min": nums[0], "med": round(float(np.median(nums)), 3), "max": nums[-1], "worst": worst[1]}
+
+
+def summarize(configs, preprocess, dispatch):
+    """One short digest per workload for the printed line; every case is in the detail file."""
+    shape = lambda r: "%dx%dx%d %s" % (r["M"], r["Ncols"], r["K"], r["pattern"])
+    s = {}
+    for key in ("llm", "ragged"):
+        if key in configs:
+            s[key] = {"frac_fp32_mfma_peak": digest(configs[key], lambda r: r["frac_fp32_mfma_peak"], shape)}
+    if "llm" in configs:
+        s["llm"]["speedup_over_ideal_4x"] = digest(configs["llm"], lambda r: r["speedup_over_ideal"], shape)
+    for key in ("decode", "decode_llm", "decode_wide"):
+        if key not in configs:
+            continue
+        s[key] = {}
+        for mode in ("hot", "cold", "cold_reference_layout", "hot_split", "cold_split"):
+            rows = [r for r in configs[key] if mode in r]
+            if not rows:
+                continue
+            if "frac_hbm" in rows[0][mode]:     # B streamed from HBM
+                s[key][mode + "_frac_hbm"] = digest(rows, lambda r: r[mode]["frac_hbm"], shape)
+            else:                               # B re-read from the Infinity Cache: a rate, no HBM fraction
+                s[key][mode + "_gbs"] = digest(rows, lambda r: r[mode]["gbs"], shape)
+    if "fine" in configs:
+        s["fine_frac_fp32_mfma_peak"] = {"%sx%d" % (r["pattern"], r["vec_len"]): r["frac_fp32_mfma_peak"]
+                                         for r in configs["fine"]}
+    if "launch_constant" in configs:
+        s["launch_constant_us"] = {r["pattern"]: r.get("constant_us") for r in configs["launch_constant"]}
+    if "compress" in configs:
+        name = lambda r: "%dx%d %s" % (r["K"], r["Ncols"], r["pattern"])
+        s["compress_frac_hbm"] = digest(configs["compress"], lambda r: r["compress"]["frac_hbm"], name)
+        s["decompress_frac_hbm"] = digest(configs["compress"], lambda r: r["decompress"]["frac_hbm"], name)
+    if "rowmajor" in configs:
+        s["rowmajor_overhead"] = digest(configs["rowmajor"], lambda r: r["overhead"], shape, higher_is_better=False)
+    if "sweep100" in configs:
+        s["sweep100"] = {k: {f: v[f] for f in ("shapes", "mean_speedup_vs_dense", "min_speedup_vs_dense",
+                                               "a100_reference_mean_speedup")}
+                         for k, v in configs["sweep100"]["by_sparsity"].items()}
+    if preprocess:
+        s["preprocess_device_ms"] = {"%sx%d" % (r["pattern"], r["vec_len"]): r["device_one_kernel_ms"] for r in preprocess}
+        s["preprocess_cpu_ms"] = {"%sx%d" % (r["pattern"], r["vec_len"]): r.get("cpu_reference_wall_ms", r["cpu_restatement_wall_ms"])
+                                  for r in preprocess}
+    if dispatch:
+        s["dispatch"] = {"n": len(dispatch["shapes"]), "mean_ratio": dispatch["mean_ratio"], "worst_ratio": dispatch["worst_ratio"]}
+    return s
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -606,6 +738,8 @@ def main():
                     help="cases of the fine part, n:m x vector length")
     ap.add_argument("--ksweep-ks", default="64,1024,4096", help="reduction lengths of the ksweep part")
     ap.add_argument("--ksweep-patterns", default="2:4,1:8,4:32", help="patterns of the ksweep part")
+    ap.add_argument("--detail", default=os.path.join(ROOT, "bench_detail.json"),
+                    help="file that receives every case of every part (the printed line holds digests)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy 5 times (known traffic, to scale rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters)")
@@ -613,7 +747,7 @@ def main():
     if args.gpus != 1:
         print("bench.py: this library is a single-GPU kernel library; run with --gpus 1", file=sys.stderr)
         return 2
-    parts = set(PARTS) if not args.only else set(p for p in args.only.split(",") if p and p != "none")
+    parts = (set(PARTS) - set(OPT_IN_PARTS)) if not args.only else set(p for p in args.only.split(",") if p and p != "none")
     if args.headline_only:
         parts = set()
     if args.cpu_rows <= 0:
@@ -707,6 +841,8 @@ def main():
         configs["compress"] = run_compress(torch, pkg)
     if "rowmajor" in parts:
         configs["rowmajor"] = run_rowmajor(torch, pkg)
+    if "sweep100" in parts:
+        configs["sweep100"] = run_sweep100(torch, pkg)
     preprocess = run_preprocess(torch, pkg, datagen) if "preprocess" in parts else None
     dispatch = run_dispatch(torch, pkg) if "dispatch" in parts else None
 
@@ -731,11 +867,23 @@ def main():
         "cpu_baseline": cpu,
         "dense_fp32_gemm": dense,
         "sweep": sweep,
-        "configs": configs,
-        "preprocess": preprocess,
-        "dispatch": dispatch,
     }
-    print(json.dumps(out))
+    detail = dict(out, configs=configs, preprocess=preprocess, dispatch=dispatch)
+    with open(args.detail, "w") as f:
+        json.dump(detail, f, indent=1)
+        f.write("\n")
+    # the line itself stays short (harnesses keep only the last few KB of a run's output): the
+    # headline fields whole, one digest per other workload, every case in the detail file
+    out["sweep"] = {k: {f: v[f] for f in ("ms", "useful_tflops", "frac_fp32_mfma_peak", "speedup_vs_dense")}
+                    for k, v in sweep.items()}
+    out["summary"] = summarize(configs, preprocess, dispatch)
+    out["detail_file"] = os.path.relpath(args.detail, ROOT) if os.path.abspath(args.detail).startswith(ROOT) else args.detail
+    line = json.dumps(out, separators=(",", ":"))
+    while len(line) > MAX_LINE_BYTES and out["summary"]:   # never at today's part list; the headline fields stay whatever happens
+        out["summary"].popitem()
+        out["summary_truncated"] = True
+        line = json.dumps(out, separators=(",", ":"))
+    print(line)
     return 0
 
 

@@ -132,6 +132,12 @@ def last_kernel():
     return lib().nmspmm_last_kernel().decode()
 
 
+def release():
+    """Frees what the library keeps per device (cached workspaces, staging); the caller makes sure
+    no launch that uses them is still pending."""
+    _check("nmspmm_release", lib().nmspmm_release())
+
+
 # ---- device-pointer forms: arguments are torch tensors on the GPU -----------------------------------
 
 def trans_index_device(dDT, W, N, Q, pN, pM):

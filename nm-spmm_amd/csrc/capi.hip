@@ -3,6 +3,7 @@
 #include "../../include/nmspmm.h"
 #include "internal.h"
 
+#include <atomic>
 #include <cmath>
 #include <mutex>
 #include <vector>
@@ -48,13 +49,25 @@ void* noalloc_scratch()
     return g_scratch_ptr[dev];
 }
 
-// Arrival counters of the decode kernel's cut reductions (NMSPMM_DECODE_SPLIT): zero when the code
-// object is loaded, and every launch leaves them zero again.
+// Arrival counters of the decode kernel's cut reductions (NMSPMM_DECODE_SPLIT), one 64-bit word per
+// vector: (epoch << 8) | arrivals.  Every launch that cuts reductions draws a new epoch for its
+// device, and a word that carries another epoch counts as "no arrivals yet": nothing has to be
+// cleared between launches, and a launch that was cut short leaves nothing behind that a later
+// one could trip over.  (56 bits of epoch: no wrap within a process's life.)
 constexpr int kDecodeTickets = 1024;
-static __device__ unsigned int decode_tickets[kDecodeTickets];
-unsigned int* g_tickets_ptr[64] = {};
+static __device__ unsigned long long decode_tickets[kDecodeTickets];
+unsigned long long* g_tickets_ptr[64] = {};
+std::atomic<unsigned long long> g_decode_epoch[64];
 
-unsigned int* decode_ticket_array()
+unsigned long long next_decode_epoch()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        dev = 0;
+    return (g_decode_epoch[dev].fetch_add(1, std::memory_order_relaxed) + 1) & 0x00ffffffffffffffull;
+}
+
+unsigned long long* decode_ticket_array()
 {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
@@ -66,14 +79,14 @@ unsigned int* decode_ticket_array()
             (void)hipGetLastError();
             return nullptr;
         }
-        g_tickets_ptr[dev] = (unsigned int*)ptr;
+        g_tickets_ptr[dev] = (unsigned long long*)ptr;
     }
     return g_tickets_ptr[dev];
 }
 
 // The GPU's figures, asked once per device; without a device, an MI355X in single-partition mode.
 Machine g_machine[kMaxDevices];
-bool g_machine_known[kMaxDevices] = {};
+std::atomic<bool> g_machine_known[kMaxDevices];
 const Machine kDefaultMachine = {256, 8, 2.4e9};
 std::mutex g_machine_mutex;
 
@@ -181,8 +194,10 @@ const Machine& machine()
         (void)hipGetLastError();
         return kDefaultMachine;
     }
+    if (g_machine_known[dev].load(std::memory_order_acquire))
+        return g_machine[dev];  // every call after the first on a device: no lock
     std::lock_guard<std::mutex> lock(g_machine_mutex);
-    if (!g_machine_known[dev]) {
+    if (!g_machine_known[dev].load(std::memory_order_relaxed)) {
         Machine m = kDefaultMachine;
         int v = 0;
         if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
@@ -195,7 +210,7 @@ const Machine& machine()
         if (m.cus % m.xcds != 0)
             m.xcds = 1;  // an odd partition: the walk then treats the GPU as one die
         g_machine[dev] = m;
-        g_machine_known[dev] = true;
+        g_machine_known[dev].store(true, std::memory_order_release);
     }
     return g_machine[dev];
 }
@@ -532,6 +547,7 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     a.decode_part = nullptr;
     a.decode_part_bytes = 0;
     a.decode_tickets = nullptr;
+    a.decode_epoch = 0;
     a.decode_ticket_count = 0;
     a.C = C;
     a.partial = split_k > 1 ? (float*)workspace : nullptr;
@@ -603,8 +619,10 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
     // the faster kernel on average, without it 4 to 8 % behind (worst 54 %).  (Fitted before the tile
     // kernel's launches of at most one 64-row workgroup per CU got eight waves along K, which only
     // moved ties towards the tile kernel.)
-    const bool decode_wins = kDecodeBias * model_decode_seconds(M, N, W / kept, kept) <
-                             model_tile_seconds(M, N, W / kept, kept, split_k);
+    // (the models are only asked where they decide: 33 to 128 rows)
+    const bool decode_wins = M > 32 && M <= 128 &&
+                             kDecodeBias * model_decode_seconds(M, N, W / kept, kept) <
+                                 model_tile_seconds(M, N, W / kept, kept, split_k);
     if (decode_supported(a) && (M <= 32 || decode_wins || !mfma_supported(a))) {
         // decode sizes with the row list: one launch, reduction inside the workgroup (or, on request,
         // across a few workgroups through the library's device-resident scratch)
@@ -614,6 +632,7 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
             if (a.decode_part && a.decode_tickets) {
                 a.decode_part_bytes = NMSPMM_NOALLOC_MAX_BYTES;
                 a.decode_ticket_count = kDecodeTickets;
+                a.decode_epoch = next_decode_epoch();
             } else {
                 a.decode_part = nullptr;
                 a.decode_tickets = nullptr;

@@ -18,7 +18,8 @@ struct SpmmArgs {
     bool stream_b;         // B is loaded with the non-temporal hint (decode kernel on the row list)
     float* decode_part;    // decode kernel on the row list: scratch for partial tiles when a vector's
     size_t decode_part_bytes;  // reduction is cut across workgroups, and one arrival counter per vector
-    unsigned int* decode_tickets;  // (zero between launches); all three 0 / nullptr: never cut
+    unsigned long long* decode_tickets;  // (epoch << 8 | arrivals); all three 0 / nullptr: never cut
+    unsigned long long decode_epoch;     // this launch's epoch: never 0, never that of an earlier launch on the device
     int decode_ticket_count;
     float* C;              // row-major M x N
     float* partial;        // split_k slices of slice_stride floats when split_k > 1, else nullptr

@@ -54,9 +54,13 @@ struct DecodeParams {
     int rotate;  // groups by which consecutive workgroups of an XCD stagger the start of their walk
     int xcds;    // accelerator dies: consecutive workgroup ids go to consecutive dies
     // cut reductions (SPLIT): workgroup id = slice * vectors + vector; each of the `slices` workgroups
-    // of a vector leaves its partial tile in `part`, takes a ticket, and the last one adds them up
+    // of a vector leaves its partial tile in `part`, takes a ticket, and the last one adds them up.
+    // A ticket word holds (epoch << 8) | arrivals; `epoch` grows with every launch on a device, so a
+    // word left behind by an earlier launch (also one that never finished) is smaller than
+    // epoch << 8 and counts as "no arrivals".
     float* part;
-    unsigned int* tickets;
+    unsigned long long* tickets;
+    unsigned long long epoch;
     int slices, vectors;
     // rows cut across workgroups: the launch has `vectors` = Ncols / 32 x `parts` workgroups (per
     // slice), workgroup (v, q) computes rows [q * part_rows, min(M, (q + 1) * part_rows)) of vector v
@@ -288,16 +292,37 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
         }
     }
     if constexpr (SPLIT) {
-        // Wait for the stores' acknowledgement, take a ticket.  No workgroup ever waits for another:
-        // whoever draws the last ticket of its vector finds all partial tiles complete.
+        // Publish, then take a ticket.  No workgroup ever waits for another: whoever draws the last
+        // ticket of its vector finds all partial tiles complete.  What makes this true:
+        //   - the partial tiles are written and read with agent-scope atomic stores and loads (sc1:
+        //     written through to, and read from, the level at which all dies agree; no cache of
+        //     this or another die can hold a stale copy for such a load to hit);
+        //   - every wave waits until all its stores have been acknowledged (s_waitcnt vmcnt(0):
+        //     on this GPU stores count in vmcnt) before it enters the barrier, so when lane 0 draws
+        //     the ticket after the barrier every lane's part of the tile has arrived;
+        //   - the last arrival reads the tiles only after it has seen its ticket (through LDS and a
+        //     barrier): its loads are issued after every other slice's arrival, hence after their
+        //     stores were acknowledged.
+        // A release fence at workgroup scope does not wait for global stores here (all waves of a
+        // workgroup share a CU), and the slices run on other CUs and dies.  A release fence at agent
+        // scope would give the order as well, but it also writes back everything the die's L2 holds
+        // dirty (other workgroups' rows of C): measured 12 -> 60 us at K = 11008 on 4096 columns.
         __shared__ unsigned int ticket;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (tid == 0)
-            ticket = __hip_atomic_fetch_add(&p.tickets[vv], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) {
+            // Raise the word to this launch's epoch with no arrivals (a word of this epoch is larger
+            // and stays), then arrive.  Both are read-modify-writes of one location by one lane, so
+            // they take effect in this order, and only the second one's answer is waited for.
+            (void)__hip_atomic_fetch_max(&p.tickets[vv], p.epoch << 8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const unsigned long long before =
+                __hip_atomic_fetch_add(&p.tickets[vv], 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            ticket = (unsigned int)(before & 0xffull);  // 0 for the first arrival
+        }
         __syncthreads();
         if (ticket != (unsigned int)(p.slices - 1))
             return;
+        asm volatile("" ::: "memory");
         for (int x = wave; x < 8 * HB; x += kDecodeWaves) {
             float s = 0.0f;
             for (int z = 0; z < p.slices; ++z)
@@ -305,8 +330,6 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
                                        __HIP_MEMORY_SCOPE_AGENT);
             store_c(x, s);
         }
-        if (tid == 0)
-            __hip_atomic_store(&p.tickets[vv], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
     }
 }
 
@@ -398,6 +421,7 @@ hipError_t launch_decode(const SpmmArgs& a)
     }
     p.part = a.decode_part;
     p.tickets = a.decode_tickets;
+    p.epoch = a.decode_epoch;
     p.slices = slices;
     p.vectors = vectors;
     const bool nt = a.stream_b;

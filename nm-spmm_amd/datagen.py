@@ -22,6 +22,8 @@ def init_data(M, N, K, n, m, vec_len=32, seed=0, dist="uniform", a_scale=1.0, b_
     Q = N // vec_len
 
     def values(shape, scale):
+        if dist == "unit":  # [0, 1): the reference's own kind of data (rand() / RAND_MAX, include/utils.h:36,42)
+            return (rng.random(shape, dtype=np.float32) * np.float32(scale)).astype(np.float32)
         if dist == "uniform":
             return ((rng.random(shape, dtype=np.float32) * 2.0 - 1.0) * np.float32(scale)).astype(np.float32)
         return (rng.standard_normal(shape, dtype=np.float32) * np.float32(scale)).astype(np.float32)

@@ -1,6 +1,6 @@
 """The benchmark's command-line contract: more than one GPU is refused with a message (the library
 is a single-GPU kernel library), and on a GPU the default run prints one JSON line with the agreed
-fields."""
+fields, short enough for a harness that keeps a few KB of output, and every case in a detail file."""
 import json
 import os
 import subprocess
@@ -20,13 +20,28 @@ def test_more_than_one_gpu_is_refused_with_a_message():
 
 
 @pytest.mark.gpu
-def test_one_json_line_with_roofline_and_cpu_baseline():
-    out = subprocess.run([sys.executable, BENCH, "--steps", "10", "--warmup", "2", "--cpu-rows", "256"],
+def test_one_json_line_with_roofline_and_cpu_baseline(tmp_path):
+    detail_path = str(tmp_path / "detail.json")
+    out = subprocess.run([sys.executable, BENCH, "--steps", "10", "--warmup", "2", "--cpu-rows", "256", "--detail", detail_path],
                          capture_output=True, text=True, timeout=600)
     assert out.returncode == 0, out.stderr
     lines = [l for l in out.stdout.splitlines() if l.strip()]
     assert len(lines) == 1
-    d = json.loads(lines[0])
+    # a harness that keeps only the tail of a run's output must still hold the whole line
+    assert len(lines[0]) <= 4096 and len(out.stdout) + len(out.stderr) <= 8000
+    line = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline", "dense_fp32_gemm", "sweep", "summary"):
+        assert key in line, key
+    assert line["roofline"]["frac"] > 0.5 and line["cpu_baseline"]["value"] > 0
+    sm = line["summary"]
+    assert sm["llm"]["frac_fp32_mfma_peak"]["n"] == 9 and sm["ragged"]["frac_fp32_mfma_peak"]["n"] == 9
+    assert sm["decode"]["cold_frac_hbm"]["n"] == 16 and 0 < sm["decode"]["cold_frac_hbm"]["max"] <= 1.0
+    assert "hot_gbs" in sm["decode"] and "hot_frac_hbm" not in sm["decode"]
+    assert 0 < sm["compress_frac_hbm"]["max"] <= 1.0 and 0 < sm["decompress_frac_hbm"]["max"] <= 1.0
+    assert sm["dispatch"]["n"] == 12
+    d = json.load(open(detail_path))
+    assert all(d[k] == line[k] for k in ("value", "ms_per_step", "roofline", "cpu_baseline", "config"))
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
                 "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
         assert key in d, key
@@ -52,8 +67,10 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert len(cfg["decode"]) == 16
     for x in cfg["decode"]:
         assert x["kernel"] == "decode" and x["kernel_reference_layout"] == "skinny"
-        for mode in ("hot", "cold", "cold_stream_hint", "hot_reference_layout", "cold_reference_layout"):
-            assert 0 < x[mode]["frac_hbm"] < 1.5 and x[mode]["us"] > 0
+        for mode in ("cold", "cold_stream_hint", "cold_reference_layout"):
+            assert 0 < x[mode]["frac_hbm"] <= 1.0 and x[mode]["us"] > 0
+        for mode in ("hot", "hot_reference_layout"):   # served by the Infinity Cache: a rate, no HBM fraction
+            assert "frac_hbm" not in x[mode] and x[mode]["gbs"] > 0 and x[mode]["served_by"] == "infinity cache"
     assert len(cfg["decode_llm"]) == 9
     for x in cfg["decode_llm"]:
         assert x["kernel"] == "decode" and x["hot_split"]["us"] > 0 and x["cold_split"]["us"] > 0
@@ -61,6 +78,9 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert [x["pattern"] for x in cfg["fine"]][:4] == ["4:32", "8:32", "16:32", "2:4"] and cfg["fine"][3]["vec_len"] == 4
     assert cfg["fine"][-1]["pattern"] == "32:32" and cfg["fine"][-1]["kernel"] == "mfma"
     assert len(cfg["launch_constant"]) == 3 and len(cfg["compress"]) == 12 and len(cfg["rowmajor"]) == 5
+    for x in cfg["compress"]:
+        for name in ("compress", "decompress"):
+            assert 0 < x[name]["frac_hbm"] <= 1.0 and "frac_hbm" not in x[name + "_hot"]
     for x in d["preprocess"]:
         assert x["host_pointer_dropin_wall_ms"] > 0 and x["cpu_restatement_wall_ms"] > 0
         assert x["device_reference_sequence_ms"] > 0
@@ -69,11 +89,15 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
 
 
 @pytest.mark.gpu
-def test_parts_can_be_selected():
-    out = subprocess.run([sys.executable, BENCH, "--steps", "5", "--warmup", "1", "--only", "fine", "--cpu-rows", "0"],
+def test_parts_can_be_selected(tmp_path):
+    detail_path = str(tmp_path / "detail.json")
+    out = subprocess.run([sys.executable, BENCH, "--steps", "5", "--warmup", "1", "--only", "fine", "--cpu-rows", "0",
+                          "--fine-cases", "16:32x32,2:4x4", "--detail", detail_path],
                          capture_output=True, text=True, timeout=600)
     assert out.returncode == 0, out.stderr
-    d = json.loads(out.stdout.strip())
-    assert list(d["configs"]) == ["fine"] and d["cpu_baseline"] is None and d["sweep"] == {} and d["dispatch"] is None
+    line = json.loads(out.stdout.strip())
+    assert list(line["summary"]) == ["fine_frac_fp32_mfma_peak"] and line["cpu_baseline"] is None and line["sweep"] == {}
+    d = json.load(open(detail_path))
+    assert list(d["configs"]) == ["fine"] and len(d["configs"]["fine"]) == 2 and d["dispatch"] is None
     bad = subprocess.run([sys.executable, BENCH, "--only", "nonsense"], capture_output=True, text=True, timeout=120)
     assert bad.returncode != 0 and "unknown part" in bad.stderr

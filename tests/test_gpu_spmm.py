@@ -343,9 +343,11 @@ def test_ragged_last_round_needs_no_workspace(oracle, M, N, K, n, m, Ns):
 
 
 def check_every_tile_once(oracle, M, N, K, n, m, Ns, **gen):
-    """Unsplit multiplication on the tile kernel; column sums of C against column sums computed
-    from the operands in fp64 (touches every tile), and the first and last rows against the
-    checker."""
+    """Unsplit multiplication on the tile kernel, checked three ways: every element of C against
+    the dense fp64 product A x decompress(B) (the textbook meaning of the operation; sees any row
+    or column that went to the wrong place inside a tile, which sums along one axis cannot), the
+    row and column sums as checksums of their own, and the first and last rows and one interior
+    row of every 32-row strip against the checker."""
     d = datagen.init_data(M, N, K, n, m, seed=M + K, **gen)
     window, kept, D, cinfo = preprocess_with_oracle(oracle, d, Ns)
     C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
@@ -353,17 +355,26 @@ def check_every_tile_once(oracle, M, N, K, n, m, Ns, **gen):
                 kept, 32, Ns, 1, None)
     torch.cuda.synchronize()
     assert nmspmm.last_kernel() == "mfma" and bool(torch.isfinite(C).all())
-    # column sums of C against column sums computed from the operands in fp64: touches every tile
     dense = torch.zeros((K, N), dtype=torch.float64, device="cuda")
     rows = (torch.arange(d["W"], device="cuda") // n * m)[:, None] + dev(d["DT"]).long()
     dense[rows.repeat_interleave(32, dim=1), torch.arange(N, device="cuda")[None, :].expand(d["W"], -1)] = dev(d["BT"]).double()
-    want = dev(d["A_km"]).double().sum(dim=1) @ dense
-    got = C.double().sum(dim=0)
-    assert float(((got - want).abs() / want.abs().clamp_min(want.pow(2).mean().sqrt())).max()) <= REL_TOL
-    for (r0, r1) in ((0, 16), (M - 16, M)):
-        ref = oracle.gemm_cpu(d["A_km"].reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), M, N, d["W"],
-                              rows=(r0, r1)).reshape(M, N)[r0:r1]
-        assert scaled_max_error(C[r0:r1].cpu().numpy(), ref) <= REL_TOL
+    A64 = dev(d["A_km"]).double()                                # [K][M]
+    scaled = lambda got, want: float(((got - want).abs() / want.abs().clamp_min(want.pow(2).mean().sqrt())).max())
+    # checksums: C^T 1 = B^T (A^T 1) and C 1 = A (B 1)
+    assert scaled(C.double().sum(dim=0), A64.sum(dim=1) @ dense) <= REL_TOL
+    assert scaled(C.double().sum(dim=1), dense.sum(dim=1) @ A64) <= REL_TOL
+    # every element, a band of rows at a time (bounds the fp64 temporaries)
+    for r0 in range(0, M, 2048):
+        want = A64[:, r0:r0 + 2048].t() @ dense
+        assert scaled(C[r0:r0 + 2048].double(), want) <= REL_TOL, "rows %d.." % r0
+        del want
+    del dense, A64
+    sample = sorted(set(list(range(16)) + list(range(M - 16, M)) + [32 * s + (7 * s + 5) % 32 for s in range(M // 32)]))
+    got = C.cpu().numpy()
+    ref = np.zeros(M * N, np.float32)  # the checker adds into the rows it is asked for: each sampled row once
+    for r in sample:
+        oracle.gemm_cpu(d["A_km"].reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), M, N, d["W"], rows=(r, r + 1), C=ref)
+    assert scaled_max_error(got[sample], ref.reshape(M, N)[sample]) <= REL_TOL
 
 
 @pytest.mark.parametrize("M,N,K,n,m", [(4096, 8448, 256, 2, 4), (8192, 4224, 512, 1, 8), (2048, 11008, 256, 2, 4),

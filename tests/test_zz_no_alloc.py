@@ -31,10 +31,21 @@ def both_ways(oracle, M, N, K, n, m, split_k, seed):
     nmspmm.spmm(A, B, Dd, ci, C_ws, M, N, K, d["W"], window, kept, 32, 128, split_k, ws)
     fam = nmspmm.last_kernel()
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # Nothing may be allocated by the call: not by torch (memory_allocated) and not by the library
+    # behind torch's back (the device's free bytes as hipMemGetInfo reports them, which a hipMalloc
+    # inside libnmspmm.so would lower).  One untimed call first, so that the code object and the
+    # scratch's address are already resolved; the library's cached workspace is released before,
+    # so that any use of it would have to allocate again and show.
+    nmspmm.spmm_noalloc(A, B, Dd, ci, C_na, M, N, K, d["W"], window, kept, 32, 128, split_k)
+    torch.cuda.synchronize()
+    nmspmm.release()
+    C_na.fill_(float("nan"))
+    torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     nmspmm.spmm_noalloc(A, B, Dd, ci, C_na, M, N, K, d["W"], window, kept, 32, 128, split_k)
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] >= free_before, "device memory was allocated during the call"
     assert nmspmm.last_kernel() == fam
     assert torch.equal(C_na, C_ws), "differs from the call with a caller-owned workspace"
     want = oracle.gemm_cpu(d["A_km"].reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), M, N,
