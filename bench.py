@@ -3,7 +3,7 @@
 
 One "step" is one launch of the hot path (nmspmm_spmm through the C-ABI) on the square sweep of
 the baseline: M = Ncols = K = 4096, fp32, operands resident in HBM, at 2:4 (the headline value).
-Prints ONE JSON line:
+Prints ONE JSON line; its parts:
 
   value            useful TFLOP/s at 2:4 = 2*M*Ncols*W / t   (W = K*n/m)
   roofline         the dominant kernel (the tile kernel at 2:4) against the fp32 MFMA peak
@@ -22,10 +22,15 @@ Prints ONE JSON line:
                      fine    4:32, 8:32, 16:32 and 2:4 with 4-column vectors at 4096 cubed
                      launch_constant, compress, rowmajor: the part of a launch that does not scale
                              with K; dense <-> compressed conversion; row-major activations
+                     sweep100  the 100 shapes x 4 sparsities of the reference's kernel-performance
+                             sweep against the dense fp32 GEMM
   preprocess       index preprocessing: one-kernel device call, the reference's call sequence on
                    the device, the host-pointer drop-in calls (wall time, PCIe included), and the
                    CPU restatement / the reference's own host code
   dispatch         the library's split / kernel choice against the best of the splits 1, 2, 4, 8
+
+The printed line holds the headline fields whole and one digest per other workload (it stays under
+4 KB); every case of every part goes to the detail file (--detail, default bench_detail.json).
 
 Timing uses HIP events on the stream the kernels are launched on (torch's current stream is the
 one handed to the C-ABI); decode-sized launches are replayed from a HIP graph so that the host's
@@ -51,7 +56,7 @@ PATTERNS = [(2, 4), (3, 8), (2, 8), (1, 8)]  # first one is the headline
 NS = 128
 GEOMETRY = {(1, 1): (32, 32), (1, 2): (32, 16), (3, 8): (32, 12), (1, 4): (64, 16), (1, 8): (64, 8)}
 PARTS = ("sweep", "llm", "ragged", "decode", "decode_llm", "decode_wide", "fine", "ksweep", "compress", "rowmajor", "preprocess", "dispatch", "cpu", "sweep100")
-OPT_IN_PARTS = ("sweep100",)   # several minutes: run by name only
+OPT_IN_PARTS = ()   # parts that only run when named
 
 
 def geometry(n, m):
@@ -600,7 +605,9 @@ def run_sweep100(torch, pkg):
     """The 100 shapes of the reference's sweep at 50, 62.5, 75 and 87.5 % (16:32, 12:32, 8:32, 4:32):
     the library's own choice of kernel and split (the reference takes the best of four tiles and
     four splits by brute force, run_nmspmm.sh:19-36) against torch.mm fp32 of the same shape.  Line
-    20*mi + i of each list is M[mi] with (Ncols, K)[i], as in the reference's result files."""
+    20*mi + i of each list is M[mi] with (Ncols, K)[i], as in the reference's result files.  Both
+    sides are replayed from a HIP graph of five launches: the smallest shapes last about ten
+    microseconds, less than a launch from Python."""
     by = {}
     dense_ms = []
     for m_rows in SWEEP100_M:
@@ -608,16 +615,15 @@ def run_sweep100(torch, pkg):
             a = torch.randn((m_rows, k), dtype=torch.float32, device="cuda")
             b = torch.randn((k, n_cols), dtype=torch.float32, device="cuda")
             c = torch.empty((m_rows, n_cols), dtype=torch.float32, device="cuda")
-            ms, _ = time_launches(torch, lambda: torch.mm(a, b, out=c), 10, 2, 0.05)
-            dense_ms.append(ms)
+            dense_ms.append(time_graph(torch, [lambda: torch.mm(a, b, out=c)] * 5, 3, 0.05))
             del a, b, c
     for kept, label in ((16, "0.5"), (12, "0.625"), (8, "0.75"), (4, "0.875")):
         rows, idx = [], 0
         for m_rows in SWEEP100_M:
             for n_cols, k in zip(SWEEP100_N, SWEEP100_K):
                 op = GpuOperands(torch, pkg, m_rows, n_cols, k, kept, 32, normal=False)
-                ms, _ = time_launches(torch, lambda: pkg.gemm_auto(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k,
-                                                                   op.W, float(label)), 10, 2, 0.05)
+                ms = time_graph(torch, [lambda: pkg.gemm_auto(op.A, op.B, op.D, op.cinfo, op.C, m_rows, n_cols, k, op.W,
+                                                              float(label))] * 5, 3, 0.05)
                 rows.append({"M": m_rows, "Ncols": n_cols, "K": k, "ms": round(ms, 4), "dense_ms": round(dense_ms[idx], 4),
                              "dense_equiv_tflops": round(2.0 * m_rows * n_cols * k / ms / 1e9, 2),
                              "speedup_vs_dense": round(dense_ms[idx] / ms, 3)})
@@ -708,9 +714,10 @@ def summarize(configs, preprocess, dispatch):
     if "rowmajor" in configs:
         s["rowmajor_overhead"] = digest(configs["rowmajor"], lambda r: r["overhead"], shape, higher_is_better=False)
     if "sweep100" in configs:
-        s["sweep100"] = {k: {f: v[f] for f in ("shapes", "mean_speedup_vs_dense", "min_speedup_vs_dense",
-                                               "a100_reference_mean_speedup")}
-                         for k, v in configs["sweep100"]["by_sparsity"].items()}
+        s["sweep100_speedup_vs_dense"] = {"columns": ["mean", "min", "reference_on_a100_mean"]}
+        for k, v in configs["sweep100"]["by_sparsity"].items():
+            s["sweep100_speedup_vs_dense"][k] = [v["mean_speedup_vs_dense"], v["min_speedup_vs_dense"],
+                                                 v["a100_reference_mean_speedup"]]
     if preprocess:
         s["preprocess_device_ms"] = {"%sx%d" % (r["pattern"], r["vec_len"]): r["device_one_kernel_ms"] for r in preprocess}
         s["preprocess_cpu_ms"] = {"%sx%d" % (r["pattern"], r["vec_len"]): r.get("cpu_reference_wall_ms", r["cpu_restatement_wall_ms"])

@@ -2,10 +2,15 @@
 runs the library's kernels: dense weight -> compress -> widen / preprocess once at construction,
 then one row-major multiplication per call.  PyTorch only supplies device memory and the stream.
 
+The multiplication is registered with torch.library as the operator `nmspmm::sparse_linear`
+(with a fake implementation that only derives the output's shape), so that tracing front ends
+(torch.compile, torch.export) see one opaque node instead of a Python function they cannot follow.
+
 The reference has no framework binding; its driver multiplies synthetic operands
 (tests/test_nmspmm.cu:72-97).  The sequence of calls here is that driver's, on real weights.
 """
 import importlib
+from typing import Optional
 
 import torch
 
@@ -25,6 +30,40 @@ def _geometry(n, m):
     if window % m != 0:
         raise ValueError("pattern window %d does not divide the kernel window %d" % (m, window))
     return window, kept
+
+
+_plans = {}  # (M, N, K, W, kept) -> (split, workspace floats): two library calls per shape, not per forward
+
+
+@torch.library.custom_op("nmspmm::sparse_linear", mutates_args=(), device_types="cuda")
+def sparse_linear(x: torch.Tensor, values: torch.Tensor, indices: torch.Tensor, column_info: Optional[torch.Tensor],
+                  row_index: Optional[torch.Tensor], bias: Optional[torch.Tensor], window: int, kept: int, Ns: int,
+                  flags: int) -> torch.Tensor:
+    """x [..., K] row-major times the compressed weight (values [W, N], preprocessed indices,
+    column_info for 64-row windows, optional row list) plus bias: [..., N].  The library's own
+    choice of kernel and split; the workspace comes from torch's caching allocator."""
+    W, N = values.shape
+    K = x.shape[-1]
+    x2 = x.reshape(-1, K).contiguous()
+    M = x2.shape[0]
+    y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+    if M > 0:
+        key = (M, N, K, W, kept)
+        if key not in _plans:
+            split = _nm.suggest_split_k(M, N, W, kept)
+            _plans[key] = (split, _nm.workspace_bytes_rowmajor(M, N, K, split) // 4)
+        split, need = _plans[key]
+        workspace = torch.empty(max(need, 4), dtype=torch.float32, device=x.device)
+        _nm.spmm_rowmajor(x2, values, indices, column_info, y, M, N, K, W, window, kept, workspace, 32, Ns, split,
+                          row_index, flags)
+        if bias is not None:
+            y += bias
+    return y.reshape(*x.shape[:-1], N)
+
+
+@sparse_linear.register_fake
+def _sparse_linear_fake(x, values, indices, column_info, row_index, bias, window, kept, Ns, flags):
+    return x.new_empty((*x.shape[:-1], values.shape[1]))
 
 
 class NMSparseLinear(torch.nn.Module):
@@ -73,8 +112,6 @@ class NMSparseLinear(torch.nn.Module):
         self.register_buffer("column_info", cinfo)
         self.register_buffer("row_index", rows)
         self.register_buffer("bias", None if bias is None else bias.detach().to(torch.float32))
-        self._workspace = None
-        self._plans = {}
 
     def dense_weight(self):
         """The pruned weight as a dense [out_features, in_features] tensor (for checking)."""
@@ -86,23 +123,8 @@ class NMSparseLinear(torch.nn.Module):
     def forward(self, x, add_bias=True):
         if x.dtype != torch.float32 or not x.is_cuda or x.shape[-1] != self.in_features:
             raise ValueError("x must be a float32 CUDA tensor whose last dimension is in_features")
-        lead = x.shape[:-1]
-        x2 = x.reshape(-1, self.in_features).contiguous()
-        M, N, K = x2.shape[0], self.out_features, self.in_features
-        y = torch.empty((M, N), dtype=torch.float32, device=x.device)
-        if M == 0:
-            return y.reshape(*lead, N)
-        if M not in self._plans:  # two library calls per row count, not per forward
-            split = _nm.suggest_split_k(M, N, self.W, self.kept)
-            self._plans[M] = (split, _nm.workspace_bytes_rowmajor(M, N, K, split) // 4)
-        split, need = self._plans[M]
-        if self._workspace is None or self._workspace.numel() < need or self._workspace.device != x.device:
-            self._workspace = torch.empty(need, dtype=torch.float32, device=x.device)
-        _nm.spmm_rowmajor(x2, self.values, self.indices, self.column_info, y, M, N, K, self.W, self.window, self.kept,
-                          self._workspace, 32, self.Ns, split, self.row_index, self.flags)
-        if add_bias and self.bias is not None:
-            y += self.bias
-        return y.reshape(*lead, N)
+        return sparse_linear(x, self.values, self.indices, self.column_info, self.row_index,
+                             self.bias if add_bias else None, self.window, self.kept, self.Ns, self.flags)
 
     def extra_repr(self):
         return "in_features=%d, out_features=%d, pattern=%d:%d, bias=%s" % (

@@ -40,6 +40,7 @@ def test_one_json_line_with_roofline_and_cpu_baseline(tmp_path):
     assert "hot_gbs" in sm["decode"] and "hot_frac_hbm" not in sm["decode"]
     assert 0 < sm["compress_frac_hbm"]["max"] <= 1.0 and 0 < sm["decompress_frac_hbm"]["max"] <= 1.0
     assert sm["dispatch"]["n"] == 12
+    assert sm["sweep100_speedup_vs_dense"]["columns"][0] == "mean" and sm["sweep100_speedup_vs_dense"]["0.5"][0] > 1.5
     d = json.load(open(detail_path))
     assert all(d[k] == line[k] for k in ("value", "ms_per_step", "roofline", "cpu_baseline", "config"))
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
@@ -84,6 +85,8 @@ def test_one_json_line_with_roofline_and_cpu_baseline(tmp_path):
     for x in d["preprocess"]:
         assert x["host_pointer_dropin_wall_ms"] > 0 and x["cpu_restatement_wall_ms"] > 0
         assert x["device_reference_sequence_ms"] > 0
+    for k, v in cfg["sweep100"]["by_sparsity"].items():
+        assert len(v["rows"]) == 100 and v["mean_speedup_vs_dense"] > 0.7 / (1.0 - float(k))
     assert len(d["dispatch"]["shapes"]) == 12 and d["dispatch"]["mean_ratio"] < 1.1
     assert d["device"]["compute_units"] > 0 and d["device"]["dies"] > 0
 
