@@ -353,7 +353,9 @@ def run_ragged(torch, pkg):
 
 DECODE_MODES = (("hot", 0, True, False), ("cold", 0, True, True), ("cold_stream_hint", 2, True, True),
                 ("hot_reference_layout", 0, False, False), ("cold_reference_layout", 0, False, True),
-                ("hot_split", 4, True, False), ("cold_split", 4, True, True))
+                ("hot_split", 4, True, False), ("cold_split", 4, True, True),
+                # rows of A staged in LDS per reduction slice (spmm_decode_lds.hip): measured and set aside
+                ("hot_stage_a", 12, True, False), ("cold_stage_a", 12, True, True))
 DECODE_DEFAULT_MODES = tuple(m[0] for m in DECODE_MODES[:5])
 # the decode sizes of the LLM-layer shapes (config 3's K x Ncols): fewer column vectors than compute
 # units, where NMSPMM_DECODE_SPLIT lets the kernel cut the reductions across workgroups
@@ -671,20 +673,21 @@ def run_dispatch(torch, pkg):
 
 
 MAX_LINE_BYTES = 4096
+DIGEST_COLUMNS = ["cases", "min", "median", "max", "worst case"]
 
 
 def digest(rows, value, name, higher_is_better=True):
-    """[cases, min, median, max, worst case] of value(row) over the rows."""
+    """[cases, min, median, max, worst case] of value(row) over the rows (DIGEST_COLUMNS)."""
     vals = [(value(r), name(r)) for r in rows]
     nums = sorted(v for v, _ in vals)
     worst = (min if higher_is_better else max)(vals)
-    return {"n": len(rows), "min": nums[0], "med": round(float(np.median(nums)), 3), "max": nums[-1], "worst": worst[1]}
+    return [len(rows), nums[0], round(float(np.median(nums)), 3), nums[-1], worst[1]]
 
 
 def summarize(configs, preprocess, dispatch):
     """One short digest per workload for the printed line; every case is in the detail file."""
     shape = lambda r: "%dx%dx%d %s" % (r["M"], r["Ncols"], r["K"], r["pattern"])
-    s = {}
+    s = {"digest_columns": DIGEST_COLUMNS}
     for key in ("llm", "ragged"):
         if key in configs:
             s[key] = {"frac_fp32_mfma_peak": digest(configs[key], lambda r: r["frac_fp32_mfma_peak"], shape)}
@@ -723,7 +726,7 @@ def summarize(configs, preprocess, dispatch):
         s["preprocess_cpu_ms"] = {"%sx%d" % (r["pattern"], r["vec_len"]): r.get("cpu_reference_wall_ms", r["cpu_restatement_wall_ms"])
                                   for r in preprocess}
     if dispatch:
-        s["dispatch"] = {"n": len(dispatch["shapes"]), "mean_ratio": dispatch["mean_ratio"], "worst_ratio": dispatch["worst_ratio"]}
+        s["dispatch"] = {"cases": len(dispatch["shapes"]), "mean_ratio": dispatch["mean_ratio"], "worst_ratio": dispatch["worst_ratio"]}
     return s
 
 

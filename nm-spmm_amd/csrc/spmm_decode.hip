@@ -55,9 +55,9 @@ struct DecodeParams {
     int xcds;    // accelerator dies: consecutive workgroup ids go to consecutive dies
     // cut reductions (SPLIT): workgroup id = slice * vectors + vector; each of the `slices` workgroups
     // of a vector leaves its partial tile in `part`, takes a ticket, and the last one adds them up.
-    // A ticket word holds (epoch << 8) | arrivals; `epoch` grows with every launch on a device, so a
-    // word left behind by an earlier launch (also one that never finished) is smaller than
-    // epoch << 8 and counts as "no arrivals".
+    // A ticket word holds (epoch << 8) | arrivals and is zero between launches; `epoch` grows with
+    // every launch on a device, so a word left behind by a launch that never finished is smaller
+    // than epoch << 8 and counts as "no arrivals" too.
     float* part;
     unsigned long long* tickets;
     unsigned long long epoch;
@@ -324,12 +324,24 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
             return;
         asm volatile("" ::: "memory");
         for (int x = wave; x < 8 * HB; x += kDecodeWaves) {
+            // the slices' values (at most eight) are requested together and added in slice order
+            float t[8];
+#pragma unroll
+            for (int z = 0; z < 8; ++z)
+                t[z] = z < p.slices ? __hip_atomic_load(&p.part[((size_t)vv * p.slices + z) * kTile + x * 64 + lane],
+                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                    : 0.0f;
             float s = 0.0f;
-            for (int z = 0; z < p.slices; ++z)
-                s += __hip_atomic_load(&p.part[((size_t)vv * p.slices + z) * kTile + x * 64 + lane], __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int z = 0; z < 8; ++z)
+                s += t[z];
             store_c(x, s);
         }
+        // The word goes back to zero: a HIP graph that replays this launch carries this launch's
+        // epoch again and must find what the first run found.  (A launch that is cut short leaves
+        // its word behind; the next launch's larger epoch overrides it.)
+        if (tid == 0)
+            __hip_atomic_store(&p.tickets[vv], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 

@@ -186,25 +186,32 @@ __global__ void __launch_bounds__(64 * kLdsWaves) spmm_decode_lds_kernel(const D
             }
     };
 
-    // B and the list do not wait for A: the first group's requests go out before the barrier that
-    // ends the fill, and from then on one group is in flight while another is multiplied
-    float2 b_cur[4], b_next[4];
-    lintx4 rows_cur, rows_next;
+    // B and the list do not wait for A: the first two groups' requests go out before the barrier
+    // that ends the fill, and from then on two groups are in flight while another is multiplied
+    float2 b0[4], b1[4], b2[4];
+    lintx4 r0, r1, r2;
     if (cnt > 0) {
-        rows_cur = load_rows(group_of(0));
-        load_b(group_of(0), b_cur);
+        r0 = load_rows(group_of(0));
+        load_b(group_of(0), b0);
+    }
+    if (cnt > 1) {
+        r1 = load_rows(group_of(1));
+        load_b(group_of(1), b1);
     }
     __syncthreads();
     for (int i = 0; i < cnt; ++i) {
-        if (i + 1 < cnt) {
-            rows_next = load_rows(group_of(i + 1));
-            load_b(group_of(i + 1), b_next);
+        if (i + 2 < cnt) {
+            r2 = load_rows(group_of(i + 2));
+            load_b(group_of(i + 2), b2);
         }
-        multiply(rows_cur, b_cur);
-        rows_cur = rows_next;
+        multiply(r0, b0);
+        r0 = r1;
+        r1 = r2;
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
-            b_cur[t] = b_next[t];
+        for (int t = 0; t < 4; ++t) {
+            b0[t] = b1[t];
+            b1[t] = b2[t];
+        }
     }
 
     // ---- the waves of a vector add their tiles in wave order ------------------------------------
@@ -254,16 +261,37 @@ __global__ void __launch_bounds__(64 * kLdsWaves) spmm_decode_lds_kernel(const D
         arrival[my_vec] = (unsigned int)(before & 0xffull);
     }
     __syncthreads();
-    if (!live || arrival[my_vec] != (unsigned int)(p.slices - 1))
-        return;
+    // Every wave helps with every vector of the workgroup whose last slice this is: item = (vector,
+    // value).  The slices' values are requested together (eight at a time) and added in slice order.
     asm volatile("" ::: "memory");
-    for (int x = my_sub; x < 8 * HB; x += wpv) {
+    for (int item = wave; item < p.V * 8 * HB; item += kLdsWaves) {
+        const int j = item / (8 * HB), x = item % (8 * HB);
+        const int vj = vgroup * p.V + j;
+        if (vj >= p.Q || arrival[j] != (unsigned int)(p.slices - 1))
+            continue;
+        const float* const tiles = p.part + (size_t)vj * p.slices * kTile + x * 64 + lane;
         float s = 0.0f;
-        for (int z = 0; z < p.slices; ++z)
-            s += __hip_atomic_load(&p.part[((size_t)v * p.slices + z) * kTile + x * 64 + lane], __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-        store_c(x, s);
+        for (int z0 = 0; z0 < p.slices; z0 += 8) {
+            float t[8];
+#pragma unroll
+            for (int z = 0; z < 8; ++z)
+                t[z] = z0 + z < p.slices
+                           ? __hip_atomic_load(&tiles[(size_t)(z0 + z) * kTile], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                           : 0.0f;
+#pragma unroll
+            for (int z = 0; z < 8; ++z)
+                s += t[z];
+        }
+        const int row = 16 * (x / 8) + 4 * kq + (x % 4);
+        if (row < M) {
+            float* const dst = p.C + (size_t)row * N + (size_t)vj * 32 + 2 * jl + (x % 8) / 4;
+            *dst = p.accumulate ? *dst + s : s;
+        }
     }
+    // the words go back to zero, so that a HIP graph that replays this launch (with this epoch)
+    // finds what the first run found
+    if (live && my_sub == 0 && lane == 0 && arrival[my_vec] == (unsigned int)(p.slices - 1))
+        __hip_atomic_store(&p.tickets[v], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 namespace {

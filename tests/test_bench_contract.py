@@ -35,11 +35,12 @@ def test_one_json_line_with_roofline_and_cpu_baseline(tmp_path):
         assert key in line, key
     assert line["roofline"]["frac"] > 0.5 and line["cpu_baseline"]["value"] > 0
     sm = line["summary"]
-    assert sm["llm"]["frac_fp32_mfma_peak"]["n"] == 9 and sm["ragged"]["frac_fp32_mfma_peak"]["n"] == 9
-    assert sm["decode"]["cold_frac_hbm"]["n"] == 16 and 0 < sm["decode"]["cold_frac_hbm"]["max"] <= 1.0
+    assert sm["digest_columns"] == ["cases", "min", "median", "max", "worst case"]
+    assert sm["llm"]["frac_fp32_mfma_peak"][0] == 9 and sm["ragged"]["frac_fp32_mfma_peak"][0] == 9
+    assert sm["decode"]["cold_frac_hbm"][0] == 16 and 0 < sm["decode"]["cold_frac_hbm"][3] <= 1.0
     assert "hot_gbs" in sm["decode"] and "hot_frac_hbm" not in sm["decode"]
-    assert 0 < sm["compress_frac_hbm"]["max"] <= 1.0 and 0 < sm["decompress_frac_hbm"]["max"] <= 1.0
-    assert sm["dispatch"]["n"] == 12
+    assert 0 < sm["compress_frac_hbm"][3] <= 1.0 and 0 < sm["decompress_frac_hbm"][3] <= 1.0
+    assert sm["dispatch"]["cases"] == 12
     assert sm["sweep100_speedup_vs_dense"]["columns"][0] == "mean" and sm["sweep100_speedup_vs_dense"]["0.5"][0] > 1.5
     d = json.load(open(detail_path))
     assert all(d[k] == line[k] for k in ("value", "ms_per_step", "roofline", "cpu_baseline", "config"))
@@ -99,7 +100,7 @@ def test_parts_can_be_selected(tmp_path):
                          capture_output=True, text=True, timeout=600)
     assert out.returncode == 0, out.stderr
     line = json.loads(out.stdout.strip())
-    assert list(line["summary"]) == ["fine_frac_fp32_mfma_peak"] and line["cpu_baseline"] is None and line["sweep"] == {}
+    assert list(line["summary"]) == ["digest_columns", "fine_frac_fp32_mfma_peak"] and line["cpu_baseline"] is None and line["sweep"] == {}
     d = json.load(open(detail_path))
     assert list(d["configs"]) == ["fine"] and len(d["configs"]["fine"]) == 2 and d["dispatch"] is None
     bad = subprocess.run([sys.executable, BENCH, "--only", "nonsense"], capture_output=True, text=True, timeout=120)
