@@ -353,9 +353,7 @@ def run_ragged(torch, pkg):
 
 DECODE_MODES = (("hot", 0, True, False), ("cold", 0, True, True), ("cold_stream_hint", 2, True, True),
                 ("hot_reference_layout", 0, False, False), ("cold_reference_layout", 0, False, True),
-                ("hot_split", 4, True, False), ("cold_split", 4, True, True),
-                # rows of A staged in LDS per reduction slice (spmm_decode_lds.hip): measured and set aside
-                ("hot_stage_a", 12, True, False), ("cold_stage_a", 12, True, True))
+                ("hot_split", 4, True, False), ("cold_split", 4, True, True))
 DECODE_DEFAULT_MODES = tuple(m[0] for m in DECODE_MODES[:5])
 # the decode sizes of the LLM-layer shapes (config 3's K x Ncols): fewer column vectors than compute
 # units, where NMSPMM_DECODE_SPLIT lets the kernel cut the reductions across workgroups

@@ -516,7 +516,7 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
                      size_t workspace_bytes, void* stream, int lda, bool dry_run, int* lda_out, bool a_rowmajor = false,
                      unsigned flags = 0, const int32_t* row_index = nullptr)
 {
-    if (flags & ~(unsigned)(NMSPMM_ACCUMULATE | NMSPMM_STREAM_B | NMSPMM_DECODE_SPLIT | 8u))
+    if (flags & ~(unsigned)(NMSPMM_ACCUMULATE | NMSPMM_STREAM_B | NMSPMM_DECODE_SPLIT))
         return NMSPMM_ERR_BAD_SHAPE;
     if (!A || !B || !D || !C)
         return NMSPMM_ERR_NULL_POINTER;
@@ -637,11 +637,6 @@ static int spmm_impl(const float* A, const float* B, const int32_t* D, const int
                 a.decode_part = nullptr;
                 a.decode_tickets = nullptr;
             }
-        }
-        if ((flags & 8u) && a.decode_part && decode_lds_supported(a)) {
-            e = launch_decode_lds(a);
-            g_last_kernel = "decode_lds";
-            return e == hipSuccess ? NMSPMM_OK : NMSPMM_ERR_HIP;
         }
         e = launch_decode(a);
         g_last_kernel = "decode";

@@ -520,8 +520,6 @@ hipError_t launch_skinny(const SpmmArgs& a);
 // Decode-sized path on the row list (spmm_decode.hip): M <= 32 and a.row_index given.
 bool decode_supported(const SpmmArgs& a);
 hipError_t launch_decode(const SpmmArgs& a);
-bool decode_lds_supported(const SpmmArgs& a);   // spmm_decode_lds.hip: rows of A staged in LDS
-hipError_t launch_decode_lds(const SpmmArgs& a);
 // Row list from the preprocessed D (and column_info on the high-sparsity layout).
 hipError_t launch_row_index(const int32_t* D, const int32_t* cinfo, int32_t* R, int W, int N, int window, int kept,
                             int Ns, hipStream_t stream);

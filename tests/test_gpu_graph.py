@@ -89,3 +89,47 @@ def test_graph_replays_of_a_call_that_hands_its_last_rows_over(oracle):
         assert torch.isfinite(C_g).all().item()
         assert torch.equal(C_g, C_e), "replay %d" % rep
 
+
+
+@pytest.mark.parametrize("M", [1, 16, 32])
+def test_graph_replays_of_cut_decode_reductions(oracle, M):
+    """NMSPMM_DECODE_SPLIT inside a graph: the captured launch carries one epoch for its arrival
+    words, and every replay presents it again, interleaved with eager launches that carry newer
+    ones.  The words are zero between launches, so each replay finds what the first run found: C
+    is written by the slice that arrives last, every time, identical to the eager call."""
+    N, K, n, m = 4096, 11008, 2, 8
+    d = datagen.init_data(M, N, K, n, m, seed=M + 3, dist="normal", b_scale=0.02)
+    window, kept, D, cinfo = preprocess_with_oracle(oracle, d, 128)
+    W = d["W"]
+    A, B, Dd, dc = dev(d["A_km"]), dev(d["BT"]), dev(D), dev(cinfo)
+    R = torch.empty(nmspmm.row_index_ints(W, N), dtype=torch.int32, device="cuda")
+    nmspmm.row_index_device(Dd, dc, W, N, window, kept, 128, R)
+    C_g = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    C_e = torch.empty_like(C_g)
+    C_plain = torch.empty_like(C_g)
+
+    def call(C, flags=nmspmm.DECODE_SPLIT):
+        nmspmm.spmm_ex(A, B, Dd, dc, C, M, N, K, W, window, kept, 32, 128, 1, None, flags, R)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(C_g)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(C_g)
+        call(C_g)   # twice in one graph: two epochs held by the same graph
+    for rep in range(5):
+        A.mul_(1.25)
+        C_g.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        call(C_e)
+        call(C_plain, 0)
+        torch.cuda.synchronize()
+        assert nmspmm.last_kernel() == "decode"
+        assert torch.isfinite(C_g).all().item(), "replay %d left rows of C unwritten" % rep
+        assert torch.equal(C_g, C_e), "replay %d" % rep
+        scale = float(C_plain.abs().max())
+        assert float((C_g - C_plain).abs().max()) <= 1e-4 * scale
