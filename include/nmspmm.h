@@ -198,6 +198,19 @@ size_t nmspmm_row_index_ints(int W, int N);
 int nmspmm_row_index_device(const int32_t* dD, const int32_t* d_column_info, int W, int N, int window,
                             int kept, int Ns, int32_t* d_row_index, void* stream);
 
+/* No counterpart in the reference: the named launchers (nmGEMM_*_matrices_*_sparsity, nmGEMM,
+ * nmspmm_gemm_low_sparsity / _high_sparsity / _auto) keep the reference's signatures, which have
+ * no argument for the row list, so their decode-sized calls (M <= 128) run on D / column_info.
+ * nmspmm_row_index_attach tells the library that `row_index` (device memory, made by
+ * nmspmm_row_index_device from this D and its column_info) belongs to the index buffer that
+ * starts at device address dD; from then on a named launcher that is handed this dD on this device
+ * passes the list on, exactly as if the caller had called nmspmm_spmm_ex with it.  The caller keeps
+ * both buffers alive and unchanged while attached; attaching again replaces the list; a NULL
+ * row_index, nmspmm_row_index_detach, or nmspmm_release end it.  Thread-safe.  Returns
+ * NMSPMM_ERR_NULL_POINTER for a NULL dD. */
+int nmspmm_row_index_attach(const int32_t* dD, const int32_t* row_index);
+int nmspmm_row_index_detach(const int32_t* dD);
+
 /* No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  nmspmm_spmm with the
  * split-K slices in a fixed device-resident array of NMSPMM_NOALLOC_MAX_BYTES that belongs to the
@@ -304,7 +317,7 @@ int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int
                      float* C, int M, int N, int K, int W, float sparsity, void* stream);
 
 /* Frees what the library keeps per device: the cached split-K workspaces and the staging buffer
- * of the host-pointer preprocessing forms. */
+ * of the host-pointer preprocessing forms; forgets every attached row list. */
 int nmspmm_release(void);
 
 /* Name of the kernel family the last successful nmspmm_spmm call on this thread dispatched to

@@ -65,6 +65,8 @@ def lib():
         L.nmspmm_row_index_ints.restype = c_size_t
         L.nmspmm_row_index_ints.argtypes = [c_int] * 2
         L.nmspmm_row_index_device.argtypes = [c_void_p, c_void_p] + [c_int] * 5 + [c_void_p, c_void_p]
+        L.nmspmm_row_index_attach.argtypes = [c_void_p, c_void_p]
+        L.nmspmm_row_index_detach.argtypes = [c_void_p]
         L.nmspmm_spmm_noalloc.argtypes = [c_void_p] * 5 + [c_int] * 9 + [c_void_p]
         L.nmspmm_gemm_low_sparsity.argtypes = [c_int] + [c_void_p] * 4 + [c_int] * 4 + [c_float, c_int, c_void_p]
         L.nmspmm_gemm_high_sparsity.argtypes = [c_int] + [c_void_p] * 5 + [c_int] * 4 + [c_float, c_int, c_void_p]
@@ -130,6 +132,12 @@ def pattern_from_sparsity(sparsity):
 
 def last_kernel():
     return lib().nmspmm_last_kernel().decode()
+
+
+def row_index_attach(dD, row_index):
+    """From now on the named launchers pass `row_index` on when they are handed this D (both stay
+    alive and unchanged while attached); None detaches."""
+    _check("nmspmm_row_index_attach", lib().nmspmm_row_index_attach(_ptr(dD), _ptr(row_index)))
 
 
 def release():

@@ -5,6 +5,7 @@
 
 #include <atomic>
 #include <cmath>
+#include <map>
 #include <mutex>
 #include <vector>
 
@@ -806,6 +807,43 @@ int nmspmm_spmm_noalloc(const float* A, const float* B, const int32_t* D, const 
                      false, nullptr);
 }
 
+// Row lists attached to index buffers (nmspmm_row_index_attach): (device, address of D) -> list.
+// The named launchers look their D up for decode-sized calls; the count lets every other call skip
+// the lock.
+static std::mutex g_attach_mutex;
+static std::map<std::pair<int, const void*>, const int32_t*> g_attached;
+static std::atomic<int> g_attached_count{0};
+
+static const int32_t* attached_row_index(const int32_t* D)
+{
+    if (g_attached_count.load(std::memory_order_acquire) == 0)
+        return nullptr;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess)
+        return nullptr;
+    std::lock_guard<std::mutex> lock(g_attach_mutex);
+    const auto it = g_attached.find({dev, D});
+    return it == g_attached.end() ? nullptr : it->second;
+}
+
+int nmspmm_row_index_attach(const int32_t* dD, const int32_t* row_index)
+{
+    if (!dD)
+        return NMSPMM_ERR_NULL_POINTER;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess)
+        return NMSPMM_ERR_HIP;
+    std::lock_guard<std::mutex> lock(g_attach_mutex);
+    if (row_index)
+        g_attached[{dev, dD}] = row_index;
+    else
+        g_attached.erase({dev, dD});
+    g_attached_count.store((int)g_attached.size(), std::memory_order_release);
+    return NMSPMM_OK;
+}
+
+int nmspmm_row_index_detach(const int32_t* dD) { return nmspmm_row_index_attach(dD, nullptr); }
+
 // `flags`: NMSPMM_ACCUMULATE for the reference launchers' replacements, whose SPLIT_K > 1 adds to C.
 static int named_gemm(int want_high, int tile, const float* A, const float* B, const int32_t* D,
                       const int32_t* column_info, float* C, int M, int N, int K, int W, float sparsity,
@@ -836,7 +874,9 @@ static int named_gemm(int want_high, int tile, const float* A, const float* B, c
         if (rc != NMSPMM_OK)
             return rc;
     }
-    return nmspmm_spmm_ex(A, B, D, want_high ? column_info : nullptr, nullptr, C, M, N, K, W, window, kept, 32, tile,
+    // decode sizes: the row list the caller attached to this D, if any
+    const int32_t* const row_index = M <= 128 ? attached_row_index(D) : nullptr;
+    return nmspmm_spmm_ex(A, B, D, want_high ? column_info : nullptr, row_index, C, M, N, K, W, window, kept, 32, tile,
                           split_k, ws, ws_bytes, flags, stream);
 }
 
@@ -965,6 +1005,11 @@ int nmspmm_gemm_auto(const float* A, const float* B, const int32_t* D, const int
 
 int nmspmm_release(void)
 {
+    {
+        std::lock_guard<std::mutex> attach_lock(g_attach_mutex);
+        g_attached.clear();
+        g_attached_count.store(0, std::memory_order_release);
+    }
     std::lock_guard<std::mutex> lock(g_workspace_mutex);
     int rc = NMSPMM_OK;
     int prev = 0;

@@ -9,6 +9,7 @@ the CPU result and the judge of closeness.  That criterion is ten times tighter 
 bound of the other tests and is relative to each element, which all-positive data makes
 meaningful."""
 import ctypes
+import importlib
 import os
 
 import numpy as np
@@ -113,3 +114,62 @@ def test_sample_of_rows_at_k_4096(cxx, sparsity):
     A_sub = np.ascontiguousarray(d["A_km"][:, rows]).reshape(-1)
     want = ref.gemm_cpu(A_sub, d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), 64, N, K, d["W"])
     assert ref.allclose(np.ascontiguousarray(got[rows]).reshape(-1), want)
+
+
+@pytest.mark.parametrize("M", [1, 16, 32])
+@pytest.mark.parametrize("sparsity", [0.5, 0.75, 0.875])
+def test_named_launchers_take_an_attached_row_list_at_decode_sizes(cxx, M, sparsity):
+    """The reference's signatures have no argument for the row list.  A caller that built one
+    attaches it to its D; from then on the C++ launchers run decode-sized calls on the kernel that
+    reads the list (same bits as nmspmm_spmm_ex with the list), and on the reference-layout kernel
+    again once it is detached.  Both pass the reference's allclose."""
+    nmspmm = importlib.import_module("nm-spmm_amd")
+    ref = Reference()
+    N, K = 1024, 2048
+    d = operands(M, N, K, sparsity, seed=50 + M)
+    W, Q, Ns = d["W"], d["Q"], 128
+    high = sparsity in (0.75, 0.875)
+    want = ref.gemm_cpu(d["A_km"].reshape(-1), d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), M, N, K, W)
+    DT = d["DT"].reshape(-1).copy()
+    window, kept = 32, d["n"]
+    ci = None
+    if high:
+        column_info = np.zeros(((W // kept) * (N // Ns) + 1) * 32 * 2, np.int32)
+        n_ref, m_ref = ctypes.c_int(kept), ctypes.c_int(32)
+        cxx["transIndex"](DT.ctypes.data, W, N, Q, ctypes.byref(n_ref), ctypes.byref(m_ref))
+        kept, window = n_ref.value, m_ref.value
+        cxx["high"](column_info.ctypes.data, window, kept, DT.ctypes.data, W, Q, N, Ns)
+        ci = torch.from_numpy(column_info).cuda()
+    else:
+        cxx["low"](DT.ctypes.data, W, Q, Ns)
+    A, B, D = torch.from_numpy(d["A_km"]).cuda(), torch.from_numpy(d["BT"]).cuda(), torch.from_numpy(DT).cuda()
+    R = torch.empty(nmspmm.row_index_ints(W, N), dtype=torch.int32, device="cuda")
+    nmspmm.row_index_device(D, ci, W, N, window, kept, Ns, R)
+    torch.cuda.synchronize()
+
+    def launch():
+        C = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+        if high:
+            cxx[("huge", True)](A.data_ptr(), B.data_ptr(), D.data_ptr(), ci.data_ptr(), C.data_ptr(), M, N, K, W, sparsity, 1)
+        else:
+            cxx[("huge", False)](A.data_ptr(), B.data_ptr(), D.data_ptr(), C.data_ptr(), M, N, K, W, sparsity, 1)
+        torch.cuda.synchronize()
+        return C, nmspmm.last_kernel()
+
+    plain, family = launch()
+    assert family in ("skinny", "mfma")
+    nmspmm.row_index_attach(D, R)
+    try:
+        listed, family = launch()
+        assert family == "decode"
+        direct = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        nmspmm.spmm_ex(A, B, D, ci, direct, M, N, K, W, window, kept, 32, Ns, 1, None, 0, R)
+        torch.cuda.synchronize()
+        assert torch.equal(listed, direct)
+    finally:
+        nmspmm.row_index_attach(D, None)
+    again, family = launch()
+    assert family in ("skinny", "mfma") and torch.equal(again, plain)
+    for got in (plain, listed):
+        assert ref.allclose(np.ascontiguousarray(got.cpu().numpy()).reshape(-1), want)
