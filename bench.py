@@ -457,13 +457,27 @@ def run_compress(torch, pkg):
     out = []
     for (k, n_cols) in ((4096, 4096), (11008, 4096), (8192, 8192)):
         dense = torch.randn((k, n_cols), dtype=torch.float32, device="cuda")
+        # the yardstick: a plain device-to-device copy of the dense operand (reads and writes it
+        # once), cold in the same way; what fraction of 8 TB/s a kernel that only moves bytes gets
+        pairs = [(dense, torch.empty_like(dense))]
+        while len(pairs) * 2 * dense.numel() * 4 < 640e6 + 2 * dense.numel() * 4:
+            pairs.append((dense.clone(), torch.empty_like(dense)))
+        turn = [0]
+
+        def copy_step():
+            turn[0] = (turn[0] + 1) % len(pairs)
+            pairs[turn[0]][1].copy_(pairs[turn[0]][0])
+
+        cms, _ = time_launches(torch, copy_step, 3 * len(pairs), len(pairs), 0.05)
+        copy = rate_entry(cms * 1e3, 2.0 * dense.numel() * 4, True, 1)
+        del pairs
         for (n, m) in ((2, 4), (2, 8), (1, 8), (8, 32)):
             w, q = k // m * n, n_cols // 32
             bt = torch.empty((w, n_cols), dtype=torch.float32, device="cuda")
             dt = torch.empty((w, q), dtype=torch.int32, device="cuda")
             back = torch.empty_like(dense)
             nbytes = 4.0 * (k * n_cols + w * n_cols + w * q)
-            row = {"K": k, "Ncols": n_cols, "pattern": "%d:%d" % (n, m)}
+            row = {"K": k, "Ncols": n_cols, "pattern": "%d:%d" % (n, m), "plain_copy_of_the_dense_operand": copy}
             for name, fn in (("compress", lambda: pkg.compress_device(dense, k, n_cols, n, m, bt, dt)),
                              ("decompress", lambda: pkg.decompress_device(bt, dt, k, n_cols, n, m, back))):
                 ms, _ = time_launches(torch, fn, 30, 5, 0.05)
@@ -712,6 +726,7 @@ def summarize(configs, preprocess, dispatch):
         name = lambda r: "%dx%d %s" % (r["K"], r["Ncols"], r["pattern"])
         s["compress_frac_hbm"] = digest(configs["compress"], lambda r: r["compress"]["frac_hbm"], name)
         s["decompress_frac_hbm"] = digest(configs["compress"], lambda r: r["decompress"]["frac_hbm"], name)
+        s["plain_copy_frac_hbm"] = digest(configs["compress"], lambda r: r["plain_copy_of_the_dense_operand"]["frac_hbm"], name)[1:4]
     if "rowmajor" in configs:
         s["rowmajor_overhead"] = digest(configs["rowmajor"], lambda r: r["overhead"], shape, higher_is_better=False)
     if "sweep100" in configs:

@@ -119,6 +119,138 @@ decompress_kernel(const float* __restrict__ BT, const int32_t* __restrict__ DT, 
     }
 }
 
+
+// ---- windows of 32 rows with 32-column vectors (the reference's n:32 patterns) ------------------
+// One thread of the kernels above would hold all 32 rows of its four columns (128 registers of
+// values alone): two waves per SIMD, and every wave loads, ranks and stores in turn with nothing
+// to cover it.  Here the window is cut into four quarters of eight rows, one per wave of the
+// workgroup: lane (vector j, position c) of wave q holds rows 8 q .. 8 q + 7 of columns
+// 4 c .. 4 c + 3 of vector j, so a wave instruction still moves 1 KB of one row (eight vectors,
+// 256 columns).  The row scores are summed in the same order as above (inside the thread, then over
+// the eight lanes of the vector by lane exchange); the four waves swap their eight scores per
+// vector through LDS, lane (j, c) of wave q ranks row 8 q + c, and the waves' ballots are put
+// together through LDS to the verdict on all 32 rows.  About 70 registers: six waves per SIMD.
+
+__device__ inline float dpp_quad_1032(float x)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0xB1, 0xF, 0xF, false));
+}
+__device__ inline float dpp_quad_2301(float x)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x4E, 0xF, 0xF, false));
+}
+__device__ inline float dpp_half_mirror(float x)  // lane i of each 8 <- lane 7 - i: the other quad
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x141, 0xF, 0xF, false));
+}
+
+constexpr int kVectorsPerBlock32 = 8;
+
+__global__ void __launch_bounds__(256)
+compress32_kernel(const float* __restrict__ B, float* __restrict__ BT, int32_t* __restrict__ DT, int N, int Q, int n)
+{
+    __shared__ __attribute__((aligned(16))) uint32_t scores[kVectorsPerBlock32][32];
+    __shared__ unsigned char verdict[kVectorsPerBlock32][4];  // byte q: rows 8 q .. 8 q + 7
+    const int w = blockIdx.x;
+    const int lane = threadIdx.x & 63, q = threadIdx.x >> 6;
+    const int c = lane & 7, j = lane >> 3;
+    const int vec = blockIdx.y * kVectorsPerBlock32 + j;
+    const bool active = vec < Q;                          // whole vectors are active or not
+    const int col = vec * 32 + c * 4;
+
+    float4 v[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+        v[r] = active ? *reinterpret_cast<const float4*>(B + ((size_t)w * 32 + q * 8 + r) * N + col)
+                      : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    uint32_t mine8[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        // neighbours at distance 1 and 2 inside the thread, then 4, 8, 16 by lane exchange: in each
+        // exchange both partners add the same two numbers, so all eight lanes end with the same bits
+        float s = (fabsf(v[r].x) + fabsf(v[r].y)) + (fabsf(v[r].z) + fabsf(v[r].w));
+        s += dpp_quad_1032(s);
+        s += dpp_quad_2301(s);
+        s += dpp_half_mirror(s);
+        mine8[r] = __float_as_uint(s);
+    }
+    if (c == 0) {
+        *reinterpret_cast<uint4*>(&scores[j][q * 8]) = make_uint4(mine8[0], mine8[1], mine8[2], mine8[3]);
+        *reinterpret_cast<uint4*>(&scores[j][q * 8 + 4]) = make_uint4(mine8[4], mine8[5], mine8[6], mine8[7]);
+    }
+    __syncthreads();
+    // lane (j, c) of wave q ranks row 8 q + c among the window's 32: larger scores first, equal
+    // scores prefer the lower row; scores are compared as bit patterns (they are sums of
+    // magnitudes, so NaNs rank above everything instead of breaking the order)
+    const int my_row = q * 8 + c;
+    uint32_t key_mine = 0;
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+        key_mine = r == c ? mine8[r] : key_mine;
+    int rank = 0;
+#pragma unroll
+    for (int r4 = 0; r4 < 8; ++r4) {
+        const uint4 k = *reinterpret_cast<const uint4*>(&scores[j][r4 * 4]);
+        const uint32_t ks[4] = {k.x, k.y, k.z, k.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int r = r4 * 4 + e;
+            rank += (ks[e] > key_mine || (ks[e] == key_mine && r < my_row)) ? 1 : 0;
+        }
+    }
+    const unsigned long long votes = __ballot(rank < n);   // bit 8 j + c: row 8 q + c of vector j
+    if (c == 0)
+        verdict[j][q] = (unsigned char)(votes >> (8 * j));
+    __syncthreads();
+    const uint32_t keep = *reinterpret_cast<const uint32_t*>(verdict[j]);   // bit r: row r of the vector is kept
+    if (!active)
+        return;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const int row = q * 8 + r;
+        if ((keep >> row) & 1u) {
+            const int p = __popc(keep & ((1u << row) - 1u));
+            const size_t out = (size_t)w * n + p;
+            *reinterpret_cast<float4*>(BT + out * N + col) = v[r];
+            if (c == r)
+                DT[out * Q + vec] = row;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256)
+decompress32_kernel(const float* __restrict__ BT, const int32_t* __restrict__ DT, float* __restrict__ B, int N, int Q,
+                    int n)
+{
+    const int w = blockIdx.x;
+    const int lane = threadIdx.x & 63, q = threadIdx.x >> 6;
+    const int c = lane & 7, j = lane >> 3;
+    const int vec = blockIdx.y * kVectorsPerBlock32 + j;
+    if (vec >= Q)
+        return;
+    const int col = vec * 32 + c * 4;
+    uint32_t keep = 0;
+    for (int p = 0; p < n; ++p) {
+        const uint32_t r = (uint32_t)DT[((size_t)w * n + p) * Q + vec];
+        if (r < 32u)  // malformed indices must not leave the window
+            keep |= 1u << r;
+    }
+    // every row of the window is written exactly once: a kept row's values or zeros
+    float4 x[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const int row = q * 8 + r;
+        x[r] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if ((keep >> row) & 1u) {
+            const int p = __popc(keep & ((1u << row) - 1u));
+            x[r] = *reinterpret_cast<const float4*>(BT + ((size_t)w * n + p) * N + col);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+        store_segment(B + (size_t)w * 32 * N, 32u * (uint32_t)N * 4u, ((uint32_t)(q * 8 + r) * N + col) * 4u, x[r]);
+}
+
 bool compress_supported(int m, int vec_len)
 {
     return (m == 4 || m == 8 || m == 16 || m == 32) && (vec_len == 4 || vec_len == 8 || vec_len == 16 || vec_len == 32);
@@ -129,6 +261,11 @@ hipError_t launch_compress(const float* B, float* BT, int32_t* DT, int K, int N,
 {
     const dim3 grid(K / m, (N + kColsPerBlock - 1) / kColsPerBlock), block(256);
     const int Q = N / vec_len;
+    if (m == 32 && vec_len == 32 && (Q + kVectorsPerBlock32 - 1) / kVectorsPerBlock32 <= 65535) {
+        const dim3 grid32(K / 32, (Q + kVectorsPerBlock32 - 1) / kVectorsPerBlock32);
+        compress32_kernel<<<grid32, block, 0, stream>>>(B, BT, DT, N, Q, n);
+        return hipGetLastError();
+    }
     switch (m) {
     case 4: compress_kernel<4><<<grid, block, 0, stream>>>(B, BT, DT, N, Q, n, vec_len); break;
     case 8: compress_kernel<8><<<grid, block, 0, stream>>>(B, BT, DT, N, Q, n, vec_len); break;
@@ -144,6 +281,11 @@ hipError_t launch_decompress(const float* BT, const int32_t* DT, float* B, int K
 {
     const dim3 grid(K / m, (N + kColsPerBlock - 1) / kColsPerBlock), block(256);
     const int Q = N / vec_len;
+    if (m == 32 && vec_len == 32 && (Q + kVectorsPerBlock32 - 1) / kVectorsPerBlock32 <= 65535) {
+        const dim3 grid32(K / 32, (Q + kVectorsPerBlock32 - 1) / kVectorsPerBlock32);
+        decompress32_kernel<<<grid32, block, 0, stream>>>(BT, DT, B, N, Q, n);
+        return hipGetLastError();
+    }
     switch (m) {
     case 4: decompress_kernel<4><<<grid, block, 0, stream>>>(BT, DT, B, N, Q, n, vec_len); break;
     case 8: decompress_kernel<8><<<grid, block, 0, stream>>>(BT, DT, B, N, Q, n, vec_len); break;
