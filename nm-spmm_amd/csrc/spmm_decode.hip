@@ -323,25 +323,20 @@ __global__ void __launch_bounds__(64 * kDecodeWaves) spmm_decode_kernel(const De
         if (ticket != (unsigned int)(p.slices - 1))
             return;
         asm volatile("" ::: "memory");
-        for (int x = wave; x < 8 * HB; x += kDecodeWaves) {
-            // the slices' values (at most eight) are requested together and added in slice order
-            float t[8];
-#pragma unroll
-            for (int z = 0; z < 8; ++z)
-                t[z] = z < p.slices ? __hip_atomic_load(&p.part[((size_t)vv * p.slices + z) * kTile + x * 64 + lane],
-                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                                    : 0.0f;
-            float s = 0.0f;
-#pragma unroll
-            for (int z = 0; z < 8; ++z)
-                s += t[z];
-            store_c(x, s);
-        }
-        // The word goes back to zero: a HIP graph that replays this launch carries this launch's
-        // epoch again and must find what the first run found.  (A launch that is cut short leaves
-        // its word behind; the next launch's larger epoch overrides it.)
+        // This is the last arrival, so nobody touches the word again in this launch: it goes back
+        // to zero now (the store travels while the tiles are added up).  A HIP graph that replays
+        // this launch carries this launch's epoch again and must find what the first run found; a
+        // launch that is cut short leaves its word behind and the next launch's larger epoch
+        // overrides it.
         if (tid == 0)
             __hip_atomic_store(&p.tickets[vv], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int x = wave; x < 8 * HB; x += kDecodeWaves) {
+            float s = 0.0f;
+            for (int z = 0; z < p.slices; ++z)
+                s += __hip_atomic_load(&p.part[((size_t)vv * p.slices + z) * kTile + x * 64 + lane], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+            store_c(x, s);
+        }
     }
 }
 
