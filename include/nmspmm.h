@@ -158,14 +158,17 @@ int nmspmm_spmm(const float* A, const float* B, const int32_t* D, const int32_t*
  * NMSPMM_DECODE_SPLIT: with fewer 32-column vectors than the GPU has compute units (Ncols below
  * 8192 on an MI355X) the decode kernel on the row list leaves compute units idle; this flag lets it
  * cut each vector's reduction across several workgroups, the last of which to finish adds the
- * partial sums up in slice order (one launch, reproducible bit for bit).  The partial sums and the
- * arrival counters live in a device-resident array of the library (the one nmspmm_spmm_noalloc
- * uses), one copy per GPU: calls with this flag, and nmspmm_spmm_noalloc calls, that overlap on
- * one GPU (two streams, two threads) race on it, so the flag is for callers that issue their
- * multiplications on one stream.  Measured: K = 11008, Ncols = 4096 at 2:8, 1 / 16 / 32 rows
- * 11.4 / 14.6 / 17.2 -> 10.1 / 11.3 / 12.6 us re-reading one B, 15.5 / 20.1 / 20.8 -> 11.4 / 13.5 /
- * 14.6 us with B from HBM; the library splits only where the model expects a gain (long
- * reductions, at most half as many vectors as compute units).
+ * partial sums up in slice order (one launch, no workgroup waits for another, reproducible bit for
+ * bit, safe to capture in a HIP graph and replay).  The partial sums and the arrival words live in
+ * a device-resident array of the library (the one nmspmm_spmm_noalloc uses), one copy per GPU:
+ * calls with this flag, and nmspmm_spmm_noalloc calls, that overlap on one GPU (two streams, two
+ * threads) race on it, so the flag is for callers that issue their multiplications on one stream.
+ * Nothing has to be cleared between calls, also not after a launch that was cut short: every
+ * launch tags its arrivals with a number that is larger than any earlier launch's.  Measured:
+ * K = 11008, Ncols = 4096 at 2:8, 1 / 16 / 32 rows 12.1 / 13.0 / 15.9 -> 11.0 / 12.3 / 13.2 us
+ * re-reading one B, 16.6 / 20.7 / 20.4 -> 12.7 / 14.7 / 15.8 us with B from HBM; the library splits
+ * only where the model expects a gain (long reductions, at most half as many vectors as compute
+ * units).
  * Any other flag bit: NMSPMM_ERR_BAD_SHAPE.
  * row_index: NULL, or the row list nmspmm_row_index_device() made from these same D / column_info
  * (16-byte aligned).  With it, M <= 32 runs on the decode kernel that reads the list instead of
