@@ -105,3 +105,37 @@ def test_parts_can_be_selected(tmp_path):
     assert list(d["configs"]) == ["fine"] and len(d["configs"]["fine"]) == 2 and d["dispatch"] is None
     bad = subprocess.run([sys.executable, BENCH, "--only", "nonsense"], capture_output=True, text=True, timeout=120)
     assert bad.returncode != 0 and "unknown part" in bad.stderr
+
+
+def test_the_printed_line_stays_short_whatever_the_parts_hold():
+    """The digests of the printed line are built from every part's rows; with rows of the real
+    shape (long case names, wide numbers) for every part the line must stay under 4 KB, and the
+    headline fields must survive the last-resort truncation."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_module", BENCH)
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    shape = {"M": 8192, "K": 11008, "Ncols": 14336, "pattern": "12:32"}
+    rate = lambda hbm: {"us": 12345.67, "gbs": 7999.0, **({"frac_hbm": 0.999} if hbm else {"served_by": "infinity cache"})}
+    decode_row = dict(shape, **{m[0]: rate(m[3]) for m in bench.DECODE_MODES})
+    configs = {
+        "llm": [dict(shape, frac_fp32_mfma_peak=0.999, speedup_over_ideal=1.234)] * 9,
+        "ragged": [dict(shape, frac_fp32_mfma_peak=0.999)] * 9,
+        "decode": [decode_row] * 16, "decode_llm": [decode_row] * 9, "decode_wide": [decode_row] * 8,
+        "fine": [{"pattern": "16:32", "vec_len": 32, "frac_fp32_mfma_peak": 0.999}] * 8,
+        "launch_constant": [{"pattern": "16:32", "constant_us": 10.25}] * 3,
+        "compress": [dict(shape, compress=rate(True), decompress=rate(True), plain_copy_of_the_dense_operand=rate(True))] * 12,
+        "rowmajor": [dict(shape, overhead=0.211)] * 5,
+        "sweep100": {"by_sparsity": {k: {"mean_speedup_vs_dense": 19.268, "min_speedup_vs_dense": 10.123,
+                                         "a100_reference_mean_speedup": 6.34} for k in ("0.5", "0.625", "0.75", "0.875")}},
+    }
+    # fine and launch_constant are keyed by pattern in the digest: give them distinct keys
+    configs["fine"] = [dict(r, pattern="%d:32" % (i + 1)) for i, r in enumerate(configs["fine"])]
+    configs["launch_constant"] = [dict(r, pattern="%d:32" % (i + 1)) for i, r in enumerate(configs["launch_constant"])]
+    preprocess = [{"pattern": "%d:32" % i, "vec_len": 32, "device_one_kernel_ms": 0.0085, "cpu_restatement_wall_ms": 0.832,
+                   "cpu_reference_wall_ms": 0.664} for i in range(4)]
+    dispatch = {"shapes": [0] * 12, "mean_ratio": 1.001, "worst_ratio": 1.013}
+    summary = bench.summarize(configs, preprocess, dispatch)
+    size = len(json.dumps(summary, separators=(",", ":")))
+    assert size <= 2400, size   # the headline fields take about 1.6 KB of the 4 KB
+    assert set(summary) >= {"llm", "ragged", "decode", "decode_llm", "decode_wide", "compress_frac_hbm", "dispatch"}
