@@ -180,6 +180,16 @@ def test_row_list_entry_points_reject_bad_arguments_without_a_gpu():
     assert call(W=60) == 2 and call(N=96) == 2 and call(Ns=48) == 2
 
 
+def test_attaching_a_row_list_checks_its_arguments():
+    """Without a device there is nothing to attach to (the registry is keyed by device), but the
+    argument check comes first; nmspmm_release forgets attachments and never fails for that."""
+    L = nmspmm.lib()
+    assert L.nmspmm_row_index_attach(None, FAKE) == 1 and L.nmspmm_row_index_detach(None) == 1
+    assert L.nmspmm_row_index_attach(FAKE, FAKE) in (0, 7)    # OK with a current device, NMSPMM_ERR_HIP without
+    assert L.nmspmm_row_index_detach(FAKE) in (0, 7)
+    assert L.nmspmm_release() == 0
+
+
 def test_named_entry_points_reject_the_other_family():
     L = nmspmm.lib()
     low = lambda s, tile=128: L.nmspmm_gemm_low_sparsity(tile, FAKE, FAKE, FAKE, FAKE, 128, 128, 128, 64, s, 1, None)
