@@ -23,6 +23,9 @@ def compress_gpu(dense, n, m, vl=32):
     (64, 128, 2, 4, 32), (256, 512, 2, 4, 32), (512, 1120, 1, 8, 32), (256, 96, 3, 8, 32), (128, 288, 2, 8, 32),
     (128, 256, 4, 32, 32), (64, 64, 8, 32, 32), (96, 160, 12, 16, 32), (64, 64, 2, 4, 4), (64, 264, 1, 8, 8),
     (128, 48, 5, 16, 16), (64, 36, 3, 4, 4), (32, 40, 17, 32, 8),
+    # 32-row windows with 32-column vectors (the kernels that cut the window into quarters): one kept
+    # row, nearly all, a column count that leaves the last workgroup with one live vector of eight
+    (96, 1120, 1, 32, 32), (64, 288, 31, 32, 32), (160, 2080, 16, 32, 32), (32, 32, 12, 32, 32),
 ])
 def test_compress_bit_exact_vs_checker(oracle, K, N, n, m, vl):
     rng = np.random.default_rng(K + N + n)
@@ -45,6 +48,29 @@ def test_ties_and_non_finite_scores(oracle):
     assert np.array_equal(DT.cpu().numpy(), want_DT)
     assert np.array_equal(BT.cpu().numpy(), want_BT, equal_nan=True)
     assert want_DT[3:6, 0].tolist() == [0, 1, 5] and want_DT[6:9, 1].tolist() == [0, 1, 6]
+
+
+def test_ties_and_non_finite_scores_in_32_row_windows(oracle):
+    """Equal scores in different quarters of a window (the quarters are ranked by different waves)
+    must still prefer the lower row; NaN and Inf scores rank above everything."""
+    K, N, n, m = 64, 96, 5, 32
+    host = np.ones((K, N), np.float32)
+    host[::3] *= -1.0
+    host[7, 40] = np.inf
+    host[29, 70] = np.nan
+    host[40:44, :32] = 2.0      # four equal larger rows in the second window's second quarter
+    BT, DT = compress_gpu(torch.from_numpy(host).cuda(), n, m)
+    want_BT, want_DT = oracle.compress(host, n, m)
+    assert np.array_equal(DT.cpu().numpy(), want_DT)
+    assert np.array_equal(BT.cpu().numpy(), want_BT, equal_nan=True)
+    assert want_DT[:5, 0].tolist() == [0, 1, 2, 3, 4] and want_DT[5:10, 0].tolist() == [0, 8, 9, 10, 11]
+    back = torch.empty((K, N), dtype=torch.float32, device="cuda")
+    nmspmm.decompress_device(BT, DT, K, N, n, m, back)
+    torch.cuda.synchronize()
+    want_back = oracle.decompress(np.ascontiguousarray(want_BT.T).reshape(-1),
+                                  np.ascontiguousarray((want_DT + (np.arange(want_DT.shape[0]) // n * m)[:, None]).T.astype(np.int32)).reshape(-1),
+                                  K, N, want_BT.shape[0])
+    assert np.array_equal(back.cpu().numpy(), want_back, equal_nan=True)
 
 
 @pytest.mark.parametrize("n,m", [(2, 4), (3, 8), (2, 8), (1, 8), (8, 32)])
