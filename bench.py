@@ -892,7 +892,14 @@ def main():
         "sweep": sweep,
     }
     detail = dict(out, configs=configs, preprocess=preprocess, dispatch=dispatch)
-    with open(args.detail, "w") as f:
+    detail_path = args.detail
+    try:
+        f = open(detail_path, "w")
+    except OSError:  # a read-only tree: the line is still printed, the cases go beside the system's temporary files
+        import tempfile
+        detail_path = os.path.join(tempfile.gettempdir(), "bench_detail.json")
+        f = open(detail_path, "w")
+    with f:
         json.dump(detail, f, indent=1)
         f.write("\n")
     # the line itself stays short (harnesses keep only the last few KB of a run's output): the
@@ -900,7 +907,7 @@ def main():
     out["sweep"] = {k: {f: v[f] for f in ("ms", "useful_tflops", "frac_fp32_mfma_peak", "speedup_vs_dense")}
                     for k, v in sweep.items()}
     out["summary"] = summarize(configs, preprocess, dispatch)
-    out["detail_file"] = os.path.relpath(args.detail, ROOT) if os.path.abspath(args.detail).startswith(ROOT) else args.detail
+    out["detail_file"] = os.path.relpath(detail_path, ROOT) if os.path.abspath(detail_path).startswith(ROOT) else detail_path
     line = json.dumps(out, separators=(",", ":"))
     while len(line) > MAX_LINE_BYTES and out["summary"]:   # never at today's part list; the headline fields stay whatever happens
         out["summary"].popitem()
