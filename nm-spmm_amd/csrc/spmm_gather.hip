@@ -12,12 +12,22 @@
 // Every MFMA needs 64 fresh values of A (4 rows for each of 16 blocks), so the kernel is bound by
 // how fast those are delivered, not by the matrix pipes: gathered straight from global memory the
 // vector L1 caps it at 42 useful TFLOP/s.  Here the four waves of a workgroup share 64 rows of C and
-// stage a chunk of 64 (32) dense rows of A in LDS, k-major with a 32-byte skew per dense row; lane
-// (b, i) reads rows 16q + 4i .. 4i+3 of its block's dense row with one ds_read_b128, which feeds four
-// MFMAs, and the value of B it needs (one 32-bit load per kept row) is reused by all sixteen MFMAs of
-// the step.  Index and B value are loaded eight steps ahead, the next chunk of A is fetched into
-// registers while the current one is multiplied.  Measured at 4096 cubed with vectors of 4 columns:
-// 1:8 85, 2:8 93, 2:4 93 useful TFLOP/s, where the expanding kernel reaches 18, 36 and 71.
+// stage a chunk of dense rows of A in LDS, k-major with a skew per dense row (64 bytes for 4-row
+// windows, where it removes every bank conflict; 32 for the others); lane (b, i) reads rows
+// 16q + 4i .. 4i+3 of its block's dense row with one ds_read_b128, which feeds four MFMAs, through
+// a ring of four such reads that is kept three reads ahead of the MFMAs.
+//
+// A chunk is as many dense rows as hold eight kept rows (a "phase": 16 to 64 rows).  The phase's
+// indices and values of B do not come through registers: two global loads per step cost the matrix
+// pipes 14 % of their time however far ahead they are issued (measured in isolation), an LDS read
+// about a cycle.  Each wave copies two of the phase's eight rows of B (the workgroup's 256 columns,
+// one 128-bit LDS-direct load per row) and their indices straight into one half of a small
+// double-buffered LDS area a phase ahead, and every lane reads its index and value from there; the
+// next chunk of A is fetched into registers while the current one is multiplied and stored between
+// the two barriers that end the chunk.  The GPU does not hold its 2.4 GHz under this kernel (LDS and
+// matrix pipes both busy: about 2.1 GHz at 2:4), so fewer instructions and fewer LDS cycles also
+// mean a higher clock.  Measured at 4096 cubed with vectors of 4 columns: 2:4 105, 2:8 97, 1:8 87
+// useful TFLOP/s, where the expanding kernel reaches 71, 36 and 18.
 #include "internal.h"
 
 namespace nmspmm {
@@ -34,7 +44,7 @@ struct GatherParams {
     int lshift;   // log2(vector length / 4): 4-column groups per vector
     int Qs;       // vectors per preprocessed column block
     int tiles_m;
-    int nchunk;   // chunks of kGatherChunk dense rows in the whole reduction
+    int nchunk;   // chunks of gather_chunk(window, kept) dense rows in the whole reduction
     int split_k;
 };
 
@@ -45,11 +55,27 @@ __device__ inline __amdgpu_buffer_rsrc_t gather_rsrc(const void* base, uint32_t 
 
 constexpr int kGatherRows = 64;     // rows of C per workgroup
 constexpr int kGatherCols = 256;    // columns of C per workgroup: four waves of 64
-constexpr int kGatherAhead = 8;     // steps by which index and B value are loaded ahead
+constexpr int kGatherPhase = 8;     // steps (kept rows) whose index and B value sit in one half of the meta buffers
 constexpr uint32_t kGatherNoLoad = 0x80000000u;  // beyond every descriptor here: loads 0
 
-template <int MWIN>
-struct GatherChunk { static constexpr int value = MWIN == 4 ? 32 : 64; };
+// Dense rows of A per chunk: as many as hold one phase of eight kept rows (16 to 64), so that a
+// chunk is one phase; 3:8 has no such size and takes 64 rows = three phases.
+constexpr int gather_chunk(int window, int kept) { return (8 * window) % kept == 0 ? 8 * window / kept : 64; }
+
+typedef __attribute__((address_space(3))) float gather_lds_f32;
+typedef __attribute__((address_space(3))) int32_t gather_lds_i32;
+
+// Global -> LDS loads without a register stop-over: lane l's 16 (4) bytes land at dst + 16 l
+// (dst + 4 l); dst is wave-uniform; completion is counted in vmcnt.  Kept out of the kernel
+// template: the host pass drops a kernel template that names the builtin directly.
+__device__ inline void gather_row_to_lds(__amdgpu_buffer_rsrc_t r, gather_lds_f32* dst, uint32_t v_off, uint32_t s_off)
+{
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, dst, 16, v_off, s_off, 0, 0);
+}
+__device__ inline void gather_word_to_lds(__amdgpu_buffer_rsrc_t r, gather_lds_i32* dst, uint32_t v_off, uint32_t s_off)
+{
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, dst, 4, v_off, s_off, 0, 0);
+}
 
 // MWIN: rows per window (4, 8, 16), NK: kept rows per window.
 template <int MWIN, int NK>
@@ -57,14 +83,23 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
 {
     constexpr int R = kGatherRows;
     constexpr int RB = R / 16;                       // 128-bit LDS reads per lane and step
-    constexpr int KC = GatherChunk<MWIN>::value;     // dense rows per chunk
-    constexpr int STRIDE = R * 4 + 32;               // bytes per dense row in LDS
+    constexpr int KC = gather_chunk(MWIN, NK);       // dense rows per chunk
+    // bytes per dense row in LDS.  A pass of a 128-bit LDS read serves 16 lanes, i.e. four blocks of
+    // 64 bytes, out of 64 banks: with a 64-byte skew the rows k, k + 1, k + 2, k + 3 of a 4-row window
+    // fall into the four quarters of the banks and no read conflicts; windows of 8 and 16 rows
+    // conflict either way and keep the 32-byte skew that measured best for them
+    constexpr int STRIDE = R * 4 + (MWIN == 4 ? 64 : 32);
     constexpr int SEGS = KC * 4 * RB;                // 16-byte segments per chunk
     constexpr int SPT = SEGS / 256;                  // per thread
     constexpr int STEPS = KC / MWIN * NK;            // kept rows per chunk: one step each
-    constexpr int PF = kGatherAhead;
-    static_assert(SEGS % 256 == 0 && STEPS % PF == 0, "chunk geometry");
+    constexpr int PH = kGatherPhase;
+    constexpr int P = STEPS / PH;                    // phases per chunk
+    static_assert(SEGS % 256 == 0 && STEPS % PH == 0, "chunk geometry");
+    // A's chunk; and, twice (the phase being multiplied and the next one), a phase's values of B (a
+    // row of the workgroup's 256 columns per step) and its indices (one per step and vector)
     __shared__ __attribute__((aligned(16))) unsigned char lds[KC * STRIDE];
+    __shared__ __attribute__((aligned(16))) float lds_b[2 * PH * kGatherCols];
+    __shared__ __attribute__((aligned(16))) int32_t lds_i[2 * PH * 64];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -73,48 +108,64 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
     const int row0 = tile_m * R;
     const int M = p.M, N = p.N, W = p.W, lda = p.lda;
     // a wave beyond the last column repeats the last 64 columns (it has to reach the barriers)
-    const int col0 = min(tile_n * kGatherCols + wave * 64, N - 64);
-    // this slice's chunks: everything below counts chunks and steps from the slice's first one
+    const int colwg = tile_n * kGatherCols;
+    const int col0 = min(colwg + wave * 64, N - 64);
+    // this slice's chunks: everything below counts chunks, phases and steps from the slice's first one
     int c_begin, c_count;
     split_windows(p.nchunk, p.split_k, blockIdx.y, &c_begin, &c_count);
-    const int s_begin = c_begin * STEPS, s_count = c_count * STEPS;
+    const int s_begin = c_begin * STEPS;
+    const int phases = c_count * P;
 
     const size_t K = (size_t)p.nchunk * KC;
     const __amdgpu_buffer_rsrc_t ra = gather_rsrc(p.A, (uint32_t)(K * lda * sizeof(float)));
-    const __amdgpu_buffer_rsrc_t rb = gather_rsrc(p.B + (size_t)s_begin * N + col0,
-                                                  (uint32_t)(((size_t)(W - 1 - s_begin) * N + 64) * sizeof(float)));
+    // B from this slice's first kept row and this workgroup's first column on
+    const __amdgpu_buffer_rsrc_t rb = gather_rsrc(p.B + (size_t)s_begin * N + colwg,
+                                                  (uint32_t)(((size_t)(W - 1 - s_begin) * N + (N - colwg)) * sizeof(float)));
     const __amdgpu_buffer_rsrc_t rd = gather_rsrc(p.D, (uint32_t)((size_t)W * (N >> (2 + p.lshift)) * sizeof(int32_t)));
     const uint32_t b_row = (uint32_t)N * 4u, d_row = (uint32_t)p.Qs * 4u;
-    // D is blocked [N / Ns][W][Qs]: this block's vector is (col0 + 4b) / L
+    // D is blocked [N / Ns][W][Qs].  The workgroup's 256 columns hold nv = 256 / L vectors; lane l
+    // fetches the index of vector l % nv (a vector beyond the last column: the last one)
     const int Ns = p.Qs << (2 + p.lshift);
-    const int col = col0 + 4 * b;
-    const uint32_t d_lane = (uint32_t)(((size_t)(col / Ns) * W * p.Qs + (size_t)s_begin * p.Qs + ((col % Ns) >> (2 + p.lshift))) *
+    const int nv = 64 >> p.lshift;
+    const int vcol = min(colwg + ((lane & (nv - 1)) << (2 + p.lshift)), N - (4 << p.lshift));
+    const uint32_t d_lane = (uint32_t)(((size_t)(vcol / Ns) * W * p.Qs + (size_t)s_begin * p.Qs + ((vcol % Ns) >> (2 + p.lshift))) *
                                        sizeof(int32_t));
-    const uint32_t b_lane = (uint32_t)lane * 4u;
-
-    // chunk copy: segment tid + 256 j is 16 bytes (4 rows) of dense row seg / 16 of the chunk
-    uint32_t cp_src[SPT], cp_dst[SPT];
+    // Phase g (eight steps of the slice) into half g & 1 of the meta buffers: step s's row of B to
+    // lds_b[half][s][0 .. 255] (one instruction of one wave; columns beyond the matrix read the next
+    // row or, behind the last one, zeros: no wave uses them) and its indices to lds_i[half][s][0 .. 63]
+    // (entry l: vector l % nv).  The uniform part of both addresses is a scalar offset.
+    auto fetch_meta = [&](int g) {
+        const int half = g & 1;
 #pragma unroll
-    for (int j = 0; j < SPT; ++j) {
-        const int seg = tid + 256 * j, kk = seg / (4 * RB), part = seg % (4 * RB);
-        cp_src[j] = (uint32_t)((((size_t)c_begin * KC + kk) * lda + row0 + part * 4) * sizeof(float));
-        cp_dst[j] = (uint32_t)(kk * STRIDE + part * 16);
-    }
+        for (int s0 = 0; s0 < PH; s0 += 4) {
+            const int s = s0 + wave;
+            const uint32_t step = (uint32_t)(g * PH + s);
+            gather_row_to_lds(rb, (gather_lds_f32*)lds_b + (half * PH + s) * kGatherCols, (uint32_t)lane * 16u, step * b_row);
+            gather_word_to_lds(rd, (gather_lds_i32*)lds_i + (half * PH + s) * 64, d_lane, step * d_row);
+        }
+    };
+
+    // chunk copy: segment tid + 256 j is 16 bytes (4 rows) of dense row seg / 16 of the chunk, i.e.
+    // thread tid's segments lie 16 dense rows apart: one vector offset each for source and
+    // destination, the rest is uniform (scalar offset of the load, immediate of the LDS write)
+    static_assert(RB == 4, "a dense row is sixteen 16-byte segments");
+    const uint32_t cp_src = (uint32_t)((((size_t)c_begin * KC + (tid >> 4)) * lda + row0 + (tid & 15) * 4) * sizeof(float));
+    const uint32_t cp_dst = (uint32_t)((tid >> 4) * STRIDE + (tid & 15) * 16);
     const uint32_t chunk_bytes = (uint32_t)((size_t)KC * lda * sizeof(float));
+    const uint32_t seg_bytes = (uint32_t)((size_t)16 * lda * sizeof(float));
     gfloatx4 stage[SPT];
     // rows beyond M are read as whatever follows them in A (or 0 beyond its end): never stored
     auto fetch_chunk = [&](int c) {
 #pragma unroll
         for (int j = 0; j < SPT; ++j) {
-            const auto x = __builtin_amdgcn_raw_buffer_load_b128(
-                ra, c < c_count ? cp_src[j] + (uint32_t)c * chunk_bytes : kGatherNoLoad, 0, 0);
+            const auto x = __builtin_amdgcn_raw_buffer_load_b128(ra, cp_src, (uint32_t)c * chunk_bytes + (uint32_t)j * seg_bytes, 0);
             stage[j] = gfloatx4{__int_as_float(x[0]), __int_as_float(x[1]), __int_as_float(x[2]), __int_as_float(x[3])};
         }
     };
     auto store_chunk = [&]() {
 #pragma unroll
         for (int j = 0; j < SPT; ++j)
-            *(gfloatx4*)(lds + cp_dst[j]) = stage[j];
+            *(gfloatx4*)(lds + cp_dst + j * 16 * STRIDE) = stage[j];
     };
 
     gfloatx4 acc[4 * RB];
@@ -122,57 +173,82 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
     for (int r = 0; r < 4 * RB; ++r)
         acc[r] = {0.0f, 0.0f, 0.0f, 0.0f};
 
-    // step s = kept row s of the slice.  The uniform part of both addresses is a scalar offset
-    // (not covered by the descriptor's range check: steps outside the slice take the vector offset
-    // that is out of range instead).
-    int idx[PF];
-    float bv[PF];
-    auto load_meta = [&](int s, int slot) {
-        const bool ok = s < s_count;
-        idx[slot] = __builtin_amdgcn_raw_buffer_load_b32(rd, ok ? d_lane : kGatherNoLoad, ok ? (uint32_t)s * d_row : 0u, 0);
-        bv[slot] = __int_as_float(
-            __builtin_amdgcn_raw_buffer_load_b32(rb, ok ? b_lane : kGatherNoLoad, ok ? (uint32_t)s * b_row : 0u, 0));
-    };
-    float a[2][4 * RB];
+    // this lane's column and its block's vector within the workgroup's meta rows
+    const int rel = col0 - colwg;
+    const int my_b = rel + lane, my_v = ((rel >> 2) + b) >> p.lshift;
     const uint32_t l_lane = (uint32_t)(i * 16);
-    // step t of the chunk lies in window t / NK of it; lane (b, i), read q: rows 16 q + 4 i .. 4 i + 3
-    auto read_a = [&](int t, int k_local, float (&dst)[4 * RB]) {
-        const uint32_t off = (uint32_t)((t / NK) * MWIN + k_local) * STRIDE + l_lane;
-#pragma unroll
-        for (int q = 0; q < RB; ++q) {
-            const gfloatx4 x = *(const gfloatx4*)(lds + off + q * 64);
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                dst[4 * q + e] = x[e];
-        }
+    // The A operands travel through a ring of kRing quarter-steps (one 128-bit read = the operands
+    // of four MFMAs): the read for quarter j + kRing - 1 is issued right before the MFMAs of quarter
+    // j, i.e. kRing - 1 groups of four 8-cycle MFMAs ahead of its use, with 4 kRing registers.
+    constexpr int kRing = 4;
+    gfloatx4 ring[kRing];
+    // step t of the chunk lies in window t / NK of it; lane (b, i), quarter q: rows 16 q + 4 i .. 4 i + 3.
+    // One full-rate multiply-add per step; the window's offset is an immediate of the read.
+    auto row_offset = [&](int k_local) { return __umul24((uint32_t)k_local, (uint32_t)STRIDE) + l_lane; };
+    auto read_quarter = [&](int t, int q, uint32_t off) {
+        return *(const gfloatx4*)(lds + off + (t / NK) * MWIN * STRIDE + q * 64);
     };
 
-#pragma unroll
-    for (int t = 0; t < PF; ++t)
-        load_meta(t, t);
+    // No vector-memory instruction between the MFMAs of a phase except the fetches for the next
+    // phase and chunk, which nothing in the phase waits for: index and B value come from LDS.
+    // (Measured: two 32-bit global loads per step cost the matrix pipes 14 % of their time however
+    // far ahead they are issued; an LDS read costs about one cycle.)
+    fetch_meta(0);
     fetch_chunk(0);
     store_chunk();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's rows of B and indices have landed in LDS
     __syncthreads();
     for (int c = 0; c < c_count; ++c) {
-        fetch_chunk(c + 1);
-        const int s_base = c * STEPS;
-        read_a(0, idx[0], a[0]);
+        if (c + 1 < c_count)
+            fetch_chunk(c + 1);   // into registers: A has one buffer, stored after the chunk's last barrier
 #pragma unroll
-        for (int t0 = 0; t0 < STEPS; t0 += PF) {
+        for (int h = 0; h < P; ++h) {
+            const int g = c * P + h, half = g & 1;
+            if (g + 1 < phases)
+                fetch_meta(g + 1);   // the other half: free since the barrier that ended the phase before
+            const float* const mb = lds_b + half * PH * kGatherCols + my_b;
+            const int32_t* const mi = lds_i + half * PH * 64 + my_v;
+            // quarter j of the phase = step j / 4, rows 16 (j % 4) ..; off[] holds the row offsets of
+            // the steps whose quarters are in flight (at most two steps at a time)
+            constexpr int Q = PH * 4;
+            static_assert(kRing <= 9, "reads reach at most two steps ahead");
+            // row offsets of this step and the two after it
+            uint32_t off0 = row_offset(mi[0]), off1 = PH > 1 ? row_offset(mi[64]) : 0u, off2 = PH > 2 ? row_offset(mi[128]) : 0u;
+            float bv_cur = mb[0], bv_next = 0.0f;
 #pragma unroll
-            for (int t = 0; t < PF; ++t) {
-                const int tt = t0 + t;
-                if (tt + 1 < STEPS)
-                    read_a(tt + 1, idx[(t + 1) % PF], a[(t + 1) & 1]);
-                const float bval = bv[t];
+            for (int j = 0; j < kRing - 1; ++j)
+                ring[j] = read_quarter(h * PH + j / 4, j % 4, j / 4 == 0 ? off0 : j / 4 == 1 ? off1 : off2);
 #pragma unroll
-                for (int r = 0; r < 4 * RB; ++r)
-                    acc[r] = __builtin_amdgcn_mfma_f32_4x4x1f32(a[t & 1][r], bval, acc[r], 0, 0, 0);
-                load_meta(s_base + tt + PF, t);
+            for (int j = 0; j < Q; ++j) {
+                const int t = j / 4, q = j % 4;
+                const int ahead = j + kRing - 1;       // the quarter whose read is issued now
+                if (ahead < Q)
+                    ring[ahead % kRing] = read_quarter(h * PH + ahead / 4, ahead % 4,
+                                                       ahead / 4 == t ? off0 : ahead / 4 == t + 1 ? off1 : off2);
+                if (q == 0 && t + 1 < PH)
+                    bv_next = mb[(t + 1) * kGatherCols];
+                __builtin_amdgcn_sched_barrier(0);  // reads are issued where they are written, ahead of these MFMAs
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    acc[4 * q + e] = __builtin_amdgcn_mfma_f32_4x4x1f32(ring[j % kRing][e], bv_cur, acc[4 * q + e], 0, 0, 0);
+                if (q == 3) {          // the step is over: shift the per-step values
+                    bv_cur = bv_next;
+                    off0 = off1;
+                    off1 = off2;
+                    if (t + 3 < PH)
+                        off2 = row_offset(mi[(t + 3) * 64]);
+                }
+            }
+            if (h + 1 < P) {
+                // the next phase's meta rows have landed (this wave's part) and every wave is done
+                // with this phase's half, which the phase after next overwrites
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
             }
         }
-        __syncthreads();
+        __syncthreads();  // every wave is done with A's chunk and with the last phase's half
         store_chunk();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
 
@@ -197,7 +273,7 @@ bool gather_supported(const SpmmArgs& a)
         return false;
     if (a.vec_len != 4 && a.vec_len != 8 && a.vec_len != 16)
         return false;
-    const int chunk = a.window == 4 ? 32 : 64;
+    const int chunk = gather_chunk(a.window, a.kept);
     if (a.N % 64 != 0 || a.Ns % a.vec_len != 0 || a.N % a.Ns != 0 || a.K % chunk != 0 || a.M < 1 || a.lda < a.M)
         return false;
     if (a.split_k < 1 || a.split_k > a.K / chunk)
@@ -226,7 +302,7 @@ static hipError_t launch_gather_cfg(const SpmmArgs& a)
     p.lshift = a.vec_len == 4 ? 0 : a.vec_len == 8 ? 1 : 2;
     p.Qs = a.Ns / a.vec_len;
     p.tiles_m = (a.M + kGatherRows - 1) / kGatherRows;
-    p.nchunk = a.K / GatherChunk<MWIN>::value;
+    p.nchunk = a.K / gather_chunk(MWIN, NK);
     p.split_k = a.split_k;
     const int tiles_n = (a.N + kGatherCols - 1) / kGatherCols;
     const dim3 grid((unsigned)(p.tiles_m * tiles_n), (unsigned)a.split_k);
