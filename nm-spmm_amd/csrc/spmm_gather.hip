@@ -12,8 +12,8 @@
 // Every MFMA needs 64 fresh values of A (4 rows for each of 16 blocks), so the kernel is bound by
 // how fast those are delivered, not by the matrix pipes: gathered straight from global memory the
 // vector L1 caps it at 42 useful TFLOP/s.  Here the four waves of a workgroup share 64 rows of C and
-// stage a chunk of dense rows of A in LDS, k-major with a skew per dense row (64 bytes for 4-row
-// windows, where it removes every bank conflict; 32 for the others); lane (b, i) reads rows
+// stage a chunk of dense rows of A in LDS, k-major with a 64-byte skew per dense row (no bank
+// conflict in 4-row windows, few in larger ones); lane (b, i) reads rows
 // 16q + 4i .. 4i+3 of its block's dense row with one ds_read_b128, which feeds four MFMAs, through
 // a ring of four such reads that is kept three reads ahead of the MFMAs.
 //
@@ -85,10 +85,10 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
     constexpr int RB = R / 16;                       // 128-bit LDS reads per lane and step
     constexpr int KC = gather_chunk(MWIN, NK);       // dense rows per chunk
     // bytes per dense row in LDS.  A pass of a 128-bit LDS read serves 16 lanes, i.e. four blocks of
-    // 64 bytes, out of 64 banks: with a 64-byte skew the rows k, k + 1, k + 2, k + 3 of a 4-row window
-    // fall into the four quarters of the banks and no read conflicts; windows of 8 and 16 rows
-    // conflict either way and keep the 32-byte skew that measured best for them
-    constexpr int STRIDE = R * 4 + (MWIN == 4 ? 64 : 32);
+    // 64 bytes, out of 64 banks: with a 64-byte skew the rows k, k + 1, k + 2, k + 3 fall into the four
+    // quarters of the banks, so a 4-row window never conflicts and in larger windows only rows 4, 8
+    // or 12 apart do (with 32 bytes neighbours overlap by half: 1:8 ran 4 % slower)
+    constexpr int STRIDE = R * 4 + 64;
     constexpr int SEGS = KC * 4 * RB;                // 16-byte segments per chunk
     constexpr int SPT = SEGS / 256;                  // per thread
     constexpr int STEPS = KC / MWIN * NK;            // kept rows per chunk: one step each
