@@ -17,8 +17,8 @@
 // 16q + 4i .. 4i+3 of its block's dense row with one ds_read_b128, which feeds four MFMAs, through
 // a ring of four such reads that is kept three reads ahead of the MFMAs.
 //
-// A chunk is as many dense rows as hold eight kept rows (a "phase": 16 to 64 rows).  The phase's
-// indices and values of B do not come through registers: two global loads per step cost the matrix
+// A chunk (32 dense rows for 4-row windows, 64 otherwise) is one to four "phases" of eight kept
+// rows.  A phase's indices and values of B do not come through registers: two global loads per step cost the matrix
 // pipes 14 % of their time however far ahead they are issued (measured in isolation), an LDS read
 // about a cycle.  Each wave copies two of the phase's eight rows of B (the workgroup's 256 columns,
 // one 128-bit LDS-direct load per row) and their indices straight into one half of a small
@@ -58,9 +58,8 @@ constexpr int kGatherCols = 256;    // columns of C per workgroup: four waves of
 constexpr int kGatherPhase = 8;     // steps (kept rows) whose index and B value sit in one half of the meta buffers
 constexpr uint32_t kGatherNoLoad = 0x80000000u;  // beyond every descriptor here: loads 0
 
-// Dense rows of A per chunk: as many as hold one phase of eight kept rows (16 to 64), so that a
-// chunk is one phase; 3:8 has no such size and takes 64 rows = three phases.
-constexpr int gather_chunk(int window, int kept) { return (8 * window) % kept == 0 ? 8 * window / kept : 64; }
+// Dense rows of A per chunk: 32 for 4-row windows, 64 otherwise: one to four phases of eight kept rows.
+constexpr int gather_chunk(int window, int kept) { return window == 4 ? 32 : 64; }
 
 typedef __attribute__((address_space(3))) float gather_lds_f32;
 typedef __attribute__((address_space(3))) int32_t gather_lds_i32;
@@ -184,7 +183,7 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
     gfloatx4 ring[kRing];
     // step t of the chunk lies in window t / NK of it; lane (b, i), quarter q: rows 16 q + 4 i .. 4 i + 3.
     // One full-rate multiply-add per step; the window's offset is an immediate of the read.
-    auto row_offset = [&](int k_local) { return __umul24((uint32_t)k_local, (uint32_t)STRIDE) + l_lane; };
+    auto row_offset = [&](int k_local, uint32_t base) { return __umul24((uint32_t)k_local, (uint32_t)STRIDE) + base; };
     auto read_quarter = [&](int t, int q, uint32_t off) {
         return *(const gfloatx4*)(lds + off + (t / NK) * MWIN * STRIDE + q * 64);
     };
@@ -201,9 +200,15 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
     for (int c = 0; c < c_count; ++c) {
         if (c + 1 < c_count)
             fetch_chunk(c + 1);   // into registers: A has one buffer, stored after the chunk's last barrier
-#pragma unroll
+        // The phases of a chunk run as a loop (its body is the eight steps, unrolled): a phase starts
+        // on a window boundary whenever eight is a multiple of the kept rows per window, and then only
+        // the base of its LDS offsets changes.  (3:8: windows straddle phases, the loop is unrolled.)
+        constexpr bool kRolled = PH % NK == 0;
+#pragma unroll(kRolled ? 1 : P)
         for (int h = 0; h < P; ++h) {
             const int g = c * P + h, half = g & 1;
+            const int hs = kRolled ? 0 : h;   // compile-time step base of the phase (rolled: in l_phase)
+            const uint32_t l_phase = l_lane + (kRolled ? (uint32_t)(h * (PH / NK) * MWIN * STRIDE) : 0u);
             if (g + 1 < phases)
                 fetch_meta(g + 1);   // the other half: free since the barrier that ended the phase before
             const float* const mb = lds_b + half * PH * kGatherCols + my_b;
@@ -213,17 +218,18 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
             constexpr int Q = PH * 4;
             static_assert(kRing <= 9, "reads reach at most two steps ahead");
             // row offsets of this step and the two after it
-            uint32_t off0 = row_offset(mi[0]), off1 = PH > 1 ? row_offset(mi[64]) : 0u, off2 = PH > 2 ? row_offset(mi[128]) : 0u;
+            uint32_t off0 = row_offset(mi[0], l_phase), off1 = PH > 1 ? row_offset(mi[64], l_phase) : 0u,
+                     off2 = PH > 2 ? row_offset(mi[128], l_phase) : 0u;
             float bv_cur = mb[0], bv_next = 0.0f;
 #pragma unroll
             for (int j = 0; j < kRing - 1; ++j)
-                ring[j] = read_quarter(h * PH + j / 4, j % 4, j / 4 == 0 ? off0 : j / 4 == 1 ? off1 : off2);
+                ring[j] = read_quarter(hs * PH + j / 4, j % 4, j / 4 == 0 ? off0 : j / 4 == 1 ? off1 : off2);
 #pragma unroll
             for (int j = 0; j < Q; ++j) {
                 const int t = j / 4, q = j % 4;
                 const int ahead = j + kRing - 1;       // the quarter whose read is issued now
                 if (ahead < Q)
-                    ring[ahead % kRing] = read_quarter(h * PH + ahead / 4, ahead % 4,
+                    ring[ahead % kRing] = read_quarter(hs * PH + ahead / 4, ahead % 4,
                                                        ahead / 4 == t ? off0 : ahead / 4 == t + 1 ? off1 : off2);
                 if (q == 0 && t + 1 < PH)
                     bv_next = mb[(t + 1) * kGatherCols];
@@ -236,7 +242,7 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
                     off0 = off1;
                     off1 = off2;
                     if (t + 3 < PH)
-                        off2 = row_offset(mi[(t + 3) * 64]);
+                        off2 = row_offset(mi[(t + 3) * 64], l_phase);
                 }
             }
             if (h + 1 < P) {

@@ -235,9 +235,8 @@ def test_short_vectors_on_the_matrix_cores(oracle, vl, n, m, Ns, M, split_k):
 @pytest.mark.parametrize("vl,n,m,Ns", [(4, 2, 4, 128), (8, 1, 8, 64), (16, 4, 16, 32), (4, 3, 4, 128)])
 @pytest.mark.parametrize("M,split_k", [(64, 1), (301, 2)])
 def test_short_vectors_on_the_expanding_kernel(oracle, vl, n, m, Ns, M, split_k):
-    """A reduction that is whole 16-row chunks but not whole chunks of the gathering kernel (as many
-    dense rows as hold eight kept rows: 16 at 2:4, 64 at 1:8, 32 at 4:16) stays on the expanding
-    kernel at any density; at 2:4 every such reduction is whole gathering chunks too."""
+    """A reduction that is whole 16-row chunks but not whole 64-row (32-row) chunks stays on the
+    expanding kernel at any density."""
     N, K = 256, 528
     d = datagen.init_data(M, N, K, n, m, vec_len=vl, seed=vl + n + M)
     W, Q = d["W"], d["Q"]
@@ -248,7 +247,7 @@ def test_short_vectors_on_the_expanding_kernel(oracle, vl, n, m, Ns, M, split_k)
     nmspmm.spmm(dev(d["A_km"]), dev(d["BT"]), dev(D), None, C, M, N, K, W, m, n, vl, Ns, split_k,
                 ws if split_k > 1 else None)
     torch.cuda.synchronize()
-    assert nmspmm.last_kernel() == ("gather" if (n, m) == (2, 4) else "short")
+    assert nmspmm.last_kernel() == "short"
     check(oracle, d, C.cpu().numpy())
 
 
@@ -264,7 +263,7 @@ def test_gathering_kernel_every_pattern_and_vector_length(oracle, vl, n, m, M, N
     W, Q = d["W"], d["Q"]
     D = d["DT"].reshape(-1).copy()
     oracle.preprocess_low(D, W, Q, Ns, vl)
-    chunk = 8 * m // n if (8 * m) % n == 0 else 64   # dense rows that hold eight kept rows (3:8: 64)
+    chunk = 32 if m == 4 else 64
     split_k = min(split_k, K // chunk)
     C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
     ws = torch.empty(max(nmspmm.workspace_bytes(M, N, split_k) // 4, 1), dtype=torch.float32, device="cuda")
