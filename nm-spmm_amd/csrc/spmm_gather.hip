@@ -175,7 +175,11 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
     // this lane's column and its block's vector within the workgroup's meta rows
     const int rel = col0 - colwg;
     const int my_b = rel + lane, my_v = ((rel >> 2) + b) >> p.lshift;
-    const uint32_t l_lane = (uint32_t)(i * 16);
+    uint32_t l_lane = (uint32_t)(i * 16);
+    // opaque, so that a step's row offset stays one multiply-add: knowing the low bits, the compiler
+    // splits it into a multiply and an OR, and every vector instruction between the MFMAs costs
+    // about four of their cycles
+    asm volatile("" : "+v"(l_lane));
     // The A operands travel through a ring of kRing quarter-steps (one 128-bit read = the operands
     // of four MFMAs): the read for quarter j + kRing - 1 is issued right before the MFMAs of quarter
     // j, i.e. kRing - 1 groups of four 8-cycle MFMAs ahead of its use, with 4 kRing registers.
@@ -208,7 +212,8 @@ __global__ void __launch_bounds__(256) spmm_gather_kernel(const GatherParams p)
         for (int h = 0; h < P; ++h) {
             const int g = c * P + h, half = g & 1;
             const int hs = kRolled ? 0 : h;   // compile-time step base of the phase (rolled: in l_phase)
-            const uint32_t l_phase = l_lane + (kRolled ? (uint32_t)(h * (PH / NK) * MWIN * STRIDE) : 0u);
+            uint32_t l_phase = l_lane + (kRolled ? (uint32_t)(h * (PH / NK) * MWIN * STRIDE) : 0u);
+            asm volatile("" : "+v"(l_phase));   // one register, for the same reason
             if (g + 1 < phases)
                 fetch_meta(g + 1);   // the other half: free since the barrier that ended the phase before
             const float* const mb = lds_b + half * PH * kGatherCols + my_b;
