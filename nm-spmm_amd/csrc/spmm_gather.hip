@@ -26,7 +26,7 @@
 // next chunk of A is fetched into registers while the current one is multiplied and stored between
 // the two barriers that end the chunk.  The GPU does not hold its 2.4 GHz under this kernel (LDS and
 // matrix pipes both busy: about 2.1 GHz at 2:4), so fewer instructions and fewer LDS cycles also
-// mean a higher clock.  Measured at 4096 cubed with vectors of 4 columns: 2:4 105, 2:8 97, 1:8 87
+// mean a higher clock.  Measured at 4096 cubed with vectors of 4 columns: 2:4 108, 2:8 100, 1:8 90
 // useful TFLOP/s, where the expanding kernel reaches 71, 36 and 18.
 #include "internal.h"
 
