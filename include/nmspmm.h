@@ -118,9 +118,12 @@ size_t nmspmm_column_info_ints(int W, int pruning_N, int pruning_M, int N, int N
  * fp32: neighbours at distance 1, then 2, 4, ...; equal sums prefer the lower row) are kept:
  * dBT[W][N] receives their values, dDT[W][N/vec_len] their window-local row numbers, ascending,
  * W = K*n/m.  The output is what the preprocessing entry points above take.
- * nmspmm_decompress_device is the inverse (dropped rows become zero).
+ * nmspmm_decompress_device is the inverse: compressed row p of a window goes to the row its index
+ * names (the indices of a window need not ascend; they are expected to be distinct), every other
+ * row of the window becomes zero, and an index outside 0 .. m-1 stores nothing.
  * Requirements: m in {4, 8, 16, 32}, 0 < n < m, vec_len in {4, 8, 16, 32}, K % m == 0,
- * N % vec_len == 0, 16-byte aligned dB and dBT.  Asynchronous on `stream`. */
+ * N % vec_len == 0, m * N * 4 bytes below 4 GiB, 16-byte aligned dB and dBT.  Asynchronous on
+ * `stream`. */
 int nmspmm_compress_device(const float* dB, int K, int N, int n, int m, int vec_len, float* dBT,
                            int32_t* dDT, void* stream);
 int nmspmm_decompress_device(const float* dBT, const int32_t* dDT, int K, int N, int n, int m,

@@ -471,7 +471,8 @@ static int check_compress(const void* dense, const void* bt, const void* dt, int
         return NMSPMM_ERR_ALIGNMENT;
     if (!compress_supported(m, vec_len) || n <= 0 || n >= m)
         return NMSPMM_ERR_BAD_PATTERN;
-    if (K <= 0 || N <= 0 || K % m != 0 || N % vec_len != 0 || (N + 1023) / 1024 > 65535)
+    // the kernels address a window of m rows through 32-bit byte offsets
+    if (K <= 0 || N <= 0 || K % m != 0 || N % vec_len != 0 || (size_t)m * N * sizeof(float) > 0xffffffffull)
         return NMSPMM_ERR_BAD_SHAPE;
     return NMSPMM_OK;
 }

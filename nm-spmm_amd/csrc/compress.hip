@@ -24,7 +24,7 @@ typedef float cfloatx4 __attribute__((ext_vector_type(4)));
 // The dense operand (compressing) and the compressed one (expanding) are read once, the compressed
 // values are written once: non-temporal 16-byte accesses.  With B from HBM the compression runs 3 to
 // 20 % faster with the loads (4096 x 4096 at 2:8: 0.52 -> 0.62 of 8 TB/s) and the 2:4 cases another
-// 10 % with the stores; the expansion gains 1 to 7 % from the loads.
+// 10 % with the stores.
 __device__ inline float4 load_streaming(const float* p)
 {
     const cfloatx4 x = __builtin_nontemporal_load(reinterpret_cast<const cfloatx4*>(p));
@@ -111,6 +111,13 @@ compress_kernel(const float* __restrict__ B, float* __restrict__ BT, int32_t* __
     }
 }
 
+// Expansion.  What a thread loads depends on nothing it has loaded: its window's n index entries and
+// its 16-byte segments of the window's n compressed rows, all requested at once through
+// descriptors that end with the window (entries and rows from n on read as zero without a memory
+// access, so the instruction count is fixed).  The rows the indices leave out are zero-filled as
+// soon as the indices are there, while the values are still on their way; then every compressed row
+// goes to the row its index names (the checker's scatter: the indices need not ascend; a malformed
+// index stores nothing).
 template <int MW>
 __global__ void __launch_bounds__(256)
 decompress_kernel(const float* __restrict__ BT, const int32_t* __restrict__ DT, float* __restrict__ B, int N,
@@ -121,22 +128,37 @@ decompress_kernel(const float* __restrict__ BT, const int32_t* __restrict__ DT, 
     if (col >= N)
         return;
     const int a = col / L;
-    uint32_t keep = 0;
-    for (int p = 0; p < n; ++p) {
-        const uint32_t r = (uint32_t)DT[((size_t)w * n + p) * Q + a];
-        if (r < (uint32_t)MW)  // malformed indices must not leave the window
-            keep |= 1u << r;
-    }
-    // every row of the window is written exactly once: a kept row's values or zeros
+    const __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(const_cast<int32_t*>(DT) + (size_t)w * n * Q, 0,
+                                                                         (int)((size_t)n * Q * sizeof(int32_t)), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(BT) + (size_t)w * n * N, 0,
+                                                                         (int)((size_t)n * N * sizeof(float)), 0x00020000);
+    uint32_t rp[MW];
+    cuintx4 x[MW];
 #pragma unroll
-    for (int r = 0; r < MW; ++r) {
-        float4 x = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        if ((keep >> r) & 1u) {
-            const int p = __popc(keep & ((1u << r) - 1u));
-            x = load_streaming(BT + ((size_t)w * n + p) * N + col);
-        }
-        store_segment(B + (size_t)w * MW * N, (uint32_t)MW * N * 4u, ((uint32_t)r * N + col) * 4u, x);
+    for (int p = 0; p < MW; ++p)
+        rp[p] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rd, (int)(((uint32_t)p * Q + a) * 4u), 0, 0);
+#pragma unroll
+    for (int p = 0; p < MW; ++p)
+        x[p] = __builtin_amdgcn_raw_buffer_load_b128(rv, (int)(((uint32_t)p * N + col) * 4u), 0, 2);  // read once: non-temporal
+    uint32_t keep = 0;
+#pragma unroll
+    for (int p = 0; p < MW; ++p) {
+        if (p >= n)
+            rp[p] = 0xffffffffu;
+        keep |= rp[p] < (uint32_t)MW ? 1u << rp[p] : 0u;
     }
+    float* const base = B + (size_t)w * MW * N;
+    const uint32_t bytes = (uint32_t)MW * N * 4u;
+#pragma unroll
+    for (int r = 0; r < MW; ++r)
+        if (!((keep >> r) & 1u))
+            store_segment(base, bytes, ((uint32_t)r * N + col) * 4u, make_float4(0.0f, 0.0f, 0.0f, 0.0f));
+#pragma unroll
+    for (int p = 0; p < MW; ++p)
+        if (rp[p] < (uint32_t)MW)
+            store_segment(base, bytes, (rp[p] * (uint32_t)N + col) * 4u,
+                          make_float4(__uint_as_float(x[p][0]), __uint_as_float(x[p][1]), __uint_as_float(x[p][2]),
+                                      __uint_as_float(x[p][3])));
 }
 
 
@@ -239,6 +261,19 @@ compress32_kernel(const float* __restrict__ B, float* __restrict__ BT, int32_t* 
     }
 }
 
+// Expansion of n:32 windows, in the manner of decompress_kernel: nothing a thread loads depends on
+// what it has loaded.  Lane (j, c) of wave q reads the index entries c, c + 8, c + 16, c + 24 of its
+// vector (the eight lanes of the vector OR their four bits each into the mask of kept rows), the
+// entries q, q + 4, ... and its 16-byte segments of those compressed rows; wave q zero-fills what
+// the mask leaves out of rows 8 q .. 8 q + 7 and sends its compressed rows where their indices say.
+__device__ inline uint32_t dpp_or_over_eight_lanes(uint32_t x)
+{
+    x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, false);
+    x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false);
+    x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x141, 0xF, 0xF, false);
+    return x;
+}
+
 __global__ void __launch_bounds__(256)
 decompress32_kernel(const float* __restrict__ BT, const int32_t* __restrict__ DT, float* __restrict__ B, int N, int Q,
                     int n, int col_blocks)
@@ -246,30 +281,46 @@ decompress32_kernel(const float* __restrict__ BT, const int32_t* __restrict__ DT
     const int w = blockIdx.x / col_blocks;
     const int lane = threadIdx.x & 63, q = threadIdx.x >> 6;
     const int c = lane & 7, j = lane >> 3;
-    const int vec = (blockIdx.x % col_blocks) * kVectorsPerBlock32 + j;
-    if (vec >= Q)
-        return;
+    // a vector beyond the last one reads the last one's entries (the lanes of a wave exchange their
+    // bits, so all of them stay) and stores nothing
+    const int vec_raw = (blockIdx.x % col_blocks) * kVectorsPerBlock32 + j;
+    const bool active = vec_raw < Q;
+    const int vec = active ? vec_raw : Q - 1;
     const int col = vec * 32 + c * 4;
-    uint32_t keep = 0;
-    for (int p = 0; p < n; ++p) {
-        const uint32_t r = (uint32_t)DT[((size_t)w * n + p) * Q + vec];
-        if (r < 32u)  // malformed indices must not leave the window
-            keep |= 1u << r;
-    }
-    // every row of the window is written exactly once: a kept row's values or zeros
-    float4 x[8];
+    const __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(const_cast<int32_t*>(DT) + (size_t)w * n * Q, 0,
+                                                                         (int)((size_t)n * Q * sizeof(int32_t)), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(BT) + (size_t)w * n * N, 0,
+                                                                         (int)((size_t)n * N * sizeof(float)), 0x00020000);
+    uint32_t part[4], rp[8];
+    cuintx4 x[8];
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-        const int row = q * 8 + r;
-        x[r] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        if ((keep >> row) & 1u) {
-            const int p = __popc(keep & ((1u << row) - 1u));
-            x[r] = load_streaming(BT + ((size_t)w * n + p) * N + col);
-        }
-    }
+    for (int u = 0; u < 4; ++u)
+        part[u] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rd, (int)(((uint32_t)(c + 8 * u) * Q + vec) * 4u), 0, 0);
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+        rp[t] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rd, (int)(((uint32_t)(q + 4 * t) * Q + vec) * 4u), 0, 0);
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+        x[t] = __builtin_amdgcn_raw_buffer_load_b128(rv, (int)(((uint32_t)(q + 4 * t) * N + col) * 4u), 0, 2);  // read once
+    uint32_t keep = 0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        keep |= (c + 8 * u < n && part[u] < 32u) ? 1u << part[u] : 0u;
+    keep = dpp_or_over_eight_lanes(keep);
+    if (!active)
+        return;
+    float* const base = B + (size_t)w * 32 * N;
+    const uint32_t bytes = 32u * (uint32_t)N * 4u;
 #pragma unroll
     for (int r = 0; r < 8; ++r)
-        store_segment(B + (size_t)w * 32 * N, 32u * (uint32_t)N * 4u, ((uint32_t)(q * 8 + r) * N + col) * 4u, x[r]);
+        if (!((keep >> (q * 8 + r)) & 1u))
+            store_segment(base, bytes, ((uint32_t)(q * 8 + r) * N + col) * 4u, make_float4(0.0f, 0.0f, 0.0f, 0.0f));
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+        if (q + 4 * t < n && rp[t] < 32u)
+            store_segment(base, bytes, (rp[t] * (uint32_t)N + col) * 4u,
+                          make_float4(__uint_as_float(x[t][0]), __uint_as_float(x[t][1]), __uint_as_float(x[t][2]),
+                                      __uint_as_float(x[t][3])));
 }
 
 bool compress_supported(int m, int vec_len)

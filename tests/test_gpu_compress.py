@@ -104,12 +104,44 @@ def test_round_trips_at_full_size(n, m):
 
 
 def test_decompress_bit_exact_vs_generator(oracle):
-    for (K, N, n, m, vl) in ((256, 512, 2, 4, 32), (128, 96, 1, 8, 32), (64, 64, 2, 4, 4), (128, 192, 3, 8, 8)):
+    for (K, N, n, m, vl) in ((256, 512, 2, 4, 32), (128, 96, 1, 8, 32), (64, 64, 2, 4, 4), (128, 192, 3, 8, 8),
+                             (128, 96, 8, 32, 32), (64, 320, 4, 32, 32), (96, 2080, 16, 32, 32), (64, 32, 12, 32, 32),
+                             (64, 544, 31, 32, 32), (64, 1056, 7, 8, 16), (64, 48, 4, 16, 4), (96, 64, 9, 32, 8)):
         d = datagen.init_data(4, N, K, n, m, vec_len=vl, seed=K + n)
         back = torch.empty((K, N), dtype=torch.float32, device="cuda")
         nmspmm.decompress_device(torch.from_numpy(d["BT"]).cuda(), torch.from_numpy(d["DT"]).cuda(), K, N, n, m, back, vl)
         want = oracle.decompress(d["B_cm"].reshape(-1), d["D_cm"].reshape(-1), K, N, d["W"], vl)
         assert np.array_equal(back.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("K,N,n,m,vl", [(64, 96, 2, 8, 32), (128, 1088, 8, 32, 32), (64, 320, 5, 32, 32), (64, 64, 3, 4, 4)])
+def test_decompress_scatters_by_index(K, N, n, m, vl):
+    """The expansion puts compressed row p of a window where its index says (the checker's scatter,
+    oracle/nm_oracle.cpp nm_oracle_decompress): the indices of a window need not ascend.  An index
+    outside the window stores nothing; the row it would have named stays zero."""
+    rng = np.random.default_rng(K + N + n)
+    W, Q, nwin = K // m * n, N // vl, K // m
+    BT = rng.uniform(-1, 1, (W, N)).astype(np.float32)
+    DT = np.empty((W, Q), dtype=np.int32)
+    for w in range(nwin):
+        for a in range(Q):
+            DT[w * n:(w + 1) * n, a] = rng.permutation(m)[:n]          # distinct, in no order
+    bad = rng.random((W, Q)) < 0.1
+    DT_bad = np.where(bad, rng.choice([-1, m, m + 7, 1 << 20, -(1 << 31)], size=(W, Q)), DT).astype(np.int32)
+    for table in (DT, DT_bad):
+        want = np.zeros((K, N), dtype=np.float32)
+        for w in range(nwin):
+            for p in range(n):
+                for a in range(Q):
+                    r = int(table[w * n + p, a])
+                    if 0 <= r < m:
+                        want[w * m + r, a * vl:(a + 1) * vl] = BT[w * n + p, a * vl:(a + 1) * vl]
+        back = torch.full((K, N), float("nan"), dtype=torch.float32, device="cuda")
+        guard = torch.full((8, N), 7.0, dtype=torch.float32, device="cuda")   # allocated right behind: must stay
+        nmspmm.decompress_device(torch.from_numpy(BT).cuda(), torch.from_numpy(table).cuda(), K, N, n, m, back, vl)
+        torch.cuda.synchronize()
+        assert np.array_equal(back.cpu().numpy(), want)
+        assert bool((guard == 7.0).all())
 
 
 @pytest.mark.parametrize("n,m", [(2, 4), (1, 8)])
