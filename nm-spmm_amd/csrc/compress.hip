@@ -79,7 +79,7 @@ compress_kernel(const float* __restrict__ B, float* __restrict__ BT, int32_t* __
         key[r] = __float_as_uint(s);
     }
 
-    // Lane c of the group ranks rows c, c + G, ...; a ballot hands the verdicts to the whole group.
+    // Lane c of the group ranks rows c, c + G, ...; a ballot hands the outcome to the whole group.
     uint32_t keep = 0;
     for (int t = 0; t * G < MW; ++t) {
         const int mine = c + t * G;
@@ -171,7 +171,7 @@ decompress_kernel(const float* __restrict__ BT, const int32_t* __restrict__ DT, 
 // 256 columns).  The row scores are summed in the same order as above (inside the thread, then over
 // the eight lanes of the vector by lane exchange); the four waves swap their eight scores per
 // vector through LDS, lane (j, c) of wave q ranks row 8 q + c, and the waves' ballots are put
-// together through LDS to the verdict on all 32 rows.  About 70 registers: six waves per SIMD.
+// together through LDS to the mask of kept rows of all 32.  About 70 registers: six waves per SIMD.
 
 __device__ inline float dpp_quad_1032(float x)
 {
@@ -193,7 +193,7 @@ compress32_kernel(const float* __restrict__ B, float* __restrict__ BT, int32_t* 
                   int col_blocks)
 {
     __shared__ __attribute__((aligned(16))) uint32_t scores[kVectorsPerBlock32][32];
-    __shared__ unsigned char verdict[kVectorsPerBlock32][4];  // byte q: rows 8 q .. 8 q + 7
+    __shared__ unsigned char kept_bits[kVectorsPerBlock32][4];  // byte q: rows 8 q .. 8 q + 7
     const int w = blockIdx.x / col_blocks;
     const int lane = threadIdx.x & 63, q = threadIdx.x >> 6;
     const int c = lane & 7, j = lane >> 3;
@@ -243,9 +243,9 @@ compress32_kernel(const float* __restrict__ B, float* __restrict__ BT, int32_t* 
     }
     const unsigned long long votes = __ballot(rank < n);   // bit 8 j + c: row 8 q + c of vector j
     if (c == 0)
-        verdict[j][q] = (unsigned char)(votes >> (8 * j));
+        kept_bits[j][q] = (unsigned char)(votes >> (8 * j));
     __syncthreads();
-    const uint32_t keep = *reinterpret_cast<const uint32_t*>(verdict[j]);   // bit r: row r of the vector is kept
+    const uint32_t keep = *reinterpret_cast<const uint32_t*>(kept_bits[j]);   // bit r: row r of the vector is kept
     if (!active)
         return;
 #pragma unroll
