@@ -238,6 +238,9 @@ def test_compress_rejects_bad_arguments_without_a_gpu():
     assert L.nmspmm_compress_device(FAKE, 66, 64, 2, 4, 32, FAKE, FAKE, None) == 2   # K % m
     assert L.nmspmm_decompress_device(FAKE, None, 64, 64, 2, 4, 32, FAKE, None) == 1
     assert L.nmspmm_decompress_device(FAKE, FAKE, 64, 40, 2, 4, 32, FAKE, None) == 2  # N % vec_len
+    # a window of m rows is addressed through 32-bit byte offsets: m * N * 4 bytes stay below 4 GiB
+    assert L.nmspmm_compress_device(FAKE, 32, (1 << 25) + 32, 8, 32, 32, FAKE, FAKE, None) == 2
+    assert L.nmspmm_decompress_device(FAKE, FAKE, 8, (1 << 27) + 32, 2, 8, 32, FAKE, None) == 2
 
 
 def test_rowmajor_entry_rejects_bad_arguments_without_a_gpu():
